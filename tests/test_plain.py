@@ -1,0 +1,198 @@
+"""Pins for the plain implementation: vectors held by the reference's own tests,
+special cases that reduce to a library routine, and invariants.  Each is chosen
+so that a plausible mistake (wrong sign or pairing, a norm in the wrong place)
+fails it."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_qwen3 as plain
+from conftest import TINY
+
+
+def test_rms_norm_reference_vector():
+    # tests/test_qwen3.py:34-44 of the reference
+    x = torch.tensor([[1.0, -2.0, 3.0, -4.0]])
+    w = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    expected = x * torch.rsqrt(x.square().mean(dim=-1, keepdim=True) + 1e-6) * w
+    torch.testing.assert_close(plain.rms_norm(x, w, 1e-6), expected)
+    # hand value: mean square 7.5
+    assert plain.rms_norm(x, w, 1e-6)[0, 3].item() == pytest.approx(-16 / math.sqrt(7.5), rel=1e-6)
+
+
+def test_rms_norm_is_library_rms_norm():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(5, 24, generator=g)
+    w = torch.randn(24, generator=g)
+    torch.testing.assert_close(plain.rms_norm(x, w, 1e-5), F.rms_norm(x, (24,), w, 1e-5))
+
+
+def test_add_rms_norm_reference_vector():
+    # tests/test_kernels.py:20-36 of the reference
+    r = torch.tensor([[1.0, -2.0, 3.0, -4.0]])
+    u = torch.tensor([[0.5, 1.0, -1.5, 2.0]])
+    w = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    summed, normed = plain.add_rms_norm(r, u, w, 1e-6)
+    s = r + u
+    torch.testing.assert_close(summed, s)
+    torch.testing.assert_close(normed, s * torch.rsqrt(s.square().mean(-1, keepdim=True) + 1e-6) * w)
+    zero_sum, zero_norm = plain.add_rms_norm(r, torch.zeros_like(r), w, 1e-6)
+    torch.testing.assert_close(zero_norm, plain.rms_norm(r, w, 1e-6))
+
+
+def test_rotary_sign_and_pairing():
+    # D = 4, theta = 10000: inv_freq = [1, 0.01].  A unit vector in dim 0 at
+    # position 1 turns into (cos 1, 0, sin 1, 0): partner of dim j is j + D/2,
+    # and the second half gets +sin.
+    cos, sin = plain.rotary_tables(torch.tensor([1]), 4, 10000.0)
+    x = torch.tensor([[[1.0, 0.0, 0.0, 0.0]]])
+    out = plain.apply_rotary(x, cos, sin)[0, 0]
+    torch.testing.assert_close(out, torch.tensor([math.cos(1.0), 0.0, math.sin(1.0), 0.0]))
+    y = torch.tensor([[[0.0, 1.0, 0.0, 0.0]]])
+    out = plain.apply_rotary(y, cos, sin)[0, 0]
+    torch.testing.assert_close(out, torch.tensor([0.0, math.cos(0.01), 0.0, math.sin(0.01)]))
+
+
+def test_rotary_position_zero_is_identity_and_norm_kept():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(3, 6, 16, generator=g)
+    cos, sin = plain.rotary_tables(torch.arange(6), 16, 1e6)
+    out = plain.apply_rotary(x, cos, sin)
+    torch.testing.assert_close(out[:, 0], x[:, 0])
+    pair_norm_in = x[..., :8] ** 2 + x[..., 8:] ** 2
+    pair_norm_out = out[..., :8] ** 2 + out[..., 8:] ** 2
+    torch.testing.assert_close(pair_norm_out, pair_norm_in)
+
+
+def test_rotary_scores_depend_on_distance_only():
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(1, 1, 32, generator=g).double()
+    k = torch.randn(1, 1, 32, generator=g).double()
+
+    def score(pq, pk):
+        cq, sq = plain.rotary_tables(torch.tensor([pq]), 32, 10000.0)
+        ck, sk = plain.rotary_tables(torch.tensor([pk]), 32, 10000.0)
+        return (plain.apply_rotary(q, cq.double(), sq.double())
+                * plain.apply_rotary(k, ck.double(), sk.double())).sum().item()
+
+    assert score(9, 4) == pytest.approx(score(25, 20), abs=1e-5)
+    assert abs(score(9, 4) - score(9, 5)) > 1e-3
+
+
+def test_attention_is_library_attention_after_group_expansion():
+    # tests/test_kernels.py:91-105 of the reference uses the same library call
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(6, 9, 8, generator=g)
+    k = torch.randn(2, 9, 8, generator=g)
+    v = torch.randn(2, 9, 8, generator=g)
+    got = plain.causal_attention(q, k, v, 8**-0.5)
+    want = F.scaled_dot_product_attention(
+        q.unsqueeze(0), k.repeat_interleave(3, 0).unsqueeze(0),
+        v.repeat_interleave(3, 0).unsqueeze(0), is_causal=True)[0]
+    torch.testing.assert_close(got, want, atol=1e-6, rtol=1e-6)
+
+
+def test_attention_group_mapping_is_blockwise():
+    # query heads 0,1 read kv head 0 and heads 2,3 read kv head 1 (h // G), not h % Hkv
+    q = torch.zeros(4, 1, 4)
+    k = torch.zeros(2, 1, 4)
+    v = torch.stack((torch.full((1, 4), 1.0), torch.full((1, 4), 2.0)))
+    out = plain.causal_attention(q, k, v, 0.5)
+    assert out[:, 0, 0].tolist() == [1.0, 1.0, 2.0, 2.0]
+
+
+def test_attention_window_keeps_last_w_keys():
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(1, 7, 4, generator=g)
+    k = torch.randn(1, 7, 4, generator=g)
+    v = torch.randn(1, 7, 4, generator=g)
+    got = plain.causal_attention(q, k, v, 0.5, window=3)[0, 6]
+    s = (k[0, 4:7] @ q[0, 6]) * 0.5
+    want = torch.softmax(s, 0) @ v[0, 4:7]
+    torch.testing.assert_close(got, want)
+
+
+def test_swiglu_is_library_expression():
+    # tests/test_cute_swiglu.py:18-27 of the reference: seed 23, [3,8] x [12,8]
+    torch.manual_seed(23)
+    x = torch.randn(3, 8)
+    wg = torch.randn(12, 8)
+    wu = torch.randn(12, 8)
+    wd = torch.eye(12)
+    weights = {"m.gate_proj.weight": wg, "m.up_proj.weight": wu, "m.down_proj.weight": wd}
+    torch.testing.assert_close(plain.swiglu_mlp(x, weights, "m"), F.silu(x @ wg.T) * (x @ wu.T))
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_shift_of_all_positions_changes_nothing(name):
+    config = TINY[name]
+    w = plain.random_weights(config, 5)
+    ids = torch.randint(0, config["vocab_size"], (12,), generator=torch.Generator().manual_seed(0))
+    a = plain.forward(w, config, ids)
+    b = plain.forward(w, config, ids, first_position=37)
+    torch.testing.assert_close(a, b, atol=2e-5, rtol=1e-4)
+    shuffled = plain.forward(w, config, ids.flip(0))
+    assert (a - shuffled.flip(0)).abs().max() > 1e-3   # positions do matter
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_prefix_logits_do_not_see_later_tokens(name):
+    config = TINY[name]
+    w = plain.random_weights(config, 6)
+    ids = torch.randint(0, config["vocab_size"], (10,), generator=torch.Generator().manual_seed(1))
+    full = plain.forward(w, config, ids)
+    torch.testing.assert_close(full[:6], plain.forward(w, config, ids[:6]), atol=1e-6, rtol=1e-5)
+
+
+def test_query_scale_is_removed_by_the_per_head_norm():
+    # q_norm sits between the projection and the rotation: scaling W_q leaves
+    # the logits unchanged (up to eps); without the norm they would change.
+    config = TINY["A"]
+    w = plain.random_weights(config, 9)
+    ids = [3, 200, 17, 17, 64]
+    a = plain.forward(w, config, ids)
+    w2 = dict(w)
+    for i in range(config["num_hidden_layers"]):
+        name = f"model.layers.{i}.self_attn.q_proj.weight"
+        w2[name] = w[name] * 8.0
+    torch.testing.assert_close(plain.forward(w2, config, ids), a, atol=1e-5, rtol=1e-4)
+
+
+def test_zeroed_output_projections_reduce_to_norm_and_head():
+    config = TINY["B"]
+    w = plain.random_weights(config, 10)
+    for i in range(config["num_hidden_layers"]):
+        w[f"model.layers.{i}.self_attn.o_proj.weight"].zero_()
+        w[f"model.layers.{i}.mlp.down_proj.weight"].zero_()
+    ids = torch.tensor([5, 6, 7])
+    e = w["model.embed_tokens.weight"][ids]
+    want = F.rms_norm(e, (config["hidden_size"],), w["model.norm.weight"], config["rms_norm_eps"]) @ w["lm_head.weight"].T
+    torch.testing.assert_close(plain.forward(w, config, ids), want, atol=1e-6, rtol=1e-5)
+
+
+def test_feed_forward_reads_the_normalised_sum():
+    # one layer, attention silenced: h = e + mlp(norm_post(e))
+    config = dict(TINY["A"], num_hidden_layers=1)
+    w = plain.random_weights(config, 11)
+    w["model.layers.0.self_attn.o_proj.weight"].zero_()
+    ids = torch.tensor([9, 8])
+    e = w["model.embed_tokens.weight"][ids]
+    y = F.rms_norm(e, (64,), w["model.layers.0.post_attention_layernorm.weight"], 1e-6)
+    m = (F.silu(y @ w["model.layers.0.mlp.gate_proj.weight"].T) * (y @ w["model.layers.0.mlp.up_proj.weight"].T)) @ w["model.layers.0.mlp.down_proj.weight"].T
+    z = F.rms_norm(e + m, (64,), w["model.norm.weight"], 1e-6)
+    torch.testing.assert_close(plain.forward(w, config, ids), z @ w["model.embed_tokens.weight"].T, atol=1e-6, rtol=1e-5)
+
+
+def test_sampling_filter_vectors():
+    # tests/test_sampling.py:47-81 of the reference
+    def kept(x):
+        return torch.isfinite(x).nonzero()[:, 1].tolist()
+
+    assert kept(plain.filter_logits(torch.tensor([[0.0, 3.0, 2.0, 1.0]]), 1.0, top_k=2)) == [1, 2]
+    assert kept(plain.filter_logits(torch.tensor([[5.0, 4.0, 0.0]]), 1.0, top_p=0.7)) == [0]
+    assert kept(plain.filter_logits(torch.tensor([[0.0, -1.0, -3.0]]), 1.0, min_p=0.2)) == [0, 1]
