@@ -1,0 +1,247 @@
+// Paged grouped-query attention for a mixed batch, general sizes.
+//
+// One launch serves every sequence of a step: portions of prompts (many query
+// tokens, some context already cached) beside single decoded tokens.  The keys
+// and values of the step's own tokens are already in the pages.  For sequence
+// s with q_len query tokens and ctx keys in total (ctx_before = ctx - q_len),
+// query token i sits at position p = ctx_before + i and reads keys
+//   max(0, p - window + 1) .. p        (window <= 0: all keys 0 .. p).
+// Query head h reads kv head h / G.  Scores, softmax (online, over key tiles)
+// and the weighted sum of values are float32 on the vector ALU; one rounding
+// at the store.  This kernel takes any head size that is a multiple of 16 up
+// to 256, any group size, any page size, float32 or bfloat16 storage; faster
+// matrix-core kernels cover the common bfloat16 shapes.
+//
+// Work split: block = (row tile, kv head, sequence); a row is one (query
+// token, query head of the group) pair, 16 rows per block, so the G heads that
+// share a kv head share its key/value tiles.  Thread (r = tid / 16, c = tid % 16)
+// owns row r: it computes the scores of keys c, c + 16, ... of the tile and
+// output dims c, c + 16, ...; the 16 lanes of a row reduce by shuffles.
+#include "common.h"
+
+#define ROWS 16
+
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ void load(const float* p, float* o) {
+    const float4 v = *(const float4*)p;
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+  }
+};
+template <> struct Vec4<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float* o) {
+    const uint2 v = *(const uint2*)p;
+    o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+    o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
+};
+
+template <typename T, int DMAX, int TK, bool FAST_EXP>
+__global__ __launch_bounds__(256) void paged_attention_generic_kernel(
+    const T* __restrict__ q, long long q_stride, const T* __restrict__ key_pages,
+    const T* __restrict__ value_pages, T* __restrict__ out, long long out_stride,
+    const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
+    const int* __restrict__ block_table, int table_stride, int kv_heads, int groups, int head_dim,
+    int block_size, int num_blocks, int window, float scale) {
+  constexpr int KPT = TK / 16;    // keys per thread in a tile
+  constexpr int DPT = DMAX / 16;  // output dims per thread
+  extern __shared__ float smem[];
+  const int D = head_dim;
+  const int kstride = D + 1;
+  float* Qs = smem;                   // [ROWS][D + 1]
+  float* Ks = Qs + ROWS * kstride;    // [TK][D + 1]
+  float* Vs = Ks + TK * kstride;      // [TK][D]
+  float* Ps = Vs + TK * D;            // [ROWS][TK]
+
+  const int seq = blockIdx.z;
+  const int hk = blockIdx.y;
+  const int q0 = cu_q[seq];
+  const int q_len = cu_q[seq + 1] - q0;
+  const int ctx = ctx_len[seq];
+  const int ctx_before = ctx - q_len;
+  const int rows_total = q_len * groups;
+  const int row0 = blockIdx.x * ROWS;
+  if (row0 >= rows_total || ctx_before < 0) return;
+
+  const int tid = threadIdx.x;
+  const int r = tid / 16;
+  const int c = tid % 16;
+  const int my_row = row0 + r;
+  const bool row_ok = my_row < rows_total;
+  const int my_tok = row_ok ? my_row / groups : 0;
+  const int my_g = row_ok ? my_row - my_tok * groups : 0;
+  const int my_pos = ctx_before + my_tok;
+  const int last_row = min(rows_total, row0 + ROWS) - 1;
+  const int pos_min = ctx_before + row0 / groups;
+  const int pos_max = ctx_before + last_row / groups;
+  const int k_begin = window > 0 ? max(0, pos_min - window + 1) : 0;
+  const int k_end = pos_max + 1;  // <= ctx
+
+  // Q tile -> LDS as float32
+  const int chunks = D / 4;
+  for (int e = tid; e < ROWS * chunks; e += 256) {
+    const int rr = e / chunks;
+    const int d4 = (e - rr * chunks) * 4;
+    const int row = row0 + rr;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (row < rows_total) {
+      const int tok = row / groups;
+      const int g = row - tok * groups;
+      Vec4<T>::load(q + (size_t)(q0 + tok) * q_stride + (size_t)(hk * groups + g) * D + d4, v);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) Qs[rr * kstride + d4 + i] = v[i];
+  }
+
+  float m = -INFINITY, l = 0.f;
+  float acc[DPT];
+#pragma unroll
+  for (int i = 0; i < DPT; ++i) acc[i] = 0.f;
+
+  const int* table = block_table + (size_t)seq * table_stride;
+  for (int kt = (k_begin / TK) * TK; kt < k_end; kt += TK) {
+    __syncthreads();  // previous tile consumed (and Q visible on the first pass)
+    for (int e = tid; e < TK * chunks; e += 256) {
+      const int kk = e / chunks;
+      const int d4 = (e - kk * chunks) * 4;
+      const int kp = kt + kk;
+      float kv[4] = {0.f, 0.f, 0.f, 0.f};
+      float vv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (kp >= k_begin && kp < k_end) {
+        const int block = table[kp / block_size];
+        if (block >= 0 && block < num_blocks) {
+          const size_t off = (((size_t)block * kv_heads + hk) * block_size + (kp % block_size)) * D + d4;
+          Vec4<T>::load(key_pages + off, kv);
+          Vec4<T>::load(value_pages + off, vv);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        Ks[kk * kstride + d4 + i] = kv[i];
+        Vs[kk * D + d4 + i] = vv[i];
+      }
+    }
+    __syncthreads();
+
+    float s[KPT];
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) s[i] = 0.f;
+    const float* qrow = Qs + r * kstride;
+    for (int d = 0; d < D; ++d) {
+      const float qv = qrow[d];
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) s[i] = fmaf(qv, Ks[(c + 16 * i) * kstride + d], s[i]);
+    }
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int kp = kt + c + 16 * i;
+      const bool visible = row_ok && kp <= my_pos && (window <= 0 || kp > my_pos - window);
+      s[i] = visible ? s[i] * scale : -INFINITY;
+      tile_max = fmaxf(tile_max, s[i]);
+    }
+#pragma unroll
+    for (int offset = 8; offset > 0; offset >>= 1) tile_max = fmaxf(tile_max, __shfl_xor(tile_max, offset, FE_WAVE));
+    const float m_new = fmaxf(m, tile_max);
+    float corr = 1.f, tile_sum = 0.f;
+    if (m_new > -INFINITY) {
+      corr = FAST_EXP ? __expf(m - m_new) : expf(m - m_new);
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) {
+        const float p = FAST_EXP ? __expf(s[i] - m_new) : expf(s[i] - m_new);
+        s[i] = p;
+        tile_sum += p;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) s[i] = 0.f;
+    }
+#pragma unroll
+    for (int offset = 8; offset > 0; offset >>= 1) tile_sum += __shfl_xor(tile_sum, offset, FE_WAVE);
+    l = l * corr + tile_sum;
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) Ps[r * TK + c + 16 * i] = s[i];
+    __syncthreads();
+
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) acc[i] *= corr;
+    const float* prow = Ps + r * TK;
+    for (int kk = 0; kk < TK; ++kk) {
+      const float p = prow[kk];
+      const float* vrow = Vs + kk * D;
+#pragma unroll
+      for (int i = 0; i < DPT; ++i)
+        if (c + 16 * i < D) acc[i] = fmaf(p, vrow[c + 16 * i], acc[i]);
+    }
+  }
+
+  if (row_ok) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    T* orow = out + (size_t)(q0 + my_tok) * out_stride + (size_t)(hk * groups + my_g) * D;
+#pragma unroll
+    for (int i = 0; i < DPT; ++i)
+      if (c + 16 * i < D) store_from_float(orow + c + 16 * i, acc[i] * inv);
+  }
+}
+
+template <typename T, int DMAX, int TK, bool FAST_EXP>
+static int launch_generic(const void* q, long long q_stride, const void* key_pages, const void* value_pages,
+                          void* out, long long out_stride, const int* cu_q, const int* ctx_len,
+                          const int* block_table, int table_stride, int num_seqs, int max_q_len,
+                          int kv_heads, int groups, int head_dim, int block_size, int num_blocks,
+                          int window, float scale, hipStream_t stream) {
+  const long long tiles = ((long long)max_q_len * groups + ROWS - 1) / ROWS;
+  if (tiles > 0x7fffffffLL || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
+  const size_t smem = sizeof(float) * ((size_t)(ROWS + TK) * (head_dim + 1) + (size_t)TK * head_dim + ROWS * TK);
+  dim3 grid((unsigned)tiles, kv_heads, num_seqs);
+  paged_attention_generic_kernel<T, DMAX, TK, FAST_EXP><<<grid, 256, smem, stream>>>(
+      (const T*)q, q_stride, (const T*)key_pages, (const T*)value_pages, (T*)out, out_stride, cu_q,
+      ctx_len, block_table, table_stride, kv_heads, groups, head_dim, block_size, num_blocks, window,
+      scale);
+  return fe_check_launch();
+}
+
+template <typename T, bool FAST_EXP>
+static int dispatch_generic(const void* q, long long q_stride, const void* key_pages, const void* value_pages,
+                            void* out, long long out_stride, const int* cu_q, const int* ctx_len,
+                            const int* block_table, int table_stride, int num_seqs, int max_q_len,
+                            int kv_heads, int groups, int head_dim, int block_size, int num_blocks,
+                            int window, float scale, hipStream_t stream) {
+#define FE_GO(DMAX, TK)                                                                              \
+  return launch_generic<T, DMAX, TK, FAST_EXP>(q, q_stride, key_pages, value_pages, out, out_stride, \
+                                               cu_q, ctx_len, block_table, table_stride, num_seqs,   \
+                                               max_q_len, kv_heads, groups, head_dim, block_size,    \
+                                               num_blocks, window, scale, stream)
+  if (head_dim <= 32) FE_GO(32, 64);
+  if (head_dim <= 64) FE_GO(64, 64);
+  if (head_dim <= 128) FE_GO(128, 32);
+  FE_GO(256, 16);
+#undef FE_GO
+}
+
+// q: [tokens, ...] with q_stride elements between tokens, heads contiguous
+// ([q_heads][D]) from the token's start; out likewise with out_stride.
+// cu_q: [num_seqs + 1] prefix sums of query lengths; ctx_len: [num_seqs] keys
+// in the cache after this step; block_table: [num_seqs, table_stride].
+extern "C" int fe_paged_attention_generic(const void* q, long long q_stride, const void* key_pages,
+                                          const void* value_pages, void* out, long long out_stride,
+                                          int dtype, const int* cu_q, const int* ctx_len,
+                                          const int* block_table, int table_stride, int num_seqs,
+                                          int max_q_len, int kv_heads, int groups, int head_dim,
+                                          int block_size, int num_blocks, int window, float scale,
+                                          hipStream_t stream) {
+  if (num_seqs <= 0 || max_q_len <= 0) return FE_OK;
+  if (head_dim < 16 || head_dim > 256 || head_dim % 16) return FE_BAD_ARGUMENT;
+  if (kv_heads <= 0 || groups <= 0 || block_size <= 0 || num_blocks <= 0 || table_stride <= 0) return FE_BAD_ARGUMENT;
+  if (q_stride % 4 || out_stride < (long long)kv_heads * groups * head_dim) return FE_BAD_ARGUMENT;
+  if (dtype == FE_F32)
+    return dispatch_generic<float, false>(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len,
+                                          block_table, table_stride, num_seqs, max_q_len, kv_heads, groups,
+                                          head_dim, block_size, num_blocks, window, scale, stream);
+  if (dtype == FE_BF16)
+    return dispatch_generic<bf16_t, true>(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len,
+                                          block_table, table_stride, num_seqs, max_q_len, kv_heads, groups,
+                                          head_dim, block_size, num_blocks, window, scale, stream);
+  return FE_BAD_ARGUMENT;
+}

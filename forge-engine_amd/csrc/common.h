@@ -1,0 +1,79 @@
+// Shared device helpers for the gfx950 kernels: element types, wave and block
+// reductions.  Everything here assumes 64-wide wavefronts.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define FE_WAVE 64
+
+// Status codes returned by every extern "C" entry point.
+#define FE_OK 0
+#define FE_BAD_ARGUMENT 1
+#define FE_LAUNCH_FAILED 2
+
+// Element type tags used across the C interface.
+#define FE_F32 0
+#define FE_BF16 1
+
+typedef uint16_t bf16_t;
+
+__device__ __forceinline__ float bf16_to_float(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// Round to nearest even; NaN stays NaN.
+__device__ __forceinline__ bf16_t float_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)0x7fc0;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float load_as_float(const float* p) { return *p; }
+__device__ __forceinline__ float load_as_float(const bf16_t* p) { return bf16_to_float(*p); }
+__device__ __forceinline__ void store_from_float(float* p, float v) { *p = v; }
+__device__ __forceinline__ void store_from_float(bf16_t* p, float v) { *p = float_to_bf16(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int offset = FE_WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, FE_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int offset = FE_WAVE / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, FE_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; `scratch` holds one float per wave
+// (at least 16).  Every thread gets the total.  Contains two barriers.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (FE_WAVE - 1);
+  const int wave = threadIdx.x / FE_WAVE;
+  const int waves = (blockDim.x + FE_WAVE - 1) / FE_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int i = 0; i < waves; ++i) total += scratch[i];
+  return total;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x & (FE_WAVE - 1);
+  const int wave = threadIdx.x / FE_WAVE;
+  const int waves = (blockDim.x + FE_WAVE - 1) / FE_WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = scratch[0];
+  for (int i = 1; i < waves; ++i) total = fmaxf(total, scratch[i]);
+  return total;
+}
+
+static inline int fe_check_launch() {
+  return hipGetLastError() == hipSuccess ? FE_OK : FE_LAUNCH_FAILED;
+}

@@ -1,0 +1,151 @@
+// Fused per-head RMSNorm of q and k, rotary position encoding, and the write of
+// k and v into the paged cache.  Input is the fused projection output
+// qkv[T, (Hq + 2*Hkv) * D]; q is normalised and rotated in place, k is
+// normalised, rotated and written to its page, v is copied to its page.
+//
+//   y      = x * rsqrt(mean_D(x^2) + eps) * w           (skipped if w is null)
+//   angle  = float(position) * inv_freq[j],  j < R/2     (R = rotary_dim <= D)
+//   out[j]       = y[j] * cos(angle) - y[j + R/2] * sin(angle)
+//   out[j + R/2] = y[j + R/2] * cos(angle) + y[j] * sin(angle)
+//   dims >= R pass through.  All arithmetic in float32, one rounding at the store.
+//
+// Cache layout per layer: pages[block][kv_head][slot][D] for keys and the same
+// for values; token at position p of sequence s lives in block
+// table[s][p / block_size], slot p % block_size.
+#include "common.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
+    T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+    const float* __restrict__ inv_freq, const int* __restrict__ positions,
+    const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_stride,
+    T* __restrict__ key_pages, T* __restrict__ value_pages, int q_heads, int kv_heads,
+    int head_dim, int rotary_dim, int block_size, int num_blocks, float eps, int write_kv,
+    int total_heads_work) {
+  const int lane = threadIdx.x & (FE_WAVE - 1);
+  const int wave = threadIdx.x / FE_WAVE;
+  const int work = blockIdx.x * (blockDim.x / FE_WAVE) + wave;  // one (token, head) per wave
+  if (work >= total_heads_work) return;
+  const int heads_all = q_heads + 2 * kv_heads;
+  const int t = work / heads_all;
+  const int head = work - t * heads_all;
+  T* x = qkv + ((size_t)t * heads_all + head) * head_dim;
+  const bool is_q = head < q_heads;
+  const bool is_k = !is_q && head < q_heads + kv_heads;
+  const int kv_head = is_q ? 0 : (is_k ? head - q_heads : head - q_heads - kv_heads);
+  const int pos = positions[t];
+
+  T* dst = x;  // q stays in place
+  if (!is_q) {
+    if (!write_kv) return;
+    const int seq = token_seq[t];
+    const int block = block_table[(size_t)seq * table_stride + pos / block_size];
+    if (block < 0 || block >= num_blocks) return;  // host reserves pages before the launch
+    T* pages = is_k ? key_pages : value_pages;
+    dst = pages + (((size_t)block * kv_heads + kv_head) * block_size + (pos % block_size)) * head_dim;
+  }
+  if (!is_q && !is_k) {  // value: copy
+    for (int d = lane; d < head_dim; d += FE_WAVE) dst[d] = x[d];
+    return;
+  }
+
+  const float* w = is_q ? q_weight : k_weight;
+  const int half = head_dim / 2;
+  const int rhalf = rotary_dim / 2;
+  // Each lane owns pairs (j, j + half) for j = lane, lane + 64, ...; head_dim <= 512.
+  float lo[4], hi[4];
+  float sumsq = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int j = lane + i * FE_WAVE;
+    lo[i] = 0.f; hi[i] = 0.f;
+    if (j < half) {
+      lo[i] = load_as_float(x + j);
+      hi[i] = load_as_float(x + j + half);
+      sumsq += lo[i] * lo[i] + hi[i] * hi[i];
+    }
+  }
+  float inv = 1.f;
+  if (w) {
+    sumsq = wave_sum(sumsq);
+    inv = rsqrtf(sumsq / (float)head_dim + eps);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int j = lane + i * FE_WAVE;
+    if (j < half) {
+      if (w) {
+        lo[i] = lo[i] * inv * w[j];
+        hi[i] = hi[i] * inv * w[j + half];
+      }
+    }
+  }
+  // Rotation pairs are (j, j + rhalf) for j < rhalf.  With rotary_dim == head_dim
+  // the partner of lo[i] is hi[i] and everything stays in registers.
+  if (rotary_dim == head_dim) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = lane + i * FE_WAVE;
+      if (j < half) {
+        float s, c;
+        sincosf((float)pos * inv_freq[j], &s, &c);
+        const float a = lo[i], b = hi[i];
+        store_from_float(dst + j, a * c - b * s);
+        store_from_float(dst + j + half, b * c + a * s);
+      }
+    }
+  } else {
+    // Partial rotation: partners may sit in other lanes, so the normalised head
+    // goes through a per-wave LDS buffer (LDS operations of one wave are ordered).
+    __shared__ float stage[4][512];
+    float* buf = stage[wave];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = lane + i * FE_WAVE;
+      if (j < half) { buf[j] = lo[i]; buf[j + half] = hi[i]; }
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    for (int d = lane; d < head_dim; d += FE_WAVE) {
+      float v = buf[d];
+      if (d < rotary_dim) {
+        const int j = d < rhalf ? d : d - rhalf;
+        float s, c;
+        sincosf((float)pos * inv_freq[j], &s, &c);
+        v = d < rhalf ? buf[d] * c - buf[d + rhalf] * s : buf[d] * c + buf[d - rhalf] * s;
+      }
+      store_from_float(dst + d, v);
+    }
+  }
+}
+
+extern "C" int fe_qk_norm_rope_write(void* qkv, int dtype, const float* q_weight, const float* k_weight,
+                                     const float* inv_freq, const int* positions, const int* token_seq,
+                                     const int* block_table, int table_stride, void* key_pages,
+                                     void* value_pages, int tokens, int q_heads, int kv_heads,
+                                     int head_dim, int rotary_dim, int block_size, int num_blocks,
+                                     float eps, int write_kv, hipStream_t stream) {
+  if (tokens <= 0) return FE_OK;
+  if (q_heads < 0 || kv_heads < 0 || head_dim <= 0 || head_dim % 2 || head_dim > 512) return FE_BAD_ARGUMENT;
+  if (rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2) return FE_BAD_ARGUMENT;
+  if (rotary_dim > 0 && !inv_freq) return FE_BAD_ARGUMENT;
+  if (write_kv && (block_size <= 0 || num_blocks <= 0 || !block_table || !key_pages || !value_pages)) return FE_BAD_ARGUMENT;
+  const long long work = (long long)tokens * (q_heads + 2 * kv_heads);
+  if (work <= 0 || work > 0x7fffffffLL) return FE_BAD_ARGUMENT;
+  const int waves_per_block = 4;
+  const long long blocks = (work + waves_per_block - 1) / waves_per_block;
+  if (blocks > 0x7fffffffLL) return FE_BAD_ARGUMENT;
+  if (dtype == FE_F32)
+    qk_norm_rope_write_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>(
+        (float*)qkv, q_weight, k_weight, inv_freq, positions, token_seq, block_table, table_stride,
+        (float*)key_pages, (float*)value_pages, q_heads, kv_heads, head_dim, rotary_dim, block_size,
+        num_blocks, eps, write_kv, (int)work);
+  else if (dtype == FE_BF16)
+    qk_norm_rope_write_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>(
+        (bf16_t*)qkv, q_weight, k_weight, inv_freq, positions, token_seq, block_table, table_stride,
+        (bf16_t*)key_pages, (bf16_t*)value_pages, q_heads, kv_heads, head_dim, rotary_dim, block_size,
+        num_blocks, eps, write_kv, (int)work);
+  else
+    return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}

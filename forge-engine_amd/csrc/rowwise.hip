@@ -1,0 +1,150 @@
+// Row-wise kernels: embedding gather, (residual add +) RMSNorm, SwiGLU.
+// The residual stream is float32 in every mode; activations handed to matrix
+// products are float32 or bfloat16.
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+// out[t, :] = float(table[ids[t], :]).  One block per token.
+template <typename TW>
+__global__ void embed_rows_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
+                                  float* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  float* dst = out + (size_t)t * hidden;
+  if (id < 0 || id >= vocab) {  // host validates ids; never read outside the table
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = __int_as_float(0x7fc00000);
+    return;
+  }
+  const TW* src = table + (size_t)id * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = load_as_float(src + i);
+}
+
+extern "C" int fe_embed_rows(const int* ids, const void* table, int table_dtype, float* out,
+                             int tokens, int hidden, int vocab, hipStream_t stream) {
+  if (tokens <= 0) return FE_OK;
+  if (hidden <= 0 || vocab <= 0) return FE_BAD_ARGUMENT;
+  const int threads = hidden >= 1024 ? 256 : 64;
+  if (table_dtype == FE_F32)
+    embed_rows_kernel<float><<<tokens, threads, 0, stream>>>(ids, (const float*)table, out, hidden, vocab);
+  else if (table_dtype == FE_BF16)
+    embed_rows_kernel<bf16_t><<<tokens, threads, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, vocab);
+  else
+    return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
+// ------------------------------------------------------- add + RMSNorm
+// For output row r (source row s = rows ? rows[r] : r):
+//   sum = h[s] + delta[s]          (float32; written back to h[s] if store_sum)
+//   out[r] = sum * rsqrt(mean(sum^2) + eps) * w
+// Statistics, scaling and the weight product are float32; one rounding at the
+// store.  One block per row; the row is re-read from h/delta in the second
+// pass (it is cache-resident), so any width works.
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                   const float* __restrict__ w, TO* __restrict__ out,
+                                   const int* __restrict__ rows, int hidden, float eps,
+                                   int store_sum) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int s = rows ? rows[r] : r;
+  float* hrow = h + (size_t)s * hidden;
+  const TD* drow = delta ? delta + (size_t)s * hidden : nullptr;
+  float sumsq = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = hrow[i];
+    if (drow) {
+      v += load_as_float(drow + i);
+      if (store_sum) hrow[i] = v;
+    }
+    sumsq += v * v;
+  }
+  const float total = block_sum(sumsq, scratch);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+  TO* orow = out + (size_t)r * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = hrow[i];
+    if (drow && !store_sum) v += load_as_float(drow + i);
+    store_from_float(orow + i, v * inv * w[i]);
+  }
+}
+
+template <typename TD>
+static int launch_add_rmsnorm(float* h, const TD* delta, const float* w, void* out, int out_dtype,
+                              const int* rows, int n_rows, int hidden, float eps, int store_sum,
+                              hipStream_t stream) {
+  const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
+  if (out_dtype == FE_F32)
+    add_rmsnorm_kernel<TD, float><<<n_rows, threads, 0, stream>>>(h, delta, w, (float*)out, rows, hidden, eps, store_sum);
+  else if (out_dtype == FE_BF16)
+    add_rmsnorm_kernel<TD, bf16_t><<<n_rows, threads, 0, stream>>>(h, delta, w, (bf16_t*)out, rows, hidden, eps, store_sum);
+  else
+    return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
+// delta may be null (plain RMSNorm).  rows may be null (all n_rows rows in order).
+// With rows given, store_sum must be 0 unless the rows are distinct.
+extern "C" int fe_add_rmsnorm(float* h, const void* delta, int delta_dtype, const float* w,
+                              void* out, int out_dtype, const int* rows, int n_rows, int hidden,
+                              float eps, int store_sum, hipStream_t stream) {
+  if (n_rows <= 0) return FE_OK;
+  if (hidden <= 0 || !(eps > 0.f)) return FE_BAD_ARGUMENT;
+  if (delta == nullptr || delta_dtype == FE_F32)
+    return launch_add_rmsnorm<float>(h, (const float*)delta, w, out, out_dtype, rows, n_rows, hidden, eps, store_sum, stream);
+  if (delta_dtype == FE_BF16)
+    return launch_add_rmsnorm<bf16_t>(h, (const bf16_t*)delta, w, out, out_dtype, rows, n_rows, hidden, eps, store_sum, stream);
+  return FE_BAD_ARGUMENT;
+}
+
+// h[t] += delta[t] for all rows (flushes a pending update without a norm).
+template <typename TD>
+__global__ void add_rows_kernel(float* __restrict__ h, const TD* __restrict__ delta, size_t count) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+    h[i] += load_as_float(delta + i);
+}
+
+extern "C" int fe_add_rows(float* h, const void* delta, int delta_dtype, long long count, hipStream_t stream) {
+  if (count <= 0) return FE_OK;
+  const int threads = 256;
+  long long want = (count + threads - 1) / threads;
+  const int blocks = (int)(want < 4096 ? want : 4096);
+  if (delta_dtype == FE_F32)
+    add_rows_kernel<float><<<blocks, threads, 0, stream>>>(h, (const float*)delta, (size_t)count);
+  else if (delta_dtype == FE_BF16)
+    add_rows_kernel<bf16_t><<<blocks, threads, 0, stream>>>(h, (const bf16_t*)delta, (size_t)count);
+  else
+    return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}
+
+// ---------------------------------------------------------------- SwiGLU
+// gate_up is [T, 2*inter] with gate in the first half of each row:
+//   out[t, i] = silu(gate[t, i]) * up[t, i],  silu(z) = z / (1 + exp(-z)),  in float32.
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = i / inter;
+    const int c = (int)(i - t * inter);
+    const T* row = gate_up + t * 2 * (size_t)inter;
+    const float g = load_as_float(row + c);
+    const float u = load_as_float(row + inter + c);
+    store_from_float(out + i, g / (1.f + expf(-g)) * u);
+  }
+}
+
+extern "C" int fe_swiglu(const void* gate_up, void* out, int dtype, int tokens, int inter, hipStream_t stream) {
+  if (tokens <= 0) return FE_OK;
+  if (inter <= 0) return FE_BAD_ARGUMENT;
+  const size_t total = (size_t)tokens * inter;
+  const int threads = 256;
+  size_t want = (total + threads - 1) / threads;
+  const int blocks = (int)(want < 8192 ? want : 8192);
+  if (dtype == FE_F32)
+    swiglu_kernel<float><<<blocks, threads, 0, stream>>>((const float*)gate_up, (float*)out, inter, total);
+  else if (dtype == FE_BF16)
+    swiglu_kernel<bf16_t><<<blocks, threads, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total);
+  else
+    return FE_BAD_ARGUMENT;
+  return fe_check_launch();
+}

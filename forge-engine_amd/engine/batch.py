@@ -1,0 +1,88 @@
+"""The flat batch of one step: the tokens of every request in it, one after the
+other, with the metadata the kernels index by."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+from torch import Tensor
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its next tokens (a portion of its prompt,
+    or one decoded token) and the places among them whose logits are wanted."""
+
+    request_id: str
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_seqs: int
+    num_wanted: int
+    max_q_len: int
+    max_ctx: int
+    token_ids: Tensor       # int32 [T]
+    positions: Tensor       # int32 [T]   absolute position of each token in its request
+    token_seq: Tensor       # int32 [T]   index of the token's request within the batch
+    cu_q: Tensor            # int32 [B+1] prefix sums of the requests' token counts
+    ctx_len: Tensor         # int32 [B]   tokens the request holds after this step
+    ctx_before: Tensor      # int32 [B]   tokens it held before
+    state_slots: Tensor     # int32 [B]   slot of its fixed-size state
+    want_rows: Tensor       # int32 [W]   flat token indices whose logits are returned
+    block_tables: list      # per cache group: int32 [B, max_blocks], -1 where no page
+    request_ids: list       # host copies, for parts that decide on the host
+    q_lens: list
+    ctx_before_host: list
+
+
+def build_batch(entries, lengths_before, state_slots, tables_per_group, device) -> StepBatch:
+    """Pack the step's metadata into one int32 buffer and copy it to the
+    device in one transfer.  ``tables_per_group[g][i]`` is request i's page
+    list in cache group g."""
+    num_seqs = len(entries)
+    q_lens = [len(e.tokens) for e in entries]
+    total = sum(q_lens)
+    token_ids, positions, token_seq, want_rows = [], [], [], []
+    cu_q = [0]
+    for i, entry in enumerate(entries):
+        start = lengths_before[i]
+        token_ids.extend(entry.tokens)
+        positions.extend(range(start, start + q_lens[i]))
+        token_seq.extend([i] * q_lens[i])
+        want_rows.extend(cu_q[-1] + w for w in entry.want)
+        cu_q.append(cu_q[-1] + q_lens[i])
+    ctx_len = [lengths_before[i] + q_lens[i] for i in range(num_seqs)]
+    widths = [max(1, max((len(t) for t in tables), default=1)) for tables in tables_per_group]
+    flat_tables = []
+    for tables, width in zip(tables_per_group, widths):
+        for table in tables:
+            flat_tables.extend(table)
+            flat_tables.extend([-1] * (width - len(table)))
+    sections = [token_ids, positions, token_seq, cu_q, ctx_len, list(lengths_before), list(state_slots),
+                want_rows, flat_tables]
+    host = torch.tensor([v for section in sections for v in section], dtype=torch.int32)
+    if device.type == "cuda":
+        host = host.pin_memory()
+    flat = host.to(device, non_blocking=True)
+    views = []
+    offset = 0
+    for section in sections:
+        views.append(flat[offset:offset + len(section)])
+        offset += len(section)
+    block_tables = []
+    table_flat = views[8]
+    offset = 0
+    for width in widths:
+        block_tables.append(table_flat[offset:offset + num_seqs * width].view(num_seqs, width))
+        offset += num_seqs * width
+    return StepBatch(
+        num_tokens=total, num_seqs=num_seqs, num_wanted=len(want_rows), max_q_len=max(q_lens),
+        max_ctx=max(ctx_len), token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
+        ctx_len=views[4], ctx_before=views[5], state_slots=views[6], want_rows=views[7],
+        block_tables=block_tables, request_ids=[e.request_id for e in entries], q_lens=q_lens,
+        ctx_before_host=list(lengths_before))

@@ -1,0 +1,309 @@
+"""Typed Python entry points of the HIP kernels.
+
+Every function checks its operands on the host (device, dtype, layout, sizes)
+before the launch, because a kernel that reads outside its buffers can take the
+GPU down.  Nothing here computes on the CPU and nothing falls back to another
+implementation: without a GPU or without the compiled library a call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_longlong, c_void_p
+
+import torch
+from torch import Tensor
+
+from . import library
+
+FE_F32 = 0
+FE_BF16 = 1
+_STATUS = {1: "bad argument", 2: "launch failed"}
+_DTYPE_CODE = {torch.float32: FE_F32, torch.bfloat16: FE_BF16}
+
+
+class KernelError(RuntimeError):
+    """A kernel entry point refused its arguments or failed to launch."""
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16, not {dtype}") from None
+
+
+def _gpu(tensor: Tensor, name: str, dtype=None, contiguous: bool = True) -> Tensor:
+    if not isinstance(tensor, Tensor):
+        raise KernelError(f"{name} must be a tensor")
+    if tensor.device.type != "cuda":
+        raise KernelError(f"{name} must live on the GPU (got {tensor.device}); there is no CPU path")
+    if dtype is not None and tensor.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {tensor.dtype}")
+    if contiguous and not tensor.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    return tensor
+
+
+def _ptr(tensor: Tensor | None) -> c_void_p:
+    return c_void_p(0 if tensor is None else tensor.data_ptr())
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _call(lib_name: str, fn_name: str, *args) -> None:
+    fn = getattr(library.load(lib_name), fn_name)
+    fn.restype = c_int
+    status = fn(*args)
+    if status != 0:
+        raise KernelError(f"{fn_name}: {_STATUS.get(status, status)}")
+
+
+# ------------------------------------------------------------------ row-wise
+
+def embed_rows(ids: Tensor, table: Tensor, out: Tensor) -> Tensor:
+    """out[t] = float32(table[ids[t]]); ids int32 [T], table [V, H], out float32 [T, H]."""
+    _gpu(ids, "ids", torch.int32)
+    _gpu(table, "table")
+    _gpu(out, "out", torch.float32)
+    tokens = ids.numel()
+    vocab, hidden = table.shape
+    if out.shape != (tokens, hidden):
+        raise KernelError(f"out must be [{tokens}, {hidden}], got {tuple(out.shape)}")
+    _call("rowwise", "fe_embed_rows", _ptr(ids), _ptr(table), c_int(_code(table.dtype)), _ptr(out),
+          c_int(tokens), c_int(hidden), c_int(vocab), _stream())
+    return out
+
+
+def add_rmsnorm(h: Tensor, delta: Tensor | None, weight: Tensor, eps: float, out: Tensor,
+                rows: Tensor | None = None, store_sum: bool = True) -> Tensor:
+    """sum = h[s] + delta[s] (float32, written back to h if store_sum);
+    out[r] = sum * rsqrt(mean(sum^2) + eps) * weight, s = rows[r] or r."""
+    _gpu(h, "h", torch.float32)
+    _gpu(weight, "weight", torch.float32)
+    _gpu(out, "out")
+    total_rows, hidden = h.shape
+    if weight.shape != (hidden,):
+        raise KernelError(f"weight must be [{hidden}], got {tuple(weight.shape)}")
+    if delta is not None:
+        _gpu(delta, "delta")
+        if delta.shape != h.shape:
+            raise KernelError(f"delta must be {tuple(h.shape)}, got {tuple(delta.shape)}")
+    n_rows = total_rows
+    if rows is not None:
+        _gpu(rows, "rows", torch.int32)
+        n_rows = rows.numel()
+        if store_sum and delta is not None:
+            raise KernelError("store_sum with a row list is not allowed (rows may repeat)")
+    if out.shape != (n_rows, hidden):
+        raise KernelError(f"out must be [{n_rows}, {hidden}], got {tuple(out.shape)}")
+    if not eps > 0.0:
+        raise KernelError("eps must be positive")
+    _call("rowwise", "fe_add_rmsnorm", _ptr(h), _ptr(delta),
+          c_int(_code(delta.dtype) if delta is not None else FE_F32), _ptr(weight), _ptr(out),
+          c_int(_code(out.dtype)), _ptr(rows), c_int(n_rows), c_int(hidden), c_float(eps),
+          c_int(1 if (store_sum and delta is not None) else 0), _stream())
+    return out
+
+
+def add_rows(h: Tensor, delta: Tensor) -> Tensor:
+    """h += delta, in float32."""
+    _gpu(h, "h", torch.float32)
+    _gpu(delta, "delta")
+    if delta.shape != h.shape:
+        raise KernelError(f"delta must be {tuple(h.shape)}, got {tuple(delta.shape)}")
+    _call("rowwise", "fe_add_rows", _ptr(h), _ptr(delta), c_int(_code(delta.dtype)),
+          c_longlong(h.numel()), _stream())
+    return h
+
+
+def swiglu(gate_up: Tensor, out: Tensor) -> Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+    _gpu(gate_up, "gate_up")
+    _gpu(out, "out", gate_up.dtype)
+    tokens, two_inter = gate_up.shape
+    if two_inter % 2 or out.shape != (tokens, two_inter // 2):
+        raise KernelError(f"out must be [{tokens}, {two_inter // 2}], got {tuple(out.shape)}")
+    _call("rowwise", "fe_swiglu", _ptr(gate_up), _ptr(out), c_int(_code(out.dtype)), c_int(tokens),
+          c_int(two_inter // 2), _stream())
+    return out
+
+
+# ------------------------------------------------------------ matrix products
+
+def gemm_nt_f32(a: Tensor, b: Tensor, bias: Tensor | None = None, out: Tensor | None = None) -> Tensor:
+    """out[M, N] = a[M, K] @ b[N, K]^T (+ bias), true float32 (FMA, no matrix cores)."""
+    _gpu(a, "a", torch.float32, contiguous=False)
+    _gpu(b, "b", torch.float32, contiguous=False)
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise KernelError(f"shapes {tuple(a.shape)} x {tuple(b.shape)}^T do not match")
+    if a.stride(1) != 1 or b.stride(1) != 1:
+        raise KernelError("both operands must be contiguous along K")
+    m, k = a.shape
+    n = b.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    _gpu(out, "out", torch.float32)
+    if out.shape != (m, n):
+        raise KernelError(f"out must be [{m}, {n}], got {tuple(out.shape)}")
+    if bias is not None:
+        _gpu(bias, "bias", torch.float32)
+        if bias.shape != (n,):
+            raise KernelError(f"bias must be [{n}]")
+    lda = a.stride(0) if m > 1 else max(k, a.stride(0))
+    ldb = b.stride(0) if n > 1 else max(k, b.stride(0))
+    _call("gemm_f32", "fe_gemm_nt_f32", _ptr(a), _ptr(b), _ptr(bias), _ptr(out), c_int(m), c_int(n),
+          c_int(k), c_longlong(lda), c_longlong(ldb), c_longlong(n), _stream())
+    return out
+
+
+def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
+    """y = x @ weight^T (+ bias) for a weight in [out, in] layout.
+
+    float32 weights go through the true float32 kernel (a weight stored in
+    32-bit stays 32-bit even in a bfloat16 model; the activation is widened).
+    bfloat16 weights use the platform's matrix library, as the reference does
+    for every projection (its nn.Linear calls, qwen3.py:115-122,215-223).
+    """
+    _gpu(x, "x")
+    _gpu(weight, "weight")
+    if weight.dtype == torch.float32:
+        y = gemm_nt_f32(x if x.dtype == torch.float32 else x.float(), weight, bias)
+        return y if x.dtype == torch.float32 else y.to(x.dtype)
+    if x.dtype != weight.dtype:
+        raise KernelError(f"activation {x.dtype} does not match weight {weight.dtype}")
+    y = torch.matmul(x, weight.t())
+    if bias is not None:
+        y += bias
+    return y
+
+
+# ------------------------------------------------------------------ attention
+
+def qk_norm_rope_write(qkv: Tensor, q_weight: Tensor | None, k_weight: Tensor | None,
+                       inv_freq: Tensor | None, positions: Tensor, token_seq: Tensor,
+                       block_table: Tensor, key_pages: Tensor, value_pages: Tensor, *, q_heads: int,
+                       kv_heads: int, head_dim: int, rotary_dim: int, eps: float,
+                       write_kv: bool = True) -> None:
+    """Per-head RMSNorm of q and k, rotation, and the write of k, v into pages.
+
+    qkv [T, (Hq + 2 Hkv) D] is changed in place (q part); pages are
+    [blocks, Hkv, block_size, D]; block_table [B, max_blocks] int32.
+    """
+    _gpu(qkv, "qkv")
+    tokens = qkv.shape[0]
+    width = (q_heads + (2 * kv_heads if write_kv else 0)) * head_dim  # q only when nothing is written
+    if qkv.dim() != 2 or qkv.shape[1] != width:
+        raise KernelError(f"qkv must be [T, {width}], got {tuple(qkv.shape)}")
+    for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+        if w is not None:
+            _gpu(w, name, torch.float32)
+            if w.shape != (head_dim,):
+                raise KernelError(f"{name} must be [{head_dim}]")
+    if rotary_dim:
+        _gpu(inv_freq, "inv_freq", torch.float32)
+        if inv_freq.shape != (rotary_dim // 2,):
+            raise KernelError(f"inv_freq must be [{rotary_dim // 2}]")
+    _gpu(positions, "positions", torch.int32)
+    _gpu(token_seq, "token_seq", torch.int32)
+    if positions.numel() != tokens or token_seq.numel() != tokens:
+        raise KernelError("positions and token_seq must have one entry per token")
+    _gpu(block_table, "block_table", torch.int32)
+    _gpu(key_pages, "key_pages", qkv.dtype)
+    _gpu(value_pages, "value_pages", qkv.dtype)
+    if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
+        raise KernelError(f"pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
+    if value_pages.shape != key_pages.shape:
+        raise KernelError("key and value pages must have one shape")
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [sequences, max_blocks]")
+    num_blocks, _, block_size, _ = key_pages.shape
+    _call("qk_rope", "fe_qk_norm_rope_write", _ptr(qkv), c_int(_code(qkv.dtype)), _ptr(q_weight),
+          _ptr(k_weight), _ptr(inv_freq if rotary_dim else None), _ptr(positions), _ptr(token_seq),
+          _ptr(block_table), c_int(block_table.stride(0)), _ptr(key_pages), _ptr(value_pages),
+          c_int(tokens), c_int(q_heads), c_int(kv_heads if write_kv else 0), c_int(head_dim), c_int(rotary_dim),
+          c_int(block_size), c_int(num_blocks), c_float(eps), c_int(1 if write_kv else 0), _stream())
+
+
+def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tensor, cu_q: Tensor,
+                    ctx_len: Tensor, block_table: Tensor, *, num_seqs: int, max_q_len: int,
+                    q_heads: int, kv_heads: int, head_dim: int, scale: float,
+                    window: int | None = None) -> Tensor:
+    """Attention of every query token of a mixed batch over its paged keys.
+
+    q: [T, >= Hq*D] (row stride may exceed Hq*D: the q part of a fused qkv
+    buffer); out [T, Hq*D]; cu_q int32 [B+1]; ctx_len int32 [B] (keys after the
+    step, the step's own included); block_table int32 [B, max_blocks].
+    """
+    _gpu(q, "q", contiguous=False)
+    _gpu(out, "out", q.dtype)
+    _gpu(key_pages, "key_pages", q.dtype)
+    _gpu(value_pages, "value_pages", q.dtype)
+    _gpu(cu_q, "cu_q", torch.int32)
+    _gpu(ctx_len, "ctx_len", torch.int32)
+    _gpu(block_table, "block_table", torch.int32)
+    tokens = q.shape[0]
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < q_heads * head_dim:
+        raise KernelError(f"q must be [T, >= {q_heads * head_dim}] with unit inner stride")
+    if out.shape != (tokens, q_heads * head_dim):
+        raise KernelError(f"out must be [{tokens}, {q_heads * head_dim}], got {tuple(out.shape)}")
+    if q_heads % kv_heads:
+        raise KernelError("query heads must be a multiple of kv heads")
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise KernelError(f"head size {head_dim} is not a multiple of 16 in [16, 256]")
+    if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
+        raise KernelError(f"pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
+    if value_pages.shape != key_pages.shape:
+        raise KernelError("key and value pages must have one shape")
+    if cu_q.numel() != num_seqs + 1 or ctx_len.numel() != num_seqs or block_table.shape[0] < num_seqs:
+        raise KernelError("cu_q, ctx_len and block_table do not match the number of sequences")
+    if q.data_ptr() % 16 or (q.stride(0) if tokens > 1 else 0) % 4:
+        raise KernelError("q rows must be 16-byte aligned")
+    num_blocks, _, block_size, _ = key_pages.shape
+    q_stride = q.stride(0) if tokens > 1 else q.shape[1]
+    _call("attention_generic", "fe_paged_attention_generic", _ptr(q), c_longlong(q_stride),
+          _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)),
+          c_int(_code(q.dtype)), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table),
+          c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(kv_heads),
+          c_int(q_heads // kv_heads), c_int(head_dim), c_int(block_size), c_int(num_blocks),
+          c_int(window or 0), c_float(scale), _stream())
+    return out
+
+
+# ------------------------------------------------------------------- sampling
+
+def argmax_rows(logits: Tensor, tokens: Tensor, status: Tensor) -> None:
+    """tokens[r] = argmax(logits[r]) (lowest index on ties); status bits: 1 NaN, 2 +inf, 4 no finite entry."""
+    _gpu(logits, "logits", torch.float32)
+    _gpu(tokens, "tokens", torch.int32)
+    _gpu(status, "status", torch.int32)
+    rows, vocab = logits.shape
+    if tokens.numel() != rows or status.numel() != rows:
+        raise KernelError("tokens and status need one entry per row")
+    _call("sample", "fe_argmax_rows", _ptr(logits), c_longlong(logits.stride(0)), c_int(rows),
+          c_int(vocab), _ptr(tokens), _ptr(status), _stream())
+
+
+def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index: Tensor,
+                tokens: Tensor, status: Tensor) -> None:
+    """Draw tokens[r] from softmax(logits[r] / temperatures[r]) with the uniform
+    philox(counter=draw_index[r], key=seeds[r]); -inf entries have probability 0."""
+    _gpu(logits, "logits", torch.float32)
+    _gpu(temperatures, "temperatures", torch.float32)
+    _gpu(seeds, "seeds", torch.int64)
+    _gpu(draw_index, "draw_index", torch.int64)
+    _gpu(tokens, "tokens", torch.int32)
+    _gpu(status, "status", torch.int32)
+    rows, vocab = logits.shape
+    for name, t in (("temperatures", temperatures), ("seeds", seeds), ("draw_index", draw_index),
+                    ("tokens", tokens), ("status", status)):
+        if t.numel() != rows:
+            raise KernelError(f"{name} needs one entry per row")
+    _call("sample", "fe_sample_rows", _ptr(logits), c_longlong(logits.stride(0)), c_int(rows),
+          c_int(vocab), _ptr(temperatures), _ptr(seeds), _ptr(draw_index), _ptr(tokens), _ptr(status),
+          _stream())
+
+
+LIBRARIES = ("rowwise", "gemm_f32", "qk_rope", "attention_generic", "sample")

@@ -1,0 +1,335 @@
+"""Each HIP kernel alone against its plain reference (tests/kernel_refs.py), at
+sizes other than the engine's tiny models: widths that are no power of two,
+group sizes 1..5, page sizes 1..32, head sizes 16..256, both dtypes."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+import kernel_refs as refs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from forge_engine_amd.kernels import ops as real_ops
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return real_ops
+
+
+def tol(dtype):
+    return dict(atol=2e-2, rtol=2e-2) if dtype == torch.bfloat16 else dict(atol=1e-5, rtol=1e-5)
+
+
+def rand(gen, *shape, dtype=torch.float32, scale=1.0):
+    return (torch.randn(*shape, generator=gen) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden", [40, 200, 2560])
+def test_embed_rows(ops, dtype, hidden):
+    g = torch.Generator().manual_seed(0)
+    table = rand(g, 77, hidden, dtype=dtype)
+    ids = torch.tensor([0, 76, 5, 5, 31], dtype=torch.int32)
+    want = refs.embed_rows(ids, table, torch.empty(5, hidden))
+    got = ops.embed_rows(ids.to(DEV), table.to(DEV), torch.empty(5, hidden, device=DEV))
+    torch.testing.assert_close(got.cpu(), want, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("delta_dtype", [None, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden", [24, 200, 2560, 5000])
+def test_add_rmsnorm(ops, out_dtype, delta_dtype, hidden):
+    g = torch.Generator().manual_seed(1)
+    h = rand(g, 7, hidden, scale=3.0)
+    delta = None if delta_dtype is None else rand(g, 7, hidden, dtype=delta_dtype)
+    w = 1.0 + rand(g, hidden, scale=0.1)
+    h_ref = h.clone()
+    want = refs.add_rmsnorm(h_ref, delta, w, 1e-5, torch.empty(7, hidden, dtype=out_dtype))
+    h_dev = h.to(DEV)
+    got = ops.add_rmsnorm(h_dev, None if delta is None else delta.to(DEV), w.to(DEV), 1e-5,
+                          torch.empty(7, hidden, dtype=out_dtype, device=DEV))
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(out_dtype))
+    torch.testing.assert_close(h_dev.cpu(), h_ref, atol=1e-6, rtol=1e-6)   # the sum went back into the stream
+
+
+def test_add_rmsnorm_reference_vectors(ops):
+    # the vectors of the reference's own tests (tests/test_qwen3.py:34-44, tests/test_kernels.py:20-36)
+    h = torch.tensor([[1.0, -2.0, 3.0, -4.0]])
+    u = torch.tensor([[0.5, 1.0, -1.5, 2.0]])
+    w = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    got = ops.add_rmsnorm(h.to(DEV), None, w.to(DEV), 1e-6, torch.empty(1, 4, device=DEV)).cpu()
+    torch.testing.assert_close(got, h * torch.rsqrt(h.square().mean(-1, keepdim=True) + 1e-6) * w)
+    h_dev = h.to(DEV)
+    got = ops.add_rmsnorm(h_dev, u.to(DEV), w.to(DEV), 1e-6, torch.empty(1, 4, device=DEV)).cpu()
+    s = h + u
+    torch.testing.assert_close(h_dev.cpu(), s)
+    torch.testing.assert_close(got, s * torch.rsqrt(s.square().mean(-1, keepdim=True) + 1e-6) * w)
+
+
+def test_add_rmsnorm_row_list(ops):
+    g = torch.Generator().manual_seed(2)
+    h = rand(g, 9, 96)
+    w = rand(g, 96)
+    rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32)
+    want = refs.add_rmsnorm(h.clone(), None, w, 1e-6, torch.empty(4, 96), rows=rows, store_sum=False)
+    got = ops.add_rmsnorm(h.to(DEV), None, w.to(DEV), 1e-6, torch.empty(4, 96, device=DEV),
+                          rows=rows.to(DEV), store_sum=False)
+    torch.testing.assert_close(got.cpu(), want, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_rows_and_swiglu(ops, dtype):
+    g = torch.Generator().manual_seed(3)
+    h = rand(g, 5, 136)
+    d = rand(g, 5, 136, dtype=dtype)
+    got = ops.add_rows(h.to(DEV), d.to(DEV)).cpu()
+    torch.testing.assert_close(got, h + d.float())
+    gu = rand(g, 6, 2 * 328, dtype=dtype, scale=2.0)
+    want = refs.swiglu(gu, torch.empty(6, 328, dtype=dtype))
+    got = ops.swiglu(gu.to(DEV), torch.empty(6, 328, dtype=dtype, device=DEV)).cpu()
+    torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
+    # the library expression of the reference's own test (tests/test_cute_swiglu.py:18-27)
+    torch.testing.assert_close(got.float(), (torch.nn.functional.silu(gu[:, :328].float()) * gu[:, 328:].float()), **tol(dtype))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 70, 50), (65, 129, 96), (130, 64, 2560), (17, 1003, 200), (5, 33, 7)])
+def test_gemm_f32(ops, m, n, k):
+    g = torch.Generator().manual_seed(4)
+    a, b, bias = rand(g, m, k), rand(g, n, k), rand(g, n)
+    want = refs.gemm_nt_f32(a, b, bias)
+    got = ops.gemm_nt_f32(a.to(DEV), b.to(DEV), bias.to(DEV)).cpu()
+    torch.testing.assert_close(got, want, atol=1e-4 * math.sqrt(k), rtol=1e-5)
+    # a row's result does not depend on the rows beside it
+    alone = ops.gemm_nt_f32(a[:1].to(DEV).contiguous(), b.to(DEV), bias.to(DEV)).cpu()
+    assert torch.equal(alone[0], got[0])
+
+
+def test_gemm_f32_is_true_float32(ops):
+    # operands whose product needs more than bfloat16's or tf32's mantissa
+    a = torch.tensor([[1.0 + 2**-20, 1.0]])
+    b = torch.tensor([[1.0, -1.0]])
+    got = ops.gemm_nt_f32(a.to(DEV), b.to(DEV)).cpu()
+    assert got.item() == pytest.approx(2**-20, rel=1e-6)
+
+
+def _qk_case(g, dtype, tokens, q_heads, kv_heads, head_dim, block_size, num_blocks):
+    width = (q_heads + 2 * kv_heads) * head_dim
+    qkv = rand(g, tokens, width, dtype=dtype)
+    qw, kw = 1.0 + rand(g, head_dim, scale=0.1), 1.0 + rand(g, head_dim, scale=0.1)
+    # two sequences: tokens [0, split) belong to sequence 1 at positions 5.., the rest to sequence 0 from 0
+    split = tokens // 2
+    positions = torch.tensor(list(range(5, 5 + split)) + list(range(tokens - split)), dtype=torch.int32)
+    token_seq = torch.tensor([1] * split + [0] * (tokens - split), dtype=torch.int32)
+    need = (max(int(positions.max()) + 1, 1) + block_size - 1) // block_size
+    perm = torch.randperm(num_blocks, generator=g)[: 2 * need].to(torch.int32)
+    table = perm.view(2, need).contiguous()
+    return qkv, qw, kw, positions, token_seq, table
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size,rotary_dim", [
+    (4, 2, 16, 4, 16), (6, 2, 32, 8, 32), (5, 1, 128, 16, 128), (3, 3, 64, 1, 32), (8, 2, 256, 32, 256),
+    (2, 1, 48, 5, 0),
+])
+def test_qk_norm_rope_write(ops, dtype, q_heads, kv_heads, head_dim, block_size, rotary_dim):
+    g = torch.Generator().manual_seed(5)
+    tokens, num_blocks = 11, 40
+    qkv, qw, kw, positions, token_seq, table = _qk_case(g, dtype, tokens, q_heads, kv_heads, head_dim, block_size, num_blocks)
+    inv_freq = None
+    if rotary_dim:
+        inv_freq = 1.0 / (10000.0 ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+    shape = (num_blocks, kv_heads, block_size, head_dim)
+    kp_ref, vp_ref = torch.zeros(shape, dtype=dtype), torch.zeros(shape, dtype=dtype)
+    qkv_ref = qkv.clone()
+    refs.qk_norm_rope_write(qkv_ref, qw, kw, inv_freq, positions, token_seq, table, kp_ref, vp_ref,
+                            q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, rotary_dim=rotary_dim, eps=1e-6)
+    qkv_dev = qkv.to(DEV)
+    kp, vp = torch.zeros(shape, dtype=dtype, device=DEV), torch.zeros(shape, dtype=dtype, device=DEV)
+    ops.qk_norm_rope_write(qkv_dev, qw.to(DEV), kw.to(DEV), None if inv_freq is None else inv_freq.to(DEV),
+                           positions.to(DEV), token_seq.to(DEV), table.to(DEV), kp, vp, q_heads=q_heads,
+                           kv_heads=kv_heads, head_dim=head_dim, rotary_dim=rotary_dim, eps=1e-6)
+    qs = q_heads * head_dim
+    torch.testing.assert_close(qkv_dev.cpu()[:, :qs].float(), qkv_ref[:, :qs].float(), **tol(dtype))
+    torch.testing.assert_close(kp.cpu().float(), kp_ref.float(), **tol(dtype))
+    torch.testing.assert_close(vp.cpu().float(), vp_ref.float(), atol=0, rtol=0)
+    assert torch.equal(qkv_dev.cpu()[:, qs:], qkv[:, qs:])   # the k and v parts of the buffer stay
+
+
+def test_rotation_sign_and_pairing_on_device(ops):
+    # unit vector in dim 0 at position 1, D = 4, theta 10000 -> (cos 1, 0, sin 1, 0)
+    qkv = torch.zeros(1, 12)
+    qkv[0, 0] = 1.0          # q
+    qkv[0, 5] = 1.0          # k, dim 1
+    inv_freq = torch.tensor([1.0, 0.01])
+    kp, vp = torch.zeros(2, 1, 2, 4, device=DEV), torch.zeros(2, 1, 2, 4, device=DEV)
+    dev = qkv.to(DEV)
+    ops.qk_norm_rope_write(dev, None, None, inv_freq.to(DEV), torch.tensor([1], dtype=torch.int32, device=DEV),
+                           torch.tensor([0], dtype=torch.int32, device=DEV),
+                           torch.tensor([[1]], dtype=torch.int32, device=DEV), kp, vp, q_heads=1, kv_heads=1,
+                           head_dim=4, rotary_dim=4, eps=1.0)
+    torch.testing.assert_close(dev.cpu()[0, :4], torch.tensor([math.cos(1.0), 0.0, math.sin(1.0), 0.0]))
+    torch.testing.assert_close(kp.cpu()[1, 0, 1], torch.tensor([0.0, math.cos(0.01), 0.0, math.sin(0.01)]))
+
+
+def _attention_case(g, dtype, seqs, q_heads, kv_heads, head_dim, block_size, extra_width=0):
+    """seqs: list of (ctx_before, q_len).  Builds pages with shuffled page ids."""
+    total_q = sum(q for _, q in seqs)
+    blocks_needed = [(b + q + block_size - 1) // block_size for b, q in seqs]
+    num_blocks = sum(blocks_needed) + 3
+    perm = torch.randperm(num_blocks, generator=g).tolist()
+    width = max(blocks_needed)
+    table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    at = 0
+    for s, n in enumerate(blocks_needed):
+        table[s, :n] = torch.tensor(perm[at:at + n], dtype=torch.int32)
+        at += n
+    shape = (num_blocks, kv_heads, block_size, head_dim)
+    kp, vp = rand(g, *shape, dtype=dtype), rand(g, *shape, dtype=dtype)
+    q = rand(g, total_q, q_heads * head_dim + extra_width, dtype=dtype)
+    cu = torch.tensor([0] + list(torch.tensor([q for _, q in seqs]).cumsum(0)), dtype=torch.int32)
+    ctx = torch.tensor([b + q for b, q in seqs], dtype=torch.int32)
+    return q, kp, vp, cu, ctx, table
+
+
+def _run_attention(ops, q, kp, vp, cu, ctx, table, *, q_heads, kv_heads, head_dim, window=None, scale=None):
+    scale = head_dim ** -0.5 if scale is None else scale
+    num_seqs = ctx.numel()
+    max_q = int((cu[1:] - cu[:-1]).max())
+    kw = dict(num_seqs=num_seqs, max_q_len=max_q, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+              scale=scale, window=window)
+    want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype), cu, ctx, table, **kw)
+    got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV),
+                              torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype, device=DEV),
+                              cu.to(DEV), ctx.to(DEV), table.to(DEV), **kw)
+    return got.cpu().float(), want.float()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [
+    (4, 2, 16, 4), (6, 2, 32, 8), (10, 2, 128, 16), (5, 5, 64, 1), (3, 1, 256, 32), (7, 1, 48, 3), (16, 1, 16, 64),
+])
+def test_paged_attention_mixed_batch(ops, dtype, q_heads, kv_heads, head_dim, block_size):
+    g = torch.Generator().manual_seed(6)
+    seqs = [(0, 37), (70, 1), (13, 9), (0, 1), (130, 2), (63, 1)]
+    case = _attention_case(g, dtype, seqs, q_heads, kv_heads, head_dim, block_size, extra_width=2 * kv_heads * head_dim)
+    got, want = _run_attention(ops, *case, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim)
+    torch.testing.assert_close(got, want, **tol(dtype))
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 40])
+def test_paged_attention_window(ops, window):
+    g = torch.Generator().manual_seed(7)
+    seqs = [(0, 50), (45, 1), (30, 7)]
+    case = _attention_case(g, torch.float32, seqs, 4, 2, 32, 8)
+    got, want = _run_attention(ops, *case, q_heads=4, kv_heads=2, head_dim=32, window=window)
+    torch.testing.assert_close(got, want, atol=1e-5, rtol=1e-5)
+
+
+def test_paged_attention_is_library_attention(ops):
+    # whole prompt, nothing cached: the library's causal attention after group expansion
+    # (the reference pins its own kernels the same way, tests/test_kernels.py:91-105)
+    g = torch.Generator().manual_seed(8)
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.float32, [(0, 21)], 6, 2, 32, 8)
+    got, _ = _run_attention(ops, q, kp, vp, cu, ctx, table, q_heads=6, kv_heads=2, head_dim=32)
+    keys = refs.gather_pages(kp, table[0], 21, 8)
+    values = refs.gather_pages(vp, table[0], 21, 8)
+    lib = torch.nn.functional.scaled_dot_product_attention(
+        q.view(21, 6, 32).transpose(0, 1).unsqueeze(0), keys.repeat_interleave(3, 0).unsqueeze(0),
+        values.repeat_interleave(3, 0).unsqueeze(0), is_causal=True)[0]
+    torch.testing.assert_close(got, lib.transpose(0, 1).reshape(21, 192), atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_paged_attention_far_key_stands_out(ops, dtype):
+    # one key among hundreds, early in the sequence and in the middle of a page,
+    # gets a score far above the rest: the output must be its value row
+    g = torch.Generator().manual_seed(9)
+    head_dim, block_size, ctx_len = 64, 16, 700
+    q, kp, vp, cu, ctx, table = _attention_case(g, dtype, [(ctx_len - 1, 1)], 2, 1, head_dim, block_size)
+    q = q * 0.01
+    far = 37
+    page, slot = int(table[0, far // block_size]), far % block_size
+    kp[page, 0, slot] = 0.0
+    kp[page, 0, slot, 3] = 40.0
+    q[0, 3] = 40.0
+    q[0, head_dim + 3] = 40.0
+    got, want = _run_attention(ops, q, kp, vp, cu, ctx, table, q_heads=2, kv_heads=1, head_dim=head_dim)
+    torch.testing.assert_close(got, want, **tol(dtype))
+    torch.testing.assert_close(got[0, :head_dim], vp[page, 0, slot].float(), **tol(dtype))
+
+
+def test_argmax_rows(ops):
+    g = torch.Generator().manual_seed(10)
+    logits = rand(g, 5, 1003)
+    logits[1, 17] = logits[1, 900] = 50.0          # tie: lowest index
+    logits[2, 5] = float("nan")
+    logits[3, :] = float("-inf")
+    logits[4, 7] = float("inf")
+    tokens = torch.zeros(5, dtype=torch.int32, device=DEV)
+    status = torch.zeros(5, dtype=torch.int32, device=DEV)
+    ops.argmax_rows(logits.to(DEV), tokens, status)
+    assert tokens.cpu()[0] == logits[0].argmax() and tokens.cpu()[1] == 17
+    assert status.cpu().tolist() == [0, 0, 1, 4, 2]
+
+
+def test_sample_rows_follows_the_distribution(ops):
+    vocab, draws = 37, 4000
+    g = torch.Generator().manual_seed(11)
+    row = rand(g, vocab, scale=2.0)
+    row[5] = float("-inf")
+    logits = row.repeat(draws, 1).to(DEV)
+    temps = torch.full((draws,), 0.8, device=DEV)
+    seeds = torch.full((draws,), 1234, dtype=torch.int64, device=DEV)
+    index = torch.arange(draws, dtype=torch.int64, device=DEV)
+    tokens = torch.zeros(draws, dtype=torch.int32, device=DEV)
+    status = torch.zeros(draws, dtype=torch.int32, device=DEV)
+    ops.sample_rows(logits, temps, seeds, index, tokens, status)
+    assert int(status.sum()) == 0
+    got = tokens.cpu()
+    # same uniforms, float64 inverse CDF: equal except where the target sits within rounding of a boundary
+    want = torch.zeros(draws, dtype=torch.int32)
+    refs.sample_rows(logits.cpu(), temps.cpu(), seeds.cpu(), index.cpu(), want, torch.zeros(draws, dtype=torch.int32))
+    assert (got != want).sum() <= 2
+    assert (got == 5).sum() == 0
+    probs = torch.softmax(row / 0.8, 0)
+    counts = torch.bincount(got.long(), minlength=vocab).float()
+    expected = probs * draws
+    mask = expected > 5
+    chi2 = (((counts - expected) ** 2 / expected)[mask]).sum()
+    assert chi2 < 2.0 * int(mask.sum()) + 20
+    # a second run with the same seeds and counters repeats the draws; another seed does not
+    again = torch.zeros_like(tokens)
+    ops.sample_rows(logits, temps, seeds, index, again, status)
+    assert torch.equal(again.cpu(), got)
+    ops.sample_rows(logits, temps, seeds + 1, index, again, status)
+    assert not torch.equal(again.cpu(), got)
+
+
+def test_sample_rows_low_temperature_is_argmax(ops):
+    g = torch.Generator().manual_seed(12)
+    logits = rand(g, 8, 1003).to(DEV)
+    tokens = torch.zeros(8, dtype=torch.int32, device=DEV)
+    status = torch.zeros(8, dtype=torch.int32, device=DEV)
+    ops.sample_rows(logits, torch.full((8,), 1e-4, device=DEV), torch.arange(8, dtype=torch.int64, device=DEV),
+                    torch.zeros(8, dtype=torch.int64, device=DEV), tokens, status)
+    assert torch.equal(tokens.cpu().long(), logits.cpu().argmax(-1))
+
+
+def test_kernels_refuse_what_they_cannot_do(ops):
+    from forge_engine_amd.kernels.ops import KernelError
+    with pytest.raises(KernelError, match="GPU"):
+        ops.swiglu(torch.zeros(2, 8), torch.zeros(2, 4))
+    q = torch.zeros(1, 40, device=DEV)
+    pages = torch.zeros(2, 1, 4, 40, device=DEV)
+    with pytest.raises(KernelError, match="head size"):
+        ops.paged_attention(q, pages, pages, torch.zeros(1, 40, device=DEV),
+                            torch.tensor([0, 1], dtype=torch.int32, device=DEV),
+                            torch.tensor([1], dtype=torch.int32, device=DEV),
+                            torch.zeros(1, 1, dtype=torch.int32, device=DEV), num_seqs=1, max_q_len=1,
+                            q_heads=1, kv_heads=1, head_dim=40, scale=1.0)
