@@ -1,0 +1,82 @@
+"""Sampling parameters and the logits filters (CPU).  The draw kernels are
+covered by the GPU tests."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+import kernel_refs
+import plain_qwen3 as plain
+from forge_engine_amd.config import EngineConfig
+from forge_engine_amd.sampling import SamplingParams
+from forge_engine_amd.sampling.sampler import Sampler, filter_logits
+
+
+@pytest.mark.parametrize("kwargs", [
+    {"temperature": -0.1}, {"temperature": float("nan")}, {"temperature": float("inf")}, {"top_k": 0},
+    {"top_p": 0.0}, {"top_p": 1.5}, {"min_p": -0.1}, {"min_p": 1.1}, {"max_new_tokens": 0},
+    {"stop_strings": ("",)}, {"stop_strings": ("a", "a")},
+])
+def test_invalid_parameters(kwargs):
+    with pytest.raises(ValueError):
+        SamplingParams(**kwargs)
+    with pytest.raises(ValueError):
+        EngineConfig(**kwargs)
+
+
+def test_defaults_follow_the_reference():
+    p = SamplingParams()
+    assert (p.temperature, p.top_k, p.top_p, p.min_p, p.max_new_tokens, p.stop_strings, p.seed) == (0.0, None, 1.0, 0.0, 256, (), None)
+    assert p.greedy and not SamplingParams(temperature=0.5).greedy
+    assert EngineConfig(temperature=0.7, seed=3).sampling_params() == SamplingParams(temperature=0.7, seed=3)
+
+
+def kept(x):
+    return torch.isfinite(x).nonzero()[:, 1].tolist()
+
+
+def test_filter_vectors_of_the_reference():
+    # tests/test_sampling.py:47-81 of the reference
+    assert kept(filter_logits(torch.tensor([[0.0, 3.0, 2.0, 1.0]]), SamplingParams(temperature=1.0, top_k=2))) == [1, 2]
+    assert kept(filter_logits(torch.tensor([[5.0, 4.0, 0.0]]), SamplingParams(temperature=1.0, top_p=0.7))) == [0]
+    assert kept(filter_logits(torch.tensor([[0.0, -1.0, -3.0]]), SamplingParams(temperature=1.0, min_p=0.2))) == [0, 1]
+    with pytest.raises(ValueError, match="greedy"):
+        filter_logits(torch.zeros(1, 3), SamplingParams())
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_filters_equal_the_plain_implementation(seed):
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(4, 50, generator=g) * 3
+    for p in (SamplingParams(temperature=0.7, top_k=5), SamplingParams(temperature=1.3, top_p=0.6),
+              SamplingParams(temperature=0.9, min_p=0.1), SamplingParams(temperature=0.5, top_k=20, top_p=0.8, min_p=0.05)):
+        got = filter_logits(logits, p)
+        want = plain.filter_logits(logits, p.temperature, p.top_k, p.top_p, p.min_p)
+        assert torch.equal(torch.isfinite(got), torch.isfinite(want))
+        torch.testing.assert_close(got, want)
+
+
+def test_sampler_routes_rows_and_raises_on_bad_logits(monkeypatch):
+    kernel_refs.install(monkeypatch)
+    sampler = Sampler(torch.device("cpu"))
+    logits = torch.tensor([[1.0, 3.0, 2.0], [7.0, -1.0, 4.0], [0.0, 0.0, 9.0]])
+    greedy = SamplingParams()
+    assert sampler.sample(logits[:2], [greedy, greedy], [0, 0], [0, 0]) == [1, 0]    # reference tests/test_sampling.py:40-45
+    only_top = SamplingParams(temperature=1.0, top_k=1)
+    assert sampler.sample(logits, [greedy, only_top, SamplingParams(temperature=1e-3)], [1, 2, 3], [0, 0, 0]) == [1, 0, 2]
+    for bad, match in (([[0.0, float("nan")]], "NaN"), ([[float("-inf")] * 2], "finite"), ([[0.0, float("inf")]], "positive infinity")):
+        with pytest.raises(ValueError, match=match):
+            sampler.sample(torch.tensor(bad), [greedy], [0], [0])
+        with pytest.raises(ValueError, match=match):
+            sampler.sample(torch.tensor(bad), [only_top], [0], [0])
+
+
+def test_uniform_logits_give_uniform_draws(monkeypatch):
+    kernel_refs.install(monkeypatch)
+    sampler = Sampler(torch.device("cpu"))
+    p = SamplingParams(temperature=1.0)
+    draws = [sampler.sample(torch.zeros(1, 8), [p], [731], [i])[0] for i in range(400)]
+    counts = torch.bincount(torch.tensor(draws), minlength=8)
+    assert counts.min() > 25 and counts.max() < 80
+    assert draws == [sampler.sample(torch.zeros(1, 8), [p], [731], [i])[0] for i in range(400)]
