@@ -1,0 +1,250 @@
+// bfloat16 matrix product for few rows (decode): y[M, N] = x[M, K] * W[N, K]^T,
+// M <= 64, float32 accumulation on the matrix cores.  The weight is streamed
+// from HBM exactly once and never staged: every weight element is used by one
+// wave only, so it goes from global memory straight into the MFMA operand
+// registers.  x is small and stays in the L2 cache; each wave reads the part
+// it needs straight into the other operand.
+//
+// Work split: one block per 16, 32 or 64 weight rows (for the gated feed-forward:
+// gate rows and the up rows that go with them); every wave of the block covers
+// all of the block's rows, so one read of x serves them all.  The waves split K among
+// themselves in interleaved 128-wide steps, so that a launch has a few thousand
+// waves with all their loads in flight at once, which is what a product of a
+// few microseconds needs.  The waves' float32 partial sums meet in LDS and are
+// added in wave order: no global scratch, no atomics, and a result that does
+// not depend on timing or on the rows beside it.
+//
+// MFMA 16x16x32 bf16 layout used here (A = x, B = W^T, D = A*B):
+//   lane l supplies A[m = l % 16][k = 8*(l / 16) .. +8] and B[k = 8*(l / 16) .. +8][n = l % 16]
+//   and receives D[m = 4*(l / 16) + i][n = l % 16], i < 4.
+//
+// Epilogues: store float32, store bfloat16, or silu(gate) * up -> bfloat16.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
+
+#define KSTEP 128   // k per wave step: 4 lane groups x 32
+#define ROWS 16     // weight rows per block and tile
+
+#define EPI_F32 0
+#define EPI_BF16 1
+#define EPI_SWIGLU 2
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + __expf(-g)) * u; }
+
+template <int MT, int NW>
+struct StepRegs {
+  uintx4 w[NW][4];
+  uintx4 x[MT][4];
+};
+
+// NT row tiles per wave (for the gated product: NT gate tiles and their NT up
+// tiles), WAVES waves per block sharing K.
+template <int MT, int NT, int EPI, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
+    int K, long long ldw, long long ldo, int second_offset) {
+  constexpr int NW = EPI == EPI_SWIGLU ? 2 * NT : NT;   // weight tiles per wave
+  __shared__ __attribute__((aligned(16))) float red[WAVES][64][4];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int lr = lane & 15;
+  const int lq = lane >> 4;
+  const int base = blockIdx.x * (ROWS * NT);
+
+  const bf16_t* wrow[NW];
+  bool row_ok[NW];
+#pragma unroll
+  for (int t = 0; t < NW; ++t) {
+    const int local = base + (t % NT) * ROWS + lr;   // row within [0, N)
+    row_ok[t] = local < N;
+    wrow[t] = w + (size_t)(row_ok[t] ? local + (t / NT) * second_offset : 0) * ldw;
+  }
+  const bf16_t* xrow[MT];
+  bool x_ok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    x_ok[mt] = mt * 16 + lr < M;
+    xrow[mt] = x + (size_t)(x_ok[mt] ? mt * 16 + lr : 0) * K;
+  }
+
+  floatx4 acc[MT][NW];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NW; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // One step = 128 k = four MFMAs; in MFMA c lane group lq holds k = 32*c + 8*lq .. +8 of
+  // both operands, so one load instruction reads 64 contiguous bytes of each of 16 rows.
+  auto load = [&](StepRegs<MT, NW>& r, int step) {
+    const int k = step * KSTEP + lq * 8;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const bool k_ok = k + c * 32 < K;
+#pragma unroll
+      for (int t = 0; t < NW; ++t) {
+        uintx4 v = uintx4{0u, 0u, 0u, 0u};
+        if (row_ok[t] && k_ok) v = *(const uintx4*)(wrow[t] + k + c * 32);
+        r.w[t][c] = v;
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        uintx4 v = uintx4{0u, 0u, 0u, 0u};
+        if (x_ok[mt] && k_ok) v = *(const uintx4*)(xrow[mt] + k + c * 32);
+        r.x[mt][c] = v;
+      }
+    }
+  };
+  auto multiply = [&](const StepRegs<MT, NW>& r) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, r.x[mt][c]);
+#pragma unroll
+        for (int t = 0; t < NW; ++t)
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, r.w[t][c]), acc[mt][t], 0, 0, 0);
+      }
+  };
+
+  // steps wave, wave + WAVES, ...: two register sets, the next step's loads fly while this one multiplies
+  const int steps = (K + KSTEP - 1) / KSTEP;
+  StepRegs<MT, NW> ra, rb;
+  int step = wave;
+  if (step < steps) load(ra, step);
+  while (step < steps) {
+    const int next = step + WAVES;
+    if (next < steps) load(rb, next);
+    multiply(ra);
+    if (next >= steps) break;
+    const int after = next + WAVES;
+    if (after < steps) load(ra, after);
+    multiply(rb);
+    step = after;
+  }
+
+  // the waves' partial sums meet in LDS, one (m tile, n tile) at a time, and are added in wave order
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int p = 0; p < NT; ++p) {
+      float gate = 0.f;
+#pragma unroll
+      for (int half = 0; half < NW / NT; ++half) {
+        __syncthreads();
+        *(floatx4*)&red[wave][lane][0] = acc[mt][p + half * NT];
+        __syncthreads();
+        if (tid < 256) {
+          const int src_lane = tid >> 2;
+          const int i = tid & 3;
+          float v = 0.f;
+#pragma unroll
+          for (int wv = 0; wv < WAVES; ++wv) v += red[wv][src_lane][i];
+          const int m = mt * 16 + (src_lane >> 4) * 4 + i;
+          const int n = base + p * ROWS + (src_lane & 15);
+          if (m < M && n < N) {
+            if (EPI == EPI_SWIGLU) {
+              if (half == 0) gate = v;
+              else ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(silu_mul(gate, v));
+            } else if (EPI == EPI_F32) {
+              ((float*)out)[(size_t)m * ldo + n] = v;
+            } else {
+              ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(v);
+            }
+          }
+        }
+      }
+    }
+}
+
+template <int MT, int NT, int EPI, int WAVES>
+static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, long long ldw,
+                         long long ldo, int second_offset, hipStream_t stream) {
+  const int blocks = (N + ROWS * NT - 1) / (ROWS * NT);
+  gemm_skinny_kernel<MT, NT, EPI, WAVES><<<blocks, WAVES * 64, 0, stream>>>(
+      (const bf16_t*)x, (const bf16_t*)w, out, M, N, K, ldw, ldo, second_offset);
+  return fe_check_launch();
+}
+
+// Register budget: a wave holds MT x (weight tiles) accumulators and two sets of
+// operand registers; shapes beyond these limits would spill.
+static constexpr bool shape_fits(int mt, int weight_tiles, int waves) {
+  const int registers = 2 * 16 * (weight_tiles + mt) + 4 * mt * weight_tiles;   // operands twice + sums
+  return registers <= 240 && (waves < 16 || (mt == 1 && weight_tiles <= 2));
+}
+
+static int clamp_tiles(int mt, int epilogue, int tiles) {
+  const int pair = epilogue == EPI_SWIGLU ? 2 : 1;
+  while (tiles > 1 && !shape_fits(mt, tiles * pair, 8)) tiles >>= 1;
+  return tiles;
+}
+
+template <int MT, int NT, int EPI>
+static int dispatch_waves(int waves, const void* x, const void* w, void* out, int M, int N, int K,
+                          long long ldw, long long ldo, int second_offset, hipStream_t stream) {
+  constexpr int WT = NT * (EPI == EPI_SWIGLU ? 2 : 1);
+  if constexpr (shape_fits(MT, WT, 16)) {
+    if (waves == 16) return launch_skinny<MT, NT, EPI, 16>(x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+  }
+  if (waves >= 8) return launch_skinny<MT, NT, EPI, 8>(x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+  return launch_skinny<MT, NT, EPI, 4>(x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+}
+
+template <int MT, int EPI>
+static int dispatch_tiles(int nt, int waves, const void* x, const void* w, void* out, int M, int N, int K,
+                          long long ldw, long long ldo, int second_offset, hipStream_t stream) {
+  constexpr int PAIR = EPI == EPI_SWIGLU ? 2 : 1;
+  if constexpr (shape_fits(MT, 4 * PAIR, 8)) {
+    if (nt == 4) return dispatch_waves<MT, 4, EPI>(waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+  }
+  if constexpr (shape_fits(MT, 2 * PAIR, 8)) {
+    if (nt >= 2) return dispatch_waves<MT, 2, EPI>(waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+  }
+  return dispatch_waves<MT, 1, EPI>(waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+}
+
+template <int EPI>
+static int dispatch(int mt, int nt, int waves, const void* x, const void* w, void* out, int M, int N,
+                    int K, long long ldw, long long ldo, int second_offset, hipStream_t stream) {
+  if (mt == 1) return dispatch_tiles<1, EPI>(nt, waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+  if (mt == 2) return dispatch_tiles<2, EPI>(nt, waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+  return dispatch_tiles<4, EPI>(nt, waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+}
+
+// x [M, K] bf16 contiguous; w [N, K] (epilogue 0, 1) or [2N, K] with the gate
+// rows first (epilogue 2), row stride ldw; out [M, N] with row stride ldo,
+// float32 (0) or bf16 (1, 2).  tiles/waves: 0 lets the kernel choose how many
+// 16-row tiles a wave takes (1, 2, 4: more tiles share each read of x) and how
+// many waves share a block's K (4, 8, 16), aiming at a few thousand waves.
+extern "C" int fe_gemm_skinny(const void* x, const void* w, void* out, int M, int N, int K,
+                              long long ldw, long long ldo, int epilogue, int tiles, int waves,
+                              hipStream_t stream) {
+  if (M < 1) return FE_OK;
+  if (M > 64 || N < 1 || K < 8 || K % 8 || ldw < K || ldw % 8 || ldo < N) return FE_BAD_ARGUMENT;
+  if ((((uintptr_t)x) & 15) || (((uintptr_t)w) & 15)) return FE_BAD_ARGUMENT;
+  if (epilogue < 0 || epilogue > 2) return FE_BAD_ARGUMENT;
+  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  const int steps = (K + KSTEP - 1) / KSTEP;
+  const int weight_rows = epilogue == EPI_SWIGLU ? 2 * N : N;
+  if (tiles == 0) {
+    // measured on MI355X: up to 16 rows of x one tile per wave is fastest at every width; with more
+    // rows two tiles share each read of x and win once the weight has a few thousand rows
+    tiles = (mt > 1 && weight_rows >= 4096) ? 2 : 1;
+    if (epilogue == EPI_SWIGLU) tiles = 1;   // a gated tile is already a pair
+  }
+  if (tiles != 1 && tiles != 2 && tiles != 4) return FE_BAD_ARGUMENT;
+  tiles = clamp_tiles(mt, epilogue, tiles);
+  if (waves == 0) {
+    waves = 8;
+    while (waves > 4 && waves > steps) waves >>= 1;
+  }
+  if (waves != 4 && waves != 8 && waves != 16) return FE_BAD_ARGUMENT;
+  if (waves == 16 && !shape_fits(mt, tiles * (epilogue == EPI_SWIGLU ? 2 : 1), 16)) waves = 8;
+  if (epilogue == EPI_SWIGLU) return dispatch<EPI_SWIGLU>(mt, tiles, waves, x, w, out, M, N, K, ldw, ldo, N, stream);
+  if (epilogue == EPI_F32) return dispatch<EPI_F32>(mt, tiles, waves, x, w, out, M, N, K, ldw, ldo, 0, stream);
+  return dispatch<EPI_BF16>(mt, tiles, waves, x, w, out, M, N, K, ldw, ldo, 0, stream);
+}

@@ -159,25 +159,78 @@ def gemm_nt_f32(a: Tensor, b: Tensor, bias: Tensor | None = None, out: Tensor | 
     return out
 
 
-def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
-    """y = x @ weight^T (+ bias) for a weight in [out, in] layout.
+SKINNY_MAX_ROWS = 64       # the decode product takes up to this many tokens
+_EPI_F32, _EPI_BF16, _EPI_SWIGLU = 0, 1, 2
+
+
+def _skinny_fits(x: Tensor, weight: Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2
+            and x.shape[0] <= SKINNY_MAX_ROWS and x.is_contiguous() and x.shape[1] % 8 == 0
+            and weight.stride(1) == 1 and weight.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def gemm_skinny(x: Tensor, weight: Tensor, epilogue: str = "bf16", tiles: int = 0, waves: int = 0) -> Tensor:
+    """y = x @ weight^T for up to 64 rows of bfloat16 x, float32 accumulation.
+
+    epilogue ``f32``/``bf16``: y [M, N] in that dtype; ``swiglu``: weight is
+    [2I, K] with the gate rows first and y = silu(x Wg^T) * (x Wu^T) in bfloat16."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(weight, "weight", torch.bfloat16, contiguous=False)
+    if not _skinny_fits(x, weight):
+        raise KernelError("the skinny product takes at most 64 contiguous bfloat16 rows with K a multiple of 8")
+    m, k = x.shape
+    rows = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"shapes {tuple(x.shape)} x {tuple(weight.shape)}^T do not match")
+    code = {"f32": _EPI_F32, "bf16": _EPI_BF16, "swiglu": _EPI_SWIGLU}[epilogue]
+    if code == _EPI_SWIGLU and rows % 2:
+        raise KernelError("a gated weight needs an even number of rows")
+    n = rows // 2 if code == _EPI_SWIGLU else rows
+    out = torch.empty((m, n), dtype=torch.float32 if code == _EPI_F32 else torch.bfloat16, device=x.device)
+    _call("gemm_skinny", "fe_gemm_skinny", _ptr(x), _ptr(weight), _ptr(out), c_int(m), c_int(n), c_int(k),
+          c_longlong(weight.stride(0)), c_longlong(n), c_int(code), c_int(tiles), c_int(waves), _stream())
+    return out
+
+
+def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None) -> Tensor:
+    """y = x @ weight^T (+ bias) for a weight in [out, in] layout; float32
+    accumulation; y in ``out_dtype`` (default: x's dtype).
 
     float32 weights go through the true float32 kernel (a weight stored in
     32-bit stays 32-bit even in a bfloat16 model; the activation is widened).
-    bfloat16 weights use the platform's matrix library, as the reference does
-    for every projection (its nn.Linear calls, qwen3.py:115-122,215-223).
+    bfloat16: up to 64 rows take the weight-streaming kernel; more rows use the
+    platform's matrix library, as the reference does for every projection (its
+    nn.Linear calls, qwen3.py:115-122,215-223).
     """
     _gpu(x, "x")
-    _gpu(weight, "weight")
+    _gpu(weight, "weight", contiguous=False)
+    out_dtype = x.dtype if out_dtype is None else out_dtype
     if weight.dtype == torch.float32:
         y = gemm_nt_f32(x if x.dtype == torch.float32 else x.float(), weight, bias)
-        return y if x.dtype == torch.float32 else y.to(x.dtype)
+        return y if out_dtype == torch.float32 else y.to(out_dtype)
     if x.dtype != weight.dtype:
         raise KernelError(f"activation {x.dtype} does not match weight {weight.dtype}")
-    y = torch.matmul(x, weight.t())
+    if bias is None and _skinny_fits(x, weight) and out_dtype in (torch.float32, torch.bfloat16):
+        return gemm_skinny(x, weight, "f32" if out_dtype == torch.float32 else "bf16")
+    if out_dtype == torch.float32:
+        y = torch.mm(x, weight.t(), out_dtype=torch.float32)
+    else:
+        y = torch.matmul(x, weight.t())
     if bias is not None:
-        y += bias
+        y += bias.to(y.dtype)
     return y
+
+
+def linear_swiglu(x: Tensor, gate_up_weight: Tensor) -> Tensor:
+    """silu(x Wg^T) * (x Wu^T) for the fused weight [2I, K] (gate rows first)."""
+    _gpu(x, "x")
+    _gpu(gate_up_weight, "gate_up_weight")
+    if _skinny_fits(x, gate_up_weight):
+        return gemm_skinny(x, gate_up_weight, "swiglu")
+    gate_up = linear(x, gate_up_weight)
+    out = torch.empty((x.shape[0], gate_up_weight.shape[0] // 2), dtype=gate_up.dtype, device=x.device)
+    return swiglu(gate_up, out)
 
 
 # ------------------------------------------------------------------ attention
@@ -306,4 +359,4 @@ def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index:
           _stream())
 
 
-LIBRARIES = ("rowwise", "gemm_f32", "qk_rope", "attention_generic", "sample")
+LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "qk_rope", "attention_generic", "sample")

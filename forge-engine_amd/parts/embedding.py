@@ -67,14 +67,11 @@ class LMHead(Head):
         return self._embedding.weight if self.tied else self.weight
 
     def forward(self, z: Tensor) -> Tensor:
-        weight = self.matrix()
-        if weight.dtype == torch.float32:
-            return ops.gemm_nt_f32(z if z.dtype == torch.float32 else z.float(), weight)
-        # bfloat16 operands, float32 accumulation and float32 result (no rounding of the logits)
-        return torch.mm(z, weight.t(), out_dtype=torch.float32)
+        # float32 accumulation and float32 logits in both modes (no rounding of the logits)
+        return ops.linear(z, self.matrix(), out_dtype=torch.float32)
 
     def kernel_libraries(self):
-        return {"gemm_f32"}
+        return {"gemm_f32", "gemm_skinny"}
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)

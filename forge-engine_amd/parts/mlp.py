@@ -44,13 +44,11 @@ class SwiGLU(FeedForward):
             raise KeyError(name)
 
     def forward(self, x: Tensor, batch=None) -> Tensor:
-        gate_up = ops.linear(x, self.gate_up_weight)
-        act = torch.empty((x.shape[0], self.intermediate_size), dtype=gate_up.dtype, device=x.device)
-        ops.swiglu(gate_up, act)
-        return ops.linear(act, self.down_weight)
+        act = ops.linear_swiglu(x, self.gate_up_weight)
+        return ops.linear(act, self.down_weight, out_dtype=torch.float32)   # the update stays float32 for the residual sum
 
     def kernel_libraries(self):
-        return {"rowwise", "gemm_f32"}
+        return {"rowwise", "gemm_f32", "gemm_skinny"}
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

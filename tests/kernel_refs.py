@@ -56,11 +56,24 @@ def gemm_nt_f32(a, b, bias=None, out=None):
     return out
 
 
-def linear(x, weight, bias=None):
+def linear(x, weight, bias=None, out_dtype=None):
     y = x.float() @ weight.float().T
     if bias is not None:
         y = y + bias.float()
-    return y.to(x.dtype)
+    return y.to(x.dtype if out_dtype is None else out_dtype)
+
+
+def linear_swiglu(x, gate_up_weight):
+    inter = gate_up_weight.shape[0] // 2
+    y = x.float() @ gate_up_weight.float().T
+    g, u = y[:, :inter], y[:, inter:]
+    return (g / (1.0 + torch.exp(-g)) * u).to(x.dtype)
+
+
+def gemm_skinny(x, weight, epilogue="bf16", tiles=0, waves=0):
+    if epilogue == "swiglu":
+        return linear_swiglu(x, weight)
+    return linear(x, weight, out_dtype=torch.float32 if epilogue == "f32" else torch.bfloat16)
 
 
 def qk_norm_rope_write(qkv, q_weight, k_weight, inv_freq, positions, token_seq, block_table,
@@ -191,7 +204,7 @@ def sample_rows(logits, temperatures, seeds, draw_index, tokens, status):
         tokens[r] = min(pick, logits.shape[1] - 1)
 
 
-NAMES = ("embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear",
+NAMES = ("embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_swiglu", "gemm_skinny",
          "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_rows")
 
 

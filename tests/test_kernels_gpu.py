@@ -333,3 +333,50 @@ def test_kernels_refuse_what_they_cannot_do(ops):
                             torch.tensor([1], dtype=torch.int32, device=DEV),
                             torch.zeros(1, 1, dtype=torch.int32, device=DEV), num_seqs=1, max_q_len=1,
                             q_heads=1, kv_heads=1, head_dim=40, scale=1.0)
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,k", [(64, 8), (200, 200), (1003, 328), (2560, 2560), (330, 9728), (6144, 264)])
+def test_gemm_skinny_store(ops, m, n, k):
+    g = torch.Generator().manual_seed(20)
+    x = rand(g, m, k, dtype=torch.bfloat16)
+    w = rand(g, n, k, dtype=torch.bfloat16, scale=0.05)
+    want = x.float() @ w.float().T
+    got32 = ops.gemm_skinny(x.to(DEV), w.to(DEV), "f32").cpu()
+    bound = 2e-6 * float(want.abs().max()) * math.sqrt(k) + 1e-6
+    assert float((got32 - want).abs().max()) <= bound
+    got16 = ops.gemm_skinny(x.to(DEV), w.to(DEV), "bf16").cpu()
+    torch.testing.assert_close(got16.float(), want, atol=1e-2 * float(want.abs().max()), rtol=1e-2)
+    # the same call again gives the same bits; a row does not depend on the rows beside it
+    assert torch.equal(ops.gemm_skinny(x.to(DEV), w.to(DEV), "f32").cpu(), got32)
+    alone = ops.gemm_skinny(x[:1].contiguous().to(DEV), w.to(DEV), "f32").cpu()
+    if m <= 16:       # up to 16 rows share one kernel shape: bit-equal; beyond, equal up to the order of the sums
+        assert torch.equal(alone[0], got32[0])
+    assert float((alone[0] - got32[0]).abs().max()) <= bound
+
+
+@pytest.mark.parametrize("m", [1, 8, 40, 64])
+@pytest.mark.parametrize("inter,k", [(64, 64), (328, 200), (9728, 2560), (100, 1024)])
+def test_gemm_skinny_swiglu(ops, m, inter, k):
+    g = torch.Generator().manual_seed(21)
+    x = rand(g, m, k, dtype=torch.bfloat16)
+    w = rand(g, 2 * inter, k, dtype=torch.bfloat16, scale=0.05)
+    want = refs.linear_swiglu(x, w).float()
+    got = ops.gemm_skinny(x.to(DEV), w.to(DEV), "swiglu").cpu().float()
+    torch.testing.assert_close(got, want, atol=1e-2 * float(want.abs().max()) + 1e-6, rtol=1e-2)
+    assert torch.equal(ops.linear_swiglu(x.to(DEV), w.to(DEV)).cpu().float(), got)
+
+
+def test_linear_routes_by_rows_and_dtype(ops):
+    g = torch.Generator().manual_seed(22)
+    w = rand(g, 136, 200, dtype=torch.bfloat16, scale=0.05)
+    for rows in (3, 64, 65, 300):     # up to 64 rows: the streaming kernel; beyond: the matrix library
+        x = rand(g, rows, 200, dtype=torch.bfloat16)
+        want = x.float() @ w.float().T
+        got = ops.linear(x.to(DEV), w.to(DEV), out_dtype=torch.float32).cpu()
+        torch.testing.assert_close(got, want, atol=1e-3, rtol=1e-3)
+        assert ops.linear(x.to(DEV), w.to(DEV)).dtype == torch.bfloat16
+    # a weight stored in 32-bit stays in 32-bit: the activation is widened
+    got = ops.linear(x.to(DEV), w.float().to(DEV)).cpu()
+    assert got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), want, atol=2e-2, rtol=2e-2)
