@@ -26,6 +26,7 @@ class StepBatch:
     num_wanted: int
     max_q_len: int
     max_ctx: int
+    num_decode: int         # sequences that bring exactly one token
     token_ids: Tensor       # int32 [T]
     positions: Tensor       # int32 [T]   absolute position of each token in its request
     token_seq: Tensor       # int32 [T]   index of the token's request within the batch
@@ -82,7 +83,7 @@ def build_batch(entries, lengths_before, state_slots, tables_per_group, device) 
         offset += num_seqs * width
     return StepBatch(
         num_tokens=total, num_seqs=num_seqs, num_wanted=len(want_rows), max_q_len=max(q_lens),
-        max_ctx=max(ctx_len), token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
+        max_ctx=max(ctx_len), num_decode=sum(1 for n in q_lens if n == 1), token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
         ctx_len=views[4], ctx_before=views[5], state_slots=views[6], want_rows=views[7],
         block_tables=block_tables, request_ids=[e.request_id for e in entries], q_lens=q_lens,
         ctx_before_host=list(lengths_before))

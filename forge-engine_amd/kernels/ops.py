@@ -280,15 +280,35 @@ def qk_norm_rope_write(qkv: Tensor, q_weight: Tensor | None, k_weight: Tensor | 
           c_int(block_size), c_int(num_blocks), c_float(eps), c_int(1 if write_kv else 0), _stream())
 
 
+DECODE_TARGET_BLOCKS = 512   # blocks the decode attention kernel aims at (key splits fill the chip)
+
+
+def _decode_kernel_fits(q: Tensor, head_dim: int, groups: int, block_size: int) -> bool:
+    return (q.dtype == torch.bfloat16 and head_dim in (64, 128, 256) and groups <= 8
+            and block_size % 16 == 0)
+
+
+def decode_splits(num_decode: int, kv_heads: int, max_ctx: int) -> int:
+    """Key splits per (sequence, kv head) for the decode kernel: enough blocks to
+    fill the chip, at least four 16-key tiles (one per wave) in each."""
+    want = -(-DECODE_TARGET_BLOCKS // max(1, num_decode * kv_heads))
+    most = max(1, -(-max_ctx // 16) // 4)
+    return max(1, min(want, most, 64))
+
+
 def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tensor, cu_q: Tensor,
                     ctx_len: Tensor, block_table: Tensor, *, num_seqs: int, max_q_len: int,
                     q_heads: int, kv_heads: int, head_dim: int, scale: float,
-                    window: int | None = None) -> Tensor:
+                    window: int | None = None, num_decode: int | None = None,
+                    max_ctx: int | None = None, splits: int | None = None) -> Tensor:
     """Attention of every query token of a mixed batch over its paged keys.
 
     q: [T, >= Hq*D] (row stride may exceed Hq*D: the q part of a fused qkv
     buffer); out [T, Hq*D]; cu_q int32 [B+1]; ctx_len int32 [B] (keys after the
     step, the step's own included); block_table int32 [B, max_blocks].
+    ``num_decode`` (how many sequences bring exactly one token) and ``max_ctx``
+    are host-side hints: with them, single-token sequences of a bfloat16 cache
+    go to the streaming decode kernel and the others to the general kernel.
     """
     _gpu(q, "q", contiguous=False)
     _gpu(out, "out", q.dtype)
@@ -312,16 +332,36 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
         raise KernelError("key and value pages must have one shape")
     if cu_q.numel() != num_seqs + 1 or ctx_len.numel() != num_seqs or block_table.shape[0] < num_seqs:
         raise KernelError("cu_q, ctx_len and block_table do not match the number of sequences")
-    if q.data_ptr() % 16 or (q.stride(0) if tokens > 1 else 0) % 4:
+    if block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
+    if q.data_ptr() % 16 or (q.stride(0) if tokens > 1 else 0) % 8:
         raise KernelError("q rows must be 16-byte aligned")
     num_blocks, _, block_size, _ = key_pages.shape
+    groups = q_heads // kv_heads
     q_stride = q.stride(0) if tokens > 1 else q.shape[1]
+    if num_decode is None:
+        num_decode = num_seqs if max_q_len == 1 else 0
+    use_decode = num_decode > 0 and _decode_kernel_fits(q, head_dim, groups, block_size)
+    if use_decode:
+        if splits is None:
+            splits = decode_splits(num_decode, kv_heads, max_ctx if max_ctx is not None else 16 * 4 * 8)
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = torch.empty(num_seqs * kv_heads * splits * groups * head_dim, dtype=torch.float32, device=q.device)
+            part_ml = torch.empty(num_seqs * kv_heads * splits * groups * 2, dtype=torch.float32, device=q.device)
+        _call("attention_decode", "fe_paged_attention_decode", _ptr(q), c_longlong(q_stride),
+              _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(part_o),
+              _ptr(part_ml), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)),
+              c_int(num_seqs), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
+              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(splits), _stream())
+        if num_decode == num_seqs:
+            return out
     _call("attention_generic", "fe_paged_attention_generic", _ptr(q), c_longlong(q_stride),
           _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)),
           c_int(_code(q.dtype)), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table),
           c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(kv_heads),
-          c_int(q_heads // kv_heads), c_int(head_dim), c_int(block_size), c_int(num_blocks),
-          c_int(window or 0), c_float(scale), _stream())
+          c_int(groups), c_int(head_dim), c_int(block_size), c_int(num_blocks),
+          c_int(window or 0), c_float(scale), c_int(2 if use_decode else 1), _stream())
     return out
 
 
@@ -359,4 +399,4 @@ def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index:
           _stream())
 
 
-LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "qk_rope", "attention_generic", "sample")
+LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "qk_rope", "attention_generic", "attention_decode", "sample")

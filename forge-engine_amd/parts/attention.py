@@ -129,11 +129,12 @@ class GroupedQueryAttention(Mixer):
         ops.paged_attention(
             qkv, cache.key_pages, cache.value_pages, attn, batch.cu_q, batch.ctx_len, cache.block_table,
             num_seqs=batch.num_seqs, max_q_len=batch.max_q_len, q_heads=self.num_heads,
-            kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window)
+            kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
+            num_decode=batch.num_decode, max_ctx=batch.max_ctx)
         return ops.linear(attn, self.o_weight, self.o_bias, out_dtype=torch.float32)   # float32 update for the residual sum
 
     def kernel_libraries(self):
-        return {"qk_rope", "attention_generic", "gemm_f32", "gemm_skinny"}
+        return {"qk_rope", "attention_generic", "attention_decode", "gemm_f32", "gemm_skinny"}
 
 
 register_part("mixer", "gqa_attention", GroupedQueryAttention)

@@ -380,3 +380,57 @@ def test_linear_routes_by_rows_and_dtype(ops):
     got = ops.linear(x.to(DEV), w.float().to(DEV)).cpu()
     assert got.dtype == torch.bfloat16
     torch.testing.assert_close(got.float(), want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("splits", [1, 3, 8])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [
+    (32, 8, 128, 16), (5, 5, 64, 16), (10, 2, 128, 32), (8, 1, 256, 16), (6, 3, 64, 64), (16, 2, 128, 16),
+])
+def test_decode_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size, splits):
+    """The streaming decode kernel (single-token sequences of a bfloat16 cache) with key splits;
+    sequences with more tokens in the same batch go to the general kernel."""
+    g = torch.Generator().manual_seed(30)
+    seqs = [(0, 1), (14, 1), (15, 1), (16, 1), (699, 1), (40, 6), (255, 1), (3, 1)]
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                extra_width=2 * kv_heads * head_dim)
+    kw = dict(num_seqs=len(seqs), max_q_len=6, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+              scale=head_dim ** -0.5)
+    want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype), cu, ctx, table, **kw).float()
+    got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV),
+                              torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
+                              cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=7, max_ctx=700, splits=splits, **kw).cpu().float()
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("window", [1, 16, 37, 300])
+def test_decode_attention_kernel_window(ops, window):
+    g = torch.Generator().manual_seed(31)
+    seqs = [(0, 1), (36, 1), (37, 1), (500, 1)]
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, 8, 2, 128, 16)
+    kw = dict(num_seqs=4, max_q_len=1, q_heads=8, kv_heads=2, head_dim=128, scale=128 ** -0.5, window=window)
+    want = refs.paged_attention(q, kp, vp, torch.empty(4, 1024, dtype=q.dtype), cu, ctx, table, **kw).float()
+    for splits in (1, 4):
+        got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), torch.empty(4, 1024, dtype=q.dtype, device=DEV),
+                                  cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=4, max_ctx=501, splits=splits, **kw).cpu().float()
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
+def test_decode_attention_far_key_and_page_edges(ops):
+    """One key far back, and keys at the first and last slot of a page, each made to stand out in turn."""
+    g = torch.Generator().manual_seed(32)
+    head_dim, block_size, ctx_len = 128, 16, 1000
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, [(ctx_len - 1, 1)], 4, 1, head_dim, block_size)
+    q = (q.float() * 0.01).to(torch.bfloat16)
+    for far in (0, 15, 16, 37, 511, 512, 991, 999):
+        kq, qq = kp.clone(), q.clone()
+        page, slot = int(table[0, far // block_size]), far % block_size
+        kq[page, 0, slot] = 0.0
+        kq[page, 0, slot, 5] = 30.0
+        for h in range(4):
+            qq[0, h * head_dim + 5] = 30.0
+        for splits in (1, 5):
+            got = ops.paged_attention(qq.to(DEV), kq.to(DEV), vp.to(DEV), torch.empty(1, 4 * head_dim, dtype=q.dtype, device=DEV),
+                                      cu.to(DEV), ctx.to(DEV), table.to(DEV), num_seqs=1, max_q_len=1, q_heads=4, kv_heads=1,
+                                      head_dim=head_dim, scale=head_dim ** -0.5, num_decode=1, max_ctx=ctx_len, splits=splits).cpu().float()
+            for h in range(4):
+                torch.testing.assert_close(got[0, h * head_dim:(h + 1) * head_dim], vp[page, 0, slot].float(), atol=2e-2, rtol=2e-2)
