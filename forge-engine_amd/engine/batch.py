@@ -39,12 +39,20 @@ class StepBatch:
     request_ids: list       # host copies, for parts that decide on the host
     q_lens: list
     ctx_before_host: list
+    state_slots_host: list
 
 
-def build_batch(entries, lengths_before, state_slots, tables_per_group, device) -> StepBatch:
+def build_batch(entries, lengths_before, state_slots, tables_per_group, device, *, widths=None,
+                static=None, max_ctx=None) -> StepBatch:
     """Pack the step's metadata into one int32 buffer and copy it to the
     device in one transfer.  ``tables_per_group[g][i]`` is request i's page
-    list in cache group g."""
+    list in cache group g.
+
+    ``widths`` fixes the block tables' widths (else: the longest table);
+    ``static`` = (pinned host buffer, device buffer) makes the batch live at
+    fixed addresses, refilled in place, which is what a captured graph reads;
+    ``max_ctx`` overrides the host-side context bound (a graph is captured for
+    a bound, not for one step's lengths)."""
     num_seqs = len(entries)
     q_lens = [len(e.tokens) for e in entries]
     total = sum(q_lens)
@@ -58,18 +66,28 @@ def build_batch(entries, lengths_before, state_slots, tables_per_group, device) 
         want_rows.extend(cu_q[-1] + w for w in entry.want)
         cu_q.append(cu_q[-1] + q_lens[i])
     ctx_len = [lengths_before[i] + q_lens[i] for i in range(num_seqs)]
-    widths = [max(1, max((len(t) for t in tables), default=1)) for tables in tables_per_group]
+    if widths is None:
+        widths = [max(1, max((len(t) for t in tables), default=1)) for tables in tables_per_group]
     flat_tables = []
     for tables, width in zip(tables_per_group, widths):
         for table in tables:
+            if len(table) > width:
+                raise ValueError(f"a block table of {len(table)} pages does not fit the width {width}")
             flat_tables.extend(table)
             flat_tables.extend([-1] * (width - len(table)))
     sections = [token_ids, positions, token_seq, cu_q, ctx_len, list(lengths_before), list(state_slots),
                 want_rows, flat_tables]
     host = torch.tensor([v for section in sections for v in section], dtype=torch.int32)
-    if device.type == "cuda":
-        host = host.pin_memory()
-    flat = host.to(device, non_blocking=True)
+    if static is not None:
+        host_static, flat = static
+        if host.numel() > flat.numel():
+            raise ValueError("the step does not fit its static buffer")
+        host_static[:host.numel()].copy_(host)
+        flat[:host.numel()].copy_(host_static[:host.numel()], non_blocking=True)
+    else:
+        if device.type == "cuda":
+            host = host.pin_memory()
+        flat = host.to(device, non_blocking=True)
     views = []
     offset = 0
     for section in sections:
@@ -83,7 +101,13 @@ def build_batch(entries, lengths_before, state_slots, tables_per_group, device) 
         offset += num_seqs * width
     return StepBatch(
         num_tokens=total, num_seqs=num_seqs, num_wanted=len(want_rows), max_q_len=max(q_lens),
-        max_ctx=max(ctx_len), num_decode=sum(1 for n in q_lens if n == 1), token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
-        ctx_len=views[4], ctx_before=views[5], state_slots=views[6], want_rows=views[7],
-        block_tables=block_tables, request_ids=[e.request_id for e in entries], q_lens=q_lens,
-        ctx_before_host=list(lengths_before))
+        max_ctx=max(ctx_len) if max_ctx is None else max_ctx,
+        num_decode=sum(1 for n in q_lens if n == 1), token_ids=views[0], positions=views[1],
+        token_seq=views[2], cu_q=views[3], ctx_len=views[4], ctx_before=views[5], state_slots=views[6],
+        want_rows=views[7], block_tables=block_tables, request_ids=[e.request_id for e in entries],
+        q_lens=q_lens, ctx_before_host=list(lengths_before), state_slots_host=list(state_slots))
+
+
+def static_batch_size(num_seqs: int, widths) -> int:
+    """int32 entries of a single-token batch of ``num_seqs`` requests."""
+    return 8 * num_seqs + 1 + num_seqs * sum(widths)

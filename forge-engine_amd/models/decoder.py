@@ -69,6 +69,11 @@ class DecoderModel:
         for part in self.parts():
             part.finalize()
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model may be captured and replayed."""
+        return all(part.graph_safe for part in self.parts())
+
     def kernel_libraries(self) -> set[str]:
         names: set[str] = set()
         for part in self.parts():

@@ -68,6 +68,9 @@ class Residual:
 
 class Part:
     role = ""
+    # False for a part whose forward decides anything on the host from the step's
+    # contents (lengths, slots): its steps are not replayed from a captured graph.
+    graph_safe = True
 
     def __init__(self, ctx: BuildContext, prefix: str = "") -> None:
         self.ctx = ctx

@@ -1,0 +1,473 @@
+"""The engine on the GPU: generation through the entry points, long decoding
+through captured graphs, the first tokens of a sequence, each part alone, and a
+toy architecture (a mixer with state of its own, a windowed mixer, a layer run
+twice, a layer reading another's cache) registered from here."""
+
+from __future__ import annotations
+
+import json
+from dataclasses import dataclass
+from typing import ClassVar
+
+import pytest
+import torch
+from safetensors.torch import load_file
+
+import plain_qwen3 as plain
+import replay_util as ru
+from conftest import BLOCK_SIZE, TINY
+from forge_engine_amd.cache import CacheNeeds, FixedState
+from forge_engine_amd.config import EngineConfig, SchedulerConfig, load_model_config
+from forge_engine_amd.config.model import KeyReader, ModelConfig
+from forge_engine_amd.engine import (GenerationEngine, ModelRunner, StepEntry, build_model,
+                                     engine_from_folder, load_model)
+from forge_engine_amd.parts import (BuildContext, LayerCall, LayerSpec, Mixer, ModelPlan, ParamSpec, PartSpec,
+                                    Residual, build_part)
+from forge_engine_amd.registry import register_architecture, register_part
+from forge_engine_amd.sampling import SamplingParams
+from forge_engine_amd.weights import fill_random_weights, write_random_model
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    made = {}
+    for name in TINY:
+        folder = tmp_path_factory.mktemp(f"engine_{name}")
+        write_random_model(load_model_config(TINY[name]), 31, folder)
+        made[name] = folder
+    return made
+
+
+def folder_weights(folder):
+    return {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
+
+
+def check_choice(weights, config, prompt, tokens, dtype):
+    """Each generated token must be the plain implementation's argmax, or (bfloat16)
+    within the rounding bound of it."""
+    ids = list(prompt)
+    for token in tokens:
+        logits = plain.forward(weights, config, ids)[-1]
+        if dtype == "float32":
+            assert token == int(logits.argmax()), f"token {token} after {len(ids)} ids"
+        else:
+            assert float(logits.max() - logits[token]) <= ru.BF16_FRACTION * float(logits.abs().max())
+        ids.append(token)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_greedy_generation_through_the_entry_point(name, dtype, folders):
+    config, weights = TINY[name], folder_weights(folders[name])
+    prompts = list(ru.make_requests(config, 8, (5, 11, 17)).values())
+    scheduler = SchedulerConfig(block_size=BLOCK_SIZE[name], block_capacity=64, token_budget=16, max_batch_size=4)
+    engine = engine_from_folder(folders[name], engine_config=EngineConfig(max_new_tokens=8),
+                                scheduler_config=scheduler, dtype=dtype)
+    outputs = engine.generate(prompts)
+    assert engine.cache_pool.allocated_pages == 0
+    for prompt, tokens in zip(prompts, outputs):
+        assert len(tokens) == 8
+        check_choice(weights, config, prompt, tokens, dtype)
+    single = GenerationEngine(engine)
+    assert single.generate(prompts[0]) == outputs[0]          # alone or batched: the same tokens
+    assert list(single.stream(prompts[1])) == outputs[1]
+
+
+def test_command_line_generates(folders, capsys):
+    from forge_engine_amd.cli import main
+    prompt = [5, 17, 3, 200, 9]
+    code = main(["generate", "--model", str(folders["A"]), "--dtype", "float32", "--prompt-ids",
+                 ",".join(map(str, prompt)), "--prompt-ids", "7,7", "--max-new-tokens", "5", "--block-size", "4"])
+    assert code == 0
+    records = [json.loads(line) for line in capsys.readouterr().out.strip().splitlines()]
+    assert [r["prompt"] for r in records] == [0, 1] and all(r["finish_reason"] == "length" for r in records)
+    check_choice(folder_weights(folders["A"]), TINY["A"], prompt, records[0]["token_ids"], "float32")
+
+
+def test_temperature_sampling_is_seeded_and_batch_independent(folders):
+    scheduler = SchedulerConfig(block_size=8, block_capacity=64)
+    engine = engine_from_folder(folders["B"], scheduler_config=scheduler, dtype="float32")
+    params = SamplingParams(temperature=0.8, seed=1234, max_new_tokens=12)
+    prompts = list(ru.make_requests(TINY["B"], 2, (1, 7, 23, 40)).values())
+    together = engine.generate(prompts, params)
+    alone = [engine.generate([p], params)[0] for p in prompts]
+    assert together == alone
+    assert engine.generate(prompts[:1], SamplingParams(temperature=0.8, seed=99, max_new_tokens=12))[0] != alone[0]
+    top = engine.generate(prompts[:2], SamplingParams(temperature=0.9, top_k=3, top_p=0.9, min_p=0.05, seed=5, max_new_tokens=6))
+    assert all(len(t) == 6 for t in top)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_through_graphs_matches_eager_and_plain(dtype, folders):
+    """300 decode steps: replays of captured graphs, with eager steps of another
+    request between them, against the eager engine and the plain implementation."""
+    name = "C"
+    config, weights = TINY[name], folder_weights(folders[name])
+    tokens = ru.make_requests(config, 13, (340,))["r0"]
+    other = ru.make_requests(config, 14, (90,))["r0"]
+    _, model = load_model(folders[name], dtype=dtype, device=DEV)
+    runs = {}
+    for graphs in (True, False):
+        runner = ModelRunner(model, block_size=16, block_capacity=40, num_state_slots=4, use_graphs=graphs)
+        runner.begin("a")
+        runner.begin("b")
+        rows = [runner.step([StepEntry("a", tokens[:40], [39])])[0].clone()]
+        fed_other = 0
+        for i in range(40, 340):
+            rows.append(runner.step([StepEntry("a", [tokens[i]], [0])])[0].clone())
+            if i % 25 == 0 and fed_other < len(other):      # eager work between the replays
+                runner.step([StepEntry("b", other[fed_other:fed_other + 9], [])])
+                fed_other += 9
+        runs[graphs] = torch.stack(rows).cpu()
+        assert (runner.graph_replays > 250) == graphs
+        runner.end("a")
+        runner.end("b")
+        assert runner.cache.allocated_pages == 0
+    want = plain.forward(weights, config, tokens)[39:]
+    scale = float(want.abs().max())
+    bound = 1e-4 * scale if dtype == "float32" else ru.BF16_FRACTION * scale
+    assert float((runs[True] - want).abs().max()) <= bound
+    assert float((runs[False] - want).abs().max()) <= bound
+    assert torch.isfinite(runs[True]).all()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens_of_a_sequence(name, dtype, folders):
+    """Position 0 alone, then 1, 2, 3: the shortest contexts, one page, first slots."""
+    config = TINY[name]
+    requests = ru.make_requests(config, 17, (1, 2, 4))
+    trace = ru.TraceBuilder()
+    trace.step([(k, v[:1]) for k, v in requests.items()])
+    trace.step([(k, v[1:2]) for k, v in requests.items() if len(v) > 1], end=["r0"])
+    trace.step([("r2", requests["r2"][2:4])], end=["r1", "r2"])
+    import tempfile
+    with tempfile.TemporaryDirectory() as out:
+        got = ru.run_trace(folders[name], dtype, trace, out, block_size=BLOCK_SIZE[name])
+    ru.compare(got, ru.plain_logits(folders[name], requests), dtype)
+
+
+# ---------------------------------------------------------------- parts alone
+
+def ctx(dtype=torch.float32):
+    return BuildContext(DEV, dtype)
+
+
+def randn(*shape, scale=1.0, seed=0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def test_norm_part_alone():
+    part = build_part("norm", PartSpec("rms_norm", {"size": 72, "eps": 1e-5}, "n"), ctx())
+    assert list(part.param_specs()) == ["n.weight"]
+    w = 1 + randn(72, scale=0.1)
+    part.set_param("n.weight", w.to(DEV))
+    h, update = randn(5, 72, seed=1), randn(5, 72, seed=2)
+    residual = Residual(h.to(DEV).clone())
+    residual.add(update.to(DEV))
+    got = part.forward(residual)
+    torch.testing.assert_close(got.cpu(), plain.rms_norm(h + update, w, 1e-5), atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(residual.h.cpu(), h + update)        # the add happened in the stream
+    assert residual.pending is None
+    rows = torch.tensor([4, 0], dtype=torch.int32, device=DEV)
+    torch.testing.assert_close(part.forward(residual, rows=rows).cpu(), plain.rms_norm((h + update)[[4, 0]], w, 1e-5),
+                               atol=1e-5, rtol=1e-5)
+
+
+def test_position_part_alone():
+    part = build_part("position", PartSpec("rotary", {"head_dim": 48, "theta": 1e6}), ctx())
+    inv_freq, rotary_dim = part.rotary()
+    assert rotary_dim == 48
+    want = 1.0 / (1e6 ** (torch.arange(0, 48, 2, dtype=torch.float32) / 48))
+    assert torch.equal(inv_freq.cpu(), want)                         # bit-equal to the reference's expression
+    partial = build_part("position", PartSpec("rotary", {"head_dim": 48, "theta": 1e4, "rotary_dim": 16}), ctx())
+    assert partial.rotary()[0].shape == (8,) and partial.rotary()[1] == 16
+    assert build_part("position", PartSpec("none"), ctx()).rotary() is None
+
+
+def test_feed_forward_part_alone():
+    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 2e-2)):
+        part = build_part("feed_forward", PartSpec("swiglu", {"hidden_size": 40, "intermediate_size": 104}, "m"), ctx(dtype))
+        weights = {"m.gate_proj.weight": randn(104, 40, scale=0.2, seed=3), "m.up_proj.weight": randn(104, 40, scale=0.2, seed=4),
+                   "m.down_proj.weight": randn(40, 104, scale=0.2, seed=5)}
+        weights = {k: v.to(dtype) for k, v in weights.items()}
+        for k, v in weights.items():
+            part.set_param(k, v.to(DEV))
+        x = randn(70, 40, seed=6).to(dtype)          # more than 64 rows: the library product; fewer: the streaming one
+        want = plain.swiglu_mlp(x.float(), {k: v.float() for k, v in weights.items()}, "m")
+        bound = tol * float(want.abs().max())     # the activation between the two products is rounded to bfloat16
+        for rows in (70, 9):
+            got = part.forward(x[:rows].to(DEV)).cpu()
+            assert got.dtype == torch.float32
+            assert float((got - want[:rows]).abs().max()) <= bound
+
+
+def test_embedding_and_head_parts_alone():
+    embedding = build_part("embedding", PartSpec("token_embedding", {"vocab_size": 50, "hidden_size": 24}, "e"), ctx())
+    table = randn(50, 24, seed=7)
+    embedding.set_param("e.weight", table.to(DEV))
+    tied = build_part("head", PartSpec("lm_head", {"vocab_size": 50, "hidden_size": 24, "tied": True}, "h"), ctx())
+    tied.tie(embedding)
+    assert tied.param_specs() == {}
+    z = randn(3, 24, seed=8)
+    torch.testing.assert_close(tied.forward(z.to(DEV)).cpu(), z @ table.T, atol=1e-5, rtol=1e-5)
+    untied = build_part("head", PartSpec("lm_head", {"vocab_size": 50, "hidden_size": 24}, "h"), ctx())
+    matrix = randn(50, 24, seed=9)
+    untied.set_param("h.weight", matrix.to(DEV))
+    torch.testing.assert_close(untied.forward(z.to(DEV)).cpu(), z @ matrix.T, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_mixer_and_block_alone(dtype):
+    """One pre-norm block built from specs, stepped over a paged cache in two portions and a
+    decode token, against the plain layer on the whole sequence."""
+    hidden, heads, kv_heads, head_dim, inter, eps, theta = 48, 3, 1, 16, 80, 1e-5, 1e4
+    plan_config = {"num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": head_dim,
+                   "rms_norm_eps": eps, "rope_theta": theta}
+    spec = LayerSpec(
+        "pre_norm",
+        PartSpec("gqa_attention", {"hidden_size": hidden, "num_heads": heads, "num_kv_heads": kv_heads, "head_dim": head_dim,
+                                   "qk_norm_eps": eps, "position": PartSpec("rotary", {"head_dim": head_dim, "theta": theta})},
+                 "model.layers.0.self_attn"),
+        PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": inter}, "model.layers.0.mlp"),
+        {"input": PartSpec("rms_norm", {"size": hidden, "eps": eps}, "model.layers.0.input_layernorm"),
+         "post_mixer": PartSpec("rms_norm", {"size": hidden, "eps": eps}, "model.layers.0.post_attention_layernorm")})
+    plan = ModelPlan(hidden, 30, PartSpec("token_embedding", {"vocab_size": 30, "hidden_size": hidden}, "model.embed_tokens"),
+                     (spec,), (LayerCall(0),), PartSpec("rms_norm", {"size": hidden, "eps": eps}, "model.norm"),
+                     PartSpec("lm_head", {"vocab_size": 30, "hidden_size": hidden, "tied": True}, "lm_head"))
+    from forge_engine_amd.models import DecoderModel
+    model = DecoderModel(plan, ctx(dtype))
+    fill_random_weights(model, 3, device=DEV, dtype=dtype)
+    block = model.layers[0]
+    weights = {}
+    for module, part in block.mixer.split_qkv_weight().items():
+        weights[f"model.layers.0.self_attn.{module}.weight"] = part.float().cpu()
+    weights["model.layers.0.self_attn.o_proj.weight"] = block.mixer.o_weight.float().cpu()
+    weights["model.layers.0.self_attn.q_norm.weight"] = block.mixer.q_norm.cpu()
+    weights["model.layers.0.self_attn.k_norm.weight"] = block.mixer.k_norm.cpu()
+    weights["model.layers.0.mlp.gate_proj.weight"] = block.feed_forward.gate_up_weight[:inter].float().cpu()
+    weights["model.layers.0.mlp.up_proj.weight"] = block.feed_forward.gate_up_weight[inter:].float().cpu()
+    weights["model.layers.0.mlp.down_proj.weight"] = block.feed_forward.down_weight.float().cpu()
+    weights["model.layers.0.input_layernorm.weight"] = block.norms["input"].weight.cpu()
+    weights["model.layers.0.post_attention_layernorm.weight"] = block.norms["post_mixer"].weight.cpu()
+    h = randn(12, hidden, seed=11)
+    want = plain.decoder_layer(h, weights, 0, plan_config, torch.arange(12))
+    runner = ModelRunner(model, block_size=4, block_capacity=8, num_state_slots=1, use_graphs=False)
+    runner.begin("s")
+    got = []
+    for start, stop in ((0, 7), (7, 11), (11, 12)):
+        batch = runner.prepare([StepEntry("s", [0] * (stop - start), [])])
+        residual = Residual(h[start:stop].to(DEV).clone())
+        block.forward(residual, batch, runner.cache_views(batch)[0])
+        got.append(residual.flush().cpu())
+        runner.cache.commit("s", stop)
+    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    torch.testing.assert_close(torch.cat(got), want, atol=tol, rtol=tol)
+
+
+# ------------------------------------------------- a toy architecture, defined here
+
+class EmaMixer(Mixer):
+    """A toy mixer with state of its own: s_t = decay * s_{t-1} + x_t (per
+    request, reset at its first token), update = W s_t.  Plain torch ops: it is
+    test code, not a kernel."""
+
+    graph_safe = False      # it loops over the step's requests on the host
+
+    def __init__(self, ctx, prefix, *, hidden_size: int, decay: float) -> None:
+        super().__init__(ctx, prefix)
+        self.hidden_size, self.decay = hidden_size, decay
+        self.weight = None
+
+    def param_specs(self):
+        return {self.name("mix.weight"): ParamSpec((self.hidden_size, self.hidden_size))}
+
+    def set_param(self, name, tensor):
+        self.weight = tensor
+
+    def cache_needs(self):
+        return CacheNeeds(state=FixedState((self.hidden_size,), torch.float32))
+
+    def forward(self, x, batch, cache, writes_cache=True):
+        out = torch.empty((x.shape[0], self.hidden_size), dtype=torch.float32, device=x.device)
+        slots = batch.state_slots_host
+        at = 0
+        for i, count in enumerate(batch.q_lens):
+            state = cache.state[slots[i]]
+            if batch.ctx_before_host[i] == 0:
+                state.zero_()                      # a slot is reused: a request's first portion starts from zero
+            for t in range(at, at + count):
+                state.mul_(self.decay).add_(x[t].float())
+                out[t] = self.weight.float() @ state
+            at += count
+        return out
+
+
+@dataclass(frozen=True)
+class ToyConfig(ModelConfig):
+    vocab_size: int
+    hidden_size: int
+    intermediate_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    window: int
+    decay: float
+    rms_norm_eps: float
+    rope_theta: float
+    architecture: ClassVar[str] = "ToyMixedLM"
+
+    @classmethod
+    def from_dict(cls, raw):
+        read = KeyReader(raw)
+        return cls(*(read.integer(k) for k in ("vocab_size", "hidden_size", "intermediate_size", "num_attention_heads",
+                                              "num_key_value_heads", "head_dim", "window")),
+                   read.number("decay"), read.number("rms_norm_eps"), read.number("rope_theta"))
+
+
+def toy_plan(config: ToyConfig) -> ModelPlan:
+    def norm(prefix):
+        return PartSpec("rms_norm", {"size": config.hidden_size, "eps": config.rms_norm_eps}, prefix)
+
+    def attention(prefix, window):
+        return PartSpec("gqa_attention", {
+            "hidden_size": config.hidden_size, "num_heads": config.num_attention_heads,
+            "num_kv_heads": config.num_key_value_heads, "head_dim": config.head_dim, "qk_norm_eps": config.rms_norm_eps,
+            "window": window, "position": PartSpec("rotary", {"head_dim": config.head_dim, "theta": config.rope_theta})}, prefix)
+
+    def layer(index, mixer):
+        prefix = f"model.layers.{index}"
+        return LayerSpec("pre_norm", mixer,
+                         PartSpec("swiglu", {"hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size}, f"{prefix}.mlp"),
+                         {"input": norm(f"{prefix}.input_layernorm"), "post_mixer": norm(f"{prefix}.post_attention_layernorm")})
+
+    layers = (layer(0, attention("model.layers.0.self_attn", None)),
+              layer(1, PartSpec("toy_ema", {"hidden_size": config.hidden_size, "decay": config.decay}, "model.layers.1.ema")),
+              layer(2, attention("model.layers.2.self_attn", config.window)))
+    # layer 0 runs twice (two caches of its own); the last call runs layer 0's weights
+    # over the cache that the first call wrote, writing nothing
+    schedule = (LayerCall(0), LayerCall(1), LayerCall(2), LayerCall(0), LayerCall(1), LayerCall(0, cache=0, writes_cache=False))
+    sizes = {"vocab_size": config.vocab_size, "hidden_size": config.hidden_size}
+    return ModelPlan(config.hidden_size, config.vocab_size, PartSpec("token_embedding", dict(sizes), "model.embed_tokens"),
+                     layers, schedule, norm("model.norm"), PartSpec("lm_head", dict(sizes, tied=True), "lm_head"))
+
+
+def toy_plain_forward(weights, config: ToyConfig, tokens):
+    """The toy model on one whole sequence with the plain implementation's functions."""
+    positions = torch.arange(len(tokens))
+    h = weights["model.embed_tokens.weight"][torch.tensor(tokens)]
+    eps = config.rms_norm_eps
+    kept = {}
+
+    def attention(x, prefix, window, reuse_kv=None):
+        heads, kv_heads, d = config.num_attention_heads, config.num_key_value_heads, config.head_dim
+        q = (x @ weights[f"{prefix}.q_proj.weight"].T).view(-1, heads, d)
+        q = plain.rms_norm(q, weights[f"{prefix}.q_norm.weight"], eps).transpose(0, 1)
+        cos, sin = plain.rotary_tables(positions, d, config.rope_theta)
+        q = plain.apply_rotary(q, cos, sin)
+        if reuse_kv is None:
+            k = (x @ weights[f"{prefix}.k_proj.weight"].T).view(-1, kv_heads, d)
+            k = plain.apply_rotary(plain.rms_norm(k, weights[f"{prefix}.k_norm.weight"], eps).transpose(0, 1), cos, sin)
+            v = (x @ weights[f"{prefix}.v_proj.weight"].T).view(-1, kv_heads, d).transpose(0, 1)
+        else:
+            k, v = reuse_kv
+        out = plain.causal_attention(q, k, v, d ** -0.5, window=window)
+        return out.transpose(0, 1).reshape(len(tokens), heads * d) @ weights[f"{prefix}.o_proj.weight"].T, (k, v)
+
+    def ema(x, prefix):
+        state = torch.zeros(config.hidden_size)
+        rows = []
+        for t in range(len(tokens)):
+            state = config.decay * state + x[t]
+            rows.append(weights[f"{prefix}.mix.weight"] @ state)
+        return torch.stack(rows)
+
+    for call, (index, mode) in enumerate([(0, "own"), (1, "ema"), (2, "window"), (0, "own"), (1, "ema"), (0, "shared")]):
+        prefix = f"model.layers.{index}"
+        x = plain.rms_norm(h, weights[f"{prefix}.input_layernorm.weight"], eps)
+        if mode == "ema":
+            update = ema(x, f"{prefix}.ema")
+        elif mode == "shared":
+            update, _ = attention(x, f"{prefix}.self_attn", None, reuse_kv=kept[0])
+        else:
+            update, kv = attention(x, f"{prefix}.self_attn", config.window if mode == "window" else None)
+            kept.setdefault(call, kv)
+        h, y = plain.add_rms_norm(h, update, weights[f"{prefix}.post_attention_layernorm.weight"], eps)
+        h = h + plain.swiglu_mlp(y, weights, f"{prefix}.mlp")
+    return plain.rms_norm(h, weights["model.norm.weight"], eps) @ weights["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_registered_from_a_test(dtype):
+    register_part("mixer", "toy_ema", EmaMixer, replace=True)
+    register_architecture("ToyMixedLM", ToyConfig, toy_plan, replace=True)
+    raw = {"architectures": ["ToyMixedLM"], "vocab_size": 90, "hidden_size": 40, "intermediate_size": 72,
+           "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16, "window": 6, "decay": 0.5,
+           "rms_norm_eps": 1e-5, "rope_theta": 1e4}
+    config = load_model_config(raw)
+    assert isinstance(config, ToyConfig)
+    model = build_model(config, dtype=dtype, device=DEV)
+    fill_random_weights(model, 7, device=DEV, dtype=model.ctx.dtype)
+    runner = ModelRunner(model, block_size=4, block_capacity=24, num_state_slots=2)
+    groups = runner.cache.groups
+    assert sorted((g.window or 0, len(g.slots)) for g in groups) == [(0, 2), (6, 1)]   # windowed pages apart from full ones
+    weights = {}
+    for name in model.param_specs():
+        owner = model._owners[name]
+        if hasattr(owner, "split_qkv_weight") and name.rsplit(".", 2)[-2] in ("q_proj", "k_proj", "v_proj"):
+            weights[name] = owner.split_qkv_weight()[name.rsplit(".", 2)[-2]].float().cpu()
+    for index in (0, 1, 2):
+        block = model.layers[index]
+        p = f"model.layers.{index}"
+        weights[f"{p}.input_layernorm.weight"] = block.norms["input"].weight.cpu()
+        weights[f"{p}.post_attention_layernorm.weight"] = block.norms["post_mixer"].weight.cpu()
+        inter = config.intermediate_size
+        weights[f"{p}.mlp.gate_proj.weight"] = block.feed_forward.gate_up_weight[:inter].float().cpu()
+        weights[f"{p}.mlp.up_proj.weight"] = block.feed_forward.gate_up_weight[inter:].float().cpu()
+        weights[f"{p}.mlp.down_proj.weight"] = block.feed_forward.down_weight.float().cpu()
+        if index == 1:
+            weights[f"{p}.ema.mix.weight"] = block.mixer.weight.float().cpu()
+        else:
+            weights[f"{p}.self_attn.o_proj.weight"] = block.mixer.o_weight.float().cpu()
+            weights[f"{p}.self_attn.q_norm.weight"] = block.mixer.q_norm.cpu()
+            weights[f"{p}.self_attn.k_norm.weight"] = block.mixer.k_norm.cpu()
+    weights["model.embed_tokens.weight"] = model.embedding.weight.float().cpu()
+    weights["model.norm.weight"] = model.final_norm.weight.cpu()
+
+    requests = ru.make_requests(raw, 3, (23, 9, 31, 14))
+    want = {k: toy_plain_forward(weights, config, v) for k, v in requests.items()}
+    # two requests at a time in two state slots: portions, then single tokens; the third and
+    # fourth request reuse the slots and pages of the first two
+    got = {k: [] for k in requests}
+    for pair in (("r0", "r1"), ("r2", "r3")):
+        at = {k: 0 for k in pair}
+        for k in pair:
+            runner.begin(k)
+        step = 0
+        while any(at[k] < len(requests[k]) for k in pair):
+            entries = []
+            for k in pair:
+                if at[k] >= len(requests[k]):
+                    continue
+                size = (5, 2, 3, 1, 1, 4)[(step + len(k)) % 6] if at[k] < len(requests[k]) - 6 else 1
+                size = min(size, len(requests[k]) - at[k])
+                entries.append(StepEntry(k, requests[k][at[k]:at[k] + size], list(range(size))))
+                at[k] += size
+            logits = runner.step(entries).cpu()
+            row = 0
+            for e in entries:
+                got[e.request_id].append(logits[row:row + len(e.tokens)])
+                row += len(e.tokens)
+            step += 1
+        for k in pair:
+            runner.end(k)
+        assert runner.cache.allocated_pages == 0
+        runner.cache.check_invariants()
+    for k in requests:
+        rows = torch.cat(got[k])
+        scale = float(want[k].abs().max())
+        bound = 1e-4 * scale + 1e-5 if dtype == "float32" else ru.BF16_FRACTION * scale
+        assert float((rows - want[k]).abs().max()) <= bound, k
