@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     const T* __restrict__ value_pages, T* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len,
     const int* __restrict__ block_table, int table_stride, int kv_heads, int groups, int head_dim,
-    int block_size, int num_blocks, int window, float scale, int min_q_len) {
+    int block_size, int num_blocks, int window, float scale, int min_q_len, int max_q_served) {
   constexpr int KPT = TK / 16;    // keys per thread in a tile
   constexpr int DPT = DMAX / 16;  // output dims per thread
   extern __shared__ float smem[];
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
   const int ctx_before = ctx - q_len;
   const int rows_total = q_len * groups;
   const int row0 = blockIdx.x * ROWS;
-  if (row0 >= rows_total || ctx_before < 0 || q_len < min_q_len) return;
+  if (row0 >= rows_total || ctx_before < 0 || q_len < min_q_len || q_len > max_q_served) return;
 
   const int tid = threadIdx.x;
   const int r = tid / 16;
@@ -190,7 +190,7 @@ static int launch_generic(const void* q, long long q_stride, const void* key_pag
                           void* out, long long out_stride, const int* cu_q, const int* ctx_len,
                           const int* block_table, int table_stride, int num_seqs, int max_q_len,
                           int kv_heads, int groups, int head_dim, int block_size, int num_blocks,
-                          int window, float scale, int min_q_len, hipStream_t stream) {
+                          int window, float scale, int min_q_len, int max_q_served, hipStream_t stream) {
   const long long tiles = ((long long)max_q_len * groups + ROWS - 1) / ROWS;
   if (tiles > 0x7fffffffLL || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
   const size_t smem = sizeof(float) * ((size_t)(ROWS + TK) * (head_dim + 1) + (size_t)TK * head_dim + ROWS * TK);
@@ -198,7 +198,7 @@ static int launch_generic(const void* q, long long q_stride, const void* key_pag
   paged_attention_generic_kernel<T, DMAX, TK, FAST_EXP><<<grid, 256, smem, stream>>>(
       (const T*)q, q_stride, (const T*)key_pages, (const T*)value_pages, (T*)out, out_stride, cu_q,
       ctx_len, block_table, table_stride, kv_heads, groups, head_dim, block_size, num_blocks, window,
-      scale, min_q_len);
+      scale, min_q_len, max_q_served);
   return fe_check_launch();
 }
 
@@ -207,12 +207,12 @@ static int dispatch_generic(const void* q, long long q_stride, const void* key_p
                             void* out, long long out_stride, const int* cu_q, const int* ctx_len,
                             const int* block_table, int table_stride, int num_seqs, int max_q_len,
                             int kv_heads, int groups, int head_dim, int block_size, int num_blocks,
-                            int window, float scale, int min_q_len, hipStream_t stream) {
+                            int window, float scale, int min_q_len, int max_q_served, hipStream_t stream) {
 #define FE_GO(DMAX, TK)                                                                              \
   return launch_generic<T, DMAX, TK, FAST_EXP>(q, q_stride, key_pages, value_pages, out, out_stride, \
                                                cu_q, ctx_len, block_table, table_stride, num_seqs,   \
                                                max_q_len, kv_heads, groups, head_dim, block_size,    \
-                                               num_blocks, window, scale, min_q_len, stream)
+                                               num_blocks, window, scale, min_q_len, max_q_served, stream)
   if (head_dim <= 32) FE_GO(32, 64);
   if (head_dim <= 64) FE_GO(64, 64);
   if (head_dim <= 128) FE_GO(128, 32);
@@ -224,25 +224,28 @@ static int dispatch_generic(const void* q, long long q_stride, const void* key_p
 // ([q_heads][D]) from the token's start; out likewise with out_stride.
 // cu_q: [num_seqs + 1] prefix sums of query lengths; ctx_len: [num_seqs] keys
 // in the cache after this step; block_table: [num_seqs, table_stride].
-// Sequences with fewer than min_q_len query tokens are skipped (another kernel serves them).
+// Sequences with fewer than min_q_len or more than max_q_served query tokens are skipped
+// (other kernels serve them).
 extern "C" int fe_paged_attention_generic(const void* q, long long q_stride, const void* key_pages,
                                           const void* value_pages, void* out, long long out_stride,
                                           int dtype, const int* cu_q, const int* ctx_len,
                                           const int* block_table, int table_stride, int num_seqs,
                                           int max_q_len, int kv_heads, int groups, int head_dim,
                                           int block_size, int num_blocks, int window, float scale,
-                                          int min_q_len, hipStream_t stream) {
+                                          int min_q_len, int max_q_served, hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len <= 0) return FE_OK;
+  if (max_q_served < max_q_len) max_q_len = max_q_served;   // the grid covers only what is served
+  if (max_q_len < min_q_len) return FE_OK;
   if (head_dim < 16 || head_dim > 256 || head_dim % 16) return FE_BAD_ARGUMENT;
   if (kv_heads <= 0 || groups <= 0 || block_size <= 0 || num_blocks <= 0 || table_stride <= 0) return FE_BAD_ARGUMENT;
   if (q_stride % 4 || out_stride < (long long)kv_heads * groups * head_dim) return FE_BAD_ARGUMENT;
   if (dtype == FE_F32)
     return dispatch_generic<float, false>(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len,
                                           block_table, table_stride, num_seqs, max_q_len, kv_heads, groups,
-                                          head_dim, block_size, num_blocks, window, scale, min_q_len, stream);
+                                          head_dim, block_size, num_blocks, window, scale, min_q_len, max_q_served, stream);
   if (dtype == FE_BF16)
     return dispatch_generic<bf16_t, true>(q, q_stride, key_pages, value_pages, out, out_stride, cu_q, ctx_len,
                                           block_table, table_stride, num_seqs, max_q_len, kv_heads, groups,
-                                          head_dim, block_size, num_blocks, window, scale, min_q_len, stream);
+                                          head_dim, block_size, num_blocks, window, scale, min_q_len, max_q_served, stream);
   return FE_BAD_ARGUMENT;
 }

@@ -339,10 +339,23 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
     num_blocks, _, block_size, _ = key_pages.shape
     groups = q_heads // kv_heads
     q_stride = q.stride(0) if tokens > 1 else q.shape[1]
-    if num_decode is None:
-        num_decode = num_seqs if max_q_len == 1 else 0
-    use_decode = num_decode > 0 and _decode_kernel_fits(q, head_dim, groups, block_size)
-    if use_decode:
+    if num_decode is None:   # unknown: single-token sequences may sit beside longer ones
+        any_single, any_longer, num_decode = True, max_q_len > 1, num_seqs
+    else:
+        any_single, any_longer = num_decode > 0, num_decode < num_seqs
+    bf16_pages = q.dtype == torch.bfloat16 and block_size % 16 == 0
+    fast_decode = bf16_pages and head_dim in (64, 128, 256) and groups <= 8
+    fast_prefill = bf16_pages and head_dim in (64, 128)
+
+    def general(min_q: int, max_q: int) -> None:
+        _call("attention_generic", "fe_paged_attention_generic", _ptr(q), c_longlong(q_stride),
+              _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)),
+              c_int(_code(q.dtype)), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table),
+              c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(kv_heads),
+              c_int(groups), c_int(head_dim), c_int(block_size), c_int(num_blocks),
+              c_int(window or 0), c_float(scale), c_int(min_q), c_int(max_q), _stream())
+
+    if any_single and fast_decode:
         if splits is None:
             splits = decode_splits(num_decode, kv_heads, max_ctx if max_ctx is not None else 16 * 4 * 8)
         part_o = part_ml = None
@@ -354,14 +367,17 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
               _ptr(part_ml), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)),
               c_int(num_seqs), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
               c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(splits), _stream())
-        if num_decode == num_seqs:
-            return out
-    _call("attention_generic", "fe_paged_attention_generic", _ptr(q), c_longlong(q_stride),
-          _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)),
-          c_int(_code(q.dtype)), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table),
-          c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(kv_heads),
-          c_int(groups), c_int(head_dim), c_int(block_size), c_int(num_blocks),
-          c_int(window or 0), c_float(scale), c_int(2 if use_decode else 1), _stream())
+    if any_longer and fast_prefill:
+        _call("attention_prefill", "fe_paged_attention_prefill", _ptr(q), c_longlong(q_stride),
+              _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
+              _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
+              c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
+              c_int(num_blocks), c_int(window or 0), c_float(scale), _stream())
+    # whatever the two fast kernels did not take goes to the general kernel
+    single_left = any_single and not fast_decode
+    longer_left = any_longer and not fast_prefill
+    if single_left or longer_left:
+        general(1 if single_left else 2, max_q_len if longer_left else 1)
     return out
 
 
@@ -399,4 +415,4 @@ def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index:
           _stream())
 
 
-LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "qk_rope", "attention_generic", "attention_decode", "sample")
+LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")

@@ -134,7 +134,7 @@ class GroupedQueryAttention(Mixer):
         return ops.linear(attn, self.o_weight, self.o_bias, out_dtype=torch.float32)   # float32 update for the residual sum
 
     def kernel_libraries(self):
-        return {"qk_rope", "attention_generic", "attention_decode", "gemm_f32", "gemm_skinny"}
+        return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny"}
 
 
 register_part("mixer", "gqa_attention", GroupedQueryAttention)

@@ -434,3 +434,66 @@ def test_decode_attention_far_key_and_page_edges(ops):
                                       head_dim=head_dim, scale=head_dim ** -0.5, num_decode=1, max_ctx=ctx_len, splits=splits).cpu().float()
             for h in range(4):
                 torch.testing.assert_close(got[0, h * head_dim:(h + 1) * head_dim], vp[page, 0, slot].float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [
+    (8, 2, 128, 16), (5, 5, 64, 16), (12, 1, 128, 32), (3, 3, 64, 64),
+])
+def test_prefill_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size):
+    """The matrix-core kernel for portions of prompts: whole prompts, portions with context already
+    cached, lengths that are no multiple of the tile, beside single tokens in the same batch."""
+    g = torch.Generator().manual_seed(40)
+    seqs = [(0, 130), (70, 1), (13, 9), (0, 2), (200, 65), (63, 64), (5, 1), (0, 64)]
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                extra_width=2 * kv_heads * head_dim)
+    kw = dict(num_seqs=len(seqs), max_q_len=130, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+              scale=head_dim ** -0.5)
+    want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype), cu, ctx, table, **kw).float()
+    got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV),
+                              torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
+                              cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=2, max_ctx=265, **kw).cpu().float()
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("window", [1, 7, 64, 100])
+def test_prefill_attention_kernel_window(ops, window):
+    g = torch.Generator().manual_seed(41)
+    seqs = [(0, 150), (90, 40), (3, 2)]
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, 4, 2, 64, 16)
+    kw = dict(num_seqs=3, max_q_len=150, q_heads=4, kv_heads=2, head_dim=64, scale=0.125, window=window)
+    want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], 256, dtype=q.dtype), cu, ctx, table, **kw).float()
+    got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), torch.empty(q.shape[0], 256, dtype=q.dtype, device=DEV),
+                              cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=0, **kw).cpu().float()
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
+def test_prefill_attention_far_key_and_tile_edges(ops):
+    """A query late in a long prompt whose score for one early key stands far out: the key is put at
+    the first and last slot of a page and of a 64-key tile in turn."""
+    g = torch.Generator().manual_seed(42)
+    head_dim, block_size, length = 128, 16, 600
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, [(0, length)], 2, 1, head_dim, block_size)
+    q = (q.float() * 0.01).to(torch.bfloat16)
+    query = 577
+    for far in (0, 15, 16, 63, 64, 127, 128, 300, 575, 576, 577):
+        kq, qq = kp.clone(), q.clone()
+        page, slot = int(table[0, far // block_size]), far % block_size
+        kq[page, 0, slot] = 0.0
+        kq[page, 0, slot, 9] = 30.0
+        qq[query, 9] = 30.0
+        qq[query, head_dim + 9] = 30.0
+        got = ops.paged_attention(qq.to(DEV), kq.to(DEV), vp.to(DEV), torch.empty(length, 2 * head_dim, dtype=q.dtype, device=DEV),
+                                  cu.to(DEV), ctx.to(DEV), table.to(DEV), num_seqs=1, max_q_len=length, q_heads=2, kv_heads=1,
+                                  head_dim=head_dim, scale=head_dim ** -0.5, num_decode=0).cpu().float()
+        for h in range(2):
+            torch.testing.assert_close(got[query, h * head_dim:(h + 1) * head_dim], vp[page, 0, slot].float(), atol=2e-2, rtol=2e-2)
+    # a key after the query must stay invisible however large its score would be
+    kq = kp.clone()
+    page, slot = int(table[0, 578 // block_size]), 578 % block_size
+    kq[page, 0, slot, 9] = 100.0
+    qq = q.clone()
+    qq[query, 9] = 30.0
+    got = ops.paged_attention(qq.to(DEV), kq.to(DEV), vp.to(DEV), torch.empty(length, 2 * head_dim, dtype=q.dtype, device=DEV),
+                              cu.to(DEV), ctx.to(DEV), table.to(DEV), num_seqs=1, max_q_len=length, q_heads=2, kv_heads=1,
+                              head_dim=head_dim, scale=head_dim ** -0.5, num_decode=0).cpu().float()
+    assert float((got[query, :head_dim] - vp[page, 0, slot].float()).abs().max()) > 0.1
