@@ -164,7 +164,7 @@ def main() -> int:
     step_bytes = weight_bytes(model) + args.batch * mean_ctx * kv_bytes_per_token
     achieved = step_bytes / seconds / 1e9
     record = {
-        "metric": "decode tok/s at batch 8 (Qwen3-4B sizes, 1,024-token prompts)",
+        "metric": f"decode tok/s at batch {args.batch} (Qwen3-4B sizes, {args.prompt_len}-token prompts)",
         "value": round(args.batch / seconds, 2),
         "unit": "tokens/s",
         "n_gpus": 1,

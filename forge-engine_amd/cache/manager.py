@@ -172,6 +172,17 @@ class CacheManager:
                     table[b] = NO_PAGE
                 entry.first_block[g] = passed[-1] + 1
 
+    def commit_single_tokens(self, entries: list[RequestCache]) -> None:
+        """``commit`` for requests that each grew by one token (the decode step)."""
+        windowed = any(group.window is not None for group in self.groups)
+        for entry in entries:
+            if windowed:
+                self.commit(entry.request_id, entry.length + 1)
+            else:
+                if any(len(table) * self.block_size <= entry.length for table in entry.tables):
+                    raise ValueError(f"request '{entry.request_id}' has no page for its next token")
+                entry.length += 1
+
     def end(self, request_id: str) -> None:
         entry = self._requests.pop(request_id, None)
         if entry is None:

@@ -69,15 +69,85 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   }
 }
 
+// The same for rows of up to 256 * 4 * VEC floats with hidden % 4 == 0: the row stays in
+// registers between the two passes and memory is touched in 16-byte pieces.
+__device__ __forceinline__ float4 load4_as_float(const float* p) { return *(const float4*)p; }
+__device__ __forceinline__ float4 load4_as_float(const bf16_t* p) {
+  const uint2 v = *(const uint2*)p;
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+                     __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+}
+__device__ __forceinline__ void store4_from_float(float* p, float4 v) { *(float4*)p = v; }
+__device__ __forceinline__ void store4_from_float(bf16_t* p, float4 v) {
+  uint2 u;
+  u.x = (uint32_t)float_to_bf16(v.x) | ((uint32_t)float_to_bf16(v.y) << 16);
+  u.y = (uint32_t)float_to_bf16(v.z) | ((uint32_t)float_to_bf16(v.w) << 16);
+  *(uint2*)p = u;
+}
+
+template <typename TD, typename TO, int VEC>
+__global__ __launch_bounds__(256) void add_rmsnorm_regs_kernel(
+    float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ w,
+    TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps, int store_sum) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int s = rows ? rows[r] : r;
+  float* hrow = h + (size_t)s * hidden;
+  const TD* drow = delta ? delta + (size_t)s * hidden : nullptr;
+  float4 v[VEC];
+  float sumsq = 0.f;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const int i = (threadIdx.x + j * 256) * 4;
+    v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < hidden) {
+      v[j] = load4_as_float(hrow + i);
+      if (drow) {
+        const float4 d = load4_as_float(drow + i);
+        v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
+        if (store_sum) *(float4*)(hrow + i) = v[j];
+      }
+      sumsq += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+    }
+  }
+  const float total = block_sum(sumsq, scratch);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+  TO* orow = out + (size_t)r * hidden;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const int i = (threadIdx.x + j * 256) * 4;
+    if (i < hidden) {
+      const float4 ww = *(const float4*)(w + i);
+      store4_from_float(orow + i, make_float4(v[j].x * inv * ww.x, v[j].y * inv * ww.y,
+                                              v[j].z * inv * ww.z, v[j].w * inv * ww.w));
+    }
+  }
+}
+
+template <typename TD, typename TO>
+static void launch_add_rmsnorm_typed(float* h, const TD* delta, const float* w, TO* out, const int* rows,
+                                     int n_rows, int hidden, float eps, int store_sum, hipStream_t stream) {
+  const bool aligned = hidden % 4 == 0 && (((uintptr_t)h | (uintptr_t)delta | (uintptr_t)w | (uintptr_t)out) & 15) == 0;
+  if (aligned && hidden <= 1024)
+    add_rmsnorm_regs_kernel<TD, TO, 1><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum);
+  else if (aligned && hidden <= 4096)
+    add_rmsnorm_regs_kernel<TD, TO, 4><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum);
+  else if (aligned && hidden <= 8192)
+    add_rmsnorm_regs_kernel<TD, TO, 8><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum);
+  else {
+    const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
+    add_rmsnorm_kernel<TD, TO><<<n_rows, threads, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum);
+  }
+}
+
 template <typename TD>
 static int launch_add_rmsnorm(float* h, const TD* delta, const float* w, void* out, int out_dtype,
                               const int* rows, int n_rows, int hidden, float eps, int store_sum,
                               hipStream_t stream) {
-  const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
   if (out_dtype == FE_F32)
-    add_rmsnorm_kernel<TD, float><<<n_rows, threads, 0, stream>>>(h, delta, w, (float*)out, rows, hidden, eps, store_sum);
+    launch_add_rmsnorm_typed<TD, float>(h, delta, w, (float*)out, rows, n_rows, hidden, eps, store_sum, stream);
   else if (out_dtype == FE_BF16)
-    add_rmsnorm_kernel<TD, bf16_t><<<n_rows, threads, 0, stream>>>(h, delta, w, (bf16_t*)out, rows, hidden, eps, store_sum);
+    launch_add_rmsnorm_typed<TD, bf16_t>(h, delta, w, (bf16_t*)out, rows, n_rows, hidden, eps, store_sum, stream);
   else
     return FE_BAD_ARGUMENT;
   return fe_check_launch();

@@ -30,36 +30,69 @@ __device__ __forceinline__ int row_status(const float* row, int vocab, float* sc
   return result;
 }
 
-// tokens[row] = index of the largest entry; the lowest index wins ties.
-__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_rows_kernel(
-    const float* __restrict__ logits, long long row_stride, int vocab, int* __restrict__ tokens,
-    int* __restrict__ status) {
-  __shared__ float best_v[SAMPLE_WAVES];
-  __shared__ int best_i[SAMPLE_WAVES];
-  __shared__ int flags[2];
-  const float* row = logits + (size_t)blockIdx.x * row_stride;
-  const int st = row_status(row, vocab, best_v, flags);
+// tokens[row] = index of the largest entry; the lowest index wins ties.  Two
+// stages so that a few long rows still fill the chip: ARGMAX_PARTS blocks per
+// row each scan a contiguous part, then one block per row merges them.
+#define ARGMAX_PARTS 32
+
+__device__ __forceinline__ void argmax_merge(float& bv, int& bi, float ov, int oi) {
+  if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+}
+
+__global__ __launch_bounds__(256) void argmax_parts_kernel(
+    const float* __restrict__ logits, long long row_stride, int vocab, float* __restrict__ part_v,
+    int* __restrict__ part_i, int* __restrict__ part_flags) {
+  __shared__ float best_v[4];
+  __shared__ int best_i[4];
+  __shared__ int flags_s[4];
+  const int part = blockIdx.x, row_id = blockIdx.y;
+  const float* row = logits + (size_t)row_id * row_stride;
+  const int per = (vocab + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
+  const int begin = part * per, end = min(vocab, begin + per);
   float bv = -INFINITY;
-  int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+  int bi = 0x7fffffff, flags = 0;   // bit 0 NaN, bit 1 +inf, bit 3 a finite entry was seen
+  for (int i = begin + threadIdx.x; i < end; i += 256) {
     const float v = row[i];
-    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+    if (v != v) flags |= 1;
+    else if (v == INFINITY) flags |= 2;
+    else if (v != -INFINITY) flags |= 8;
+    argmax_merge(bv, bi, v, i);
   }
 #pragma unroll
   for (int offset = FE_WAVE / 2; offset > 0; offset >>= 1) {
-    const float ov = __shfl_xor(bv, offset, FE_WAVE);
-    const int oi = __shfl_xor(bi, offset, FE_WAVE);
-    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    argmax_merge(bv, bi, __shfl_xor(bv, offset, FE_WAVE), __shfl_xor(bi, offset, FE_WAVE));
+    flags |= __shfl_xor(flags, offset, FE_WAVE);
   }
-  const int lane = threadIdx.x & (FE_WAVE - 1);
-  const int wave = threadIdx.x / FE_WAVE;
-  if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
+  const int lane = threadIdx.x & (FE_WAVE - 1), wave = threadIdx.x / FE_WAVE;
+  if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; flags_s[wave] = flags; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int w = 1; w < SAMPLE_WAVES; ++w)
-      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
-    tokens[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
-    status[blockIdx.x] = st;
+    for (int w = 1; w < 4; ++w) { argmax_merge(bv, bi, best_v[w], best_i[w]); flags |= flags_s[w]; }
+    part_v[row_id * ARGMAX_PARTS + part] = bv;
+    part_i[row_id * ARGMAX_PARTS + part] = bi;
+    part_flags[row_id * ARGMAX_PARTS + part] = flags;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_merge_kernel(
+    const float* __restrict__ part_v, const int* __restrict__ part_i, const int* __restrict__ part_flags,
+    int* __restrict__ tokens, int* __restrict__ status) {
+  const int row_id = blockIdx.x, lane = threadIdx.x;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff, flags = 0;
+  if (lane < ARGMAX_PARTS) {
+    bv = part_v[row_id * ARGMAX_PARTS + lane];
+    bi = part_i[row_id * ARGMAX_PARTS + lane];
+    flags = part_flags[row_id * ARGMAX_PARTS + lane];
+  }
+#pragma unroll
+  for (int offset = FE_WAVE / 2; offset > 0; offset >>= 1) {
+    argmax_merge(bv, bi, __shfl_xor(bv, offset, FE_WAVE), __shfl_xor(bi, offset, FE_WAVE));
+    flags |= __shfl_xor(flags, offset, FE_WAVE);
+  }
+  if (lane == 0) {
+    tokens[row_id] = bi == 0x7fffffff ? 0 : bi;
+    status[row_id] = (flags & 3) | ((flags & 8) ? 0 : 4);
   }
 }
 
@@ -161,11 +194,17 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
   }
 }
 
+// scratch: at least rows * 32 * 3 four-byte words (partial maxima, indices, flags).
 extern "C" int fe_argmax_rows(const float* logits, long long row_stride, int rows, int vocab,
-                              int* tokens, int* status, hipStream_t stream) {
+                              int* tokens, int* status, void* scratch, hipStream_t stream) {
   if (rows <= 0) return FE_OK;
-  if (vocab <= 0 || row_stride < vocab) return FE_BAD_ARGUMENT;
-  argmax_rows_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, row_stride, vocab, tokens, status);
+  if (vocab <= 0 || row_stride < vocab || !scratch || rows > 65535) return FE_BAD_ARGUMENT;
+  float* part_v = (float*)scratch;
+  int* part_i = (int*)scratch + (size_t)rows * ARGMAX_PARTS;
+  int* part_flags = part_i + (size_t)rows * ARGMAX_PARTS;
+  dim3 grid(ARGMAX_PARTS, rows);
+  argmax_parts_kernel<<<grid, 256, 0, stream>>>(logits, row_stride, vocab, part_v, part_i, part_flags);
+  argmax_merge_kernel<<<rows, 64, 0, stream>>>(part_v, part_i, part_flags, tokens, status);
   return fe_check_launch();
 }
 

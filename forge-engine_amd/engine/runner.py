@@ -7,6 +7,7 @@ trace replay all go through ``ModelRunner.step``.
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 from torch import Tensor
 
@@ -22,17 +23,52 @@ GRAPH_LIMIT = 24             # captured graphs kept (least recently used goes fi
 
 class _DecodeGraph:
     """One captured decode step: fixed request count and block-table widths.
-    The step's metadata lives in a static buffer that each replay refills."""
+    The step's metadata lives in a static buffer (laid out as ``build_batch``
+    lays out a batch of single tokens) that each replay refills; block-table
+    rows are rewritten only when a request's table changed."""
 
     def __init__(self, num_seqs: int, widths, device) -> None:
-        size = static_batch_size(num_seqs, widths)
+        n = num_seqs
+        size = static_batch_size(n, widths)
         self.host = torch.empty(size, dtype=torch.int32).pin_memory()
         self.dev = torch.zeros(size, dtype=torch.int32, device=device)
+        self.np = self.host.numpy()
         self.widths = list(widths)
+        self.n = n
+        self.np[:] = -1
+        self.np[2 * n:3 * n] = np.arange(n)              # token_seq
+        self.np[3 * n:4 * n + 1] = np.arange(n + 1)      # cu_q
+        self.np[7 * n + 1:8 * n + 1] = np.arange(n)      # want_rows
+        self.table_at = []
+        offset = 8 * n + 1
+        for width in self.widths:
+            self.table_at.append(offset)
+            offset += n * width
+        self.row_keys = [[None] * n for _ in self.widths]
         self.graph = None
         self.logits = None
         self.views = None
+        self.batch = None
         self.copied = torch.cuda.Event()   # the last upload of the host buffer
+
+    def fill(self, tokens, before, records) -> None:
+        n, buf = self.n, self.np
+        before = np.asarray(before, dtype=np.int32)
+        buf[0:n] = tokens
+        buf[n:2 * n] = before                            # positions
+        buf[4 * n + 1:5 * n + 1] = before + 1            # ctx_len
+        buf[5 * n + 1:6 * n + 1] = before                # ctx_before
+        buf[6 * n + 1:7 * n + 1] = [r.state_slot for r in records]
+        for g, width in enumerate(self.widths):
+            keys, base = self.row_keys[g], self.table_at[g]
+            for i, record in enumerate(records):
+                table = record.tables[g]
+                key = (record.request_id, len(table), record.first_block[g])
+                if keys[i] != key:
+                    row = buf[base + i * width:base + (i + 1) * width]
+                    row[:len(table)] = table
+                    row[len(table):] = -1
+                    keys[i] = key
 
 
 class ModelRunner:
@@ -129,13 +165,22 @@ class ModelRunner:
         """A decode-only step (one token and one wanted row per request) as a
         replay of a captured HIP graph: the launches of a step cost more host
         time than the step takes on the GPU."""
-        self._check(entries)
-        before = [self.cache.length(e.request_id) for e in entries]
-        self.cache.reserve({e.request_id: before[i] + 1 for i, e in enumerate(entries)})
-        records = [self.cache.request(e.request_id) for e in entries]
-        tables = [[record.tables[g] for record in records] for g in range(len(self.cache.groups))]
-        widths = tuple(-(-max(1, max(len(t) for t in group)) // GRAPH_TABLE_STEP) * GRAPH_TABLE_STEP
-                       for group in tables)
+        cache = self.cache
+        vocab = self.model.plan.vocab_size
+        records = [cache.request(e.request_id) for e in entries]
+        if len({e.request_id for e in entries}) != len(entries):
+            raise ValueError("a request appears twice in one step")
+        tokens = [e.tokens[0] for e in entries]
+        if min(tokens) < 0 or max(tokens) >= vocab:
+            raise ValueError(f"a token id is outside the vocabulary of {vocab}")
+        before = [r.length for r in records]
+        need = {r.request_id: b + 1 for r, b in zip(records, before)
+                if any(len(t) * self.block_size <= b for t in r.tables)}
+        if need:
+            cache.reserve(need)
+        groups = range(len(cache.groups))
+        widths = tuple(-(-max(1, max(len(r.tables[g]) for r in records)) // GRAPH_TABLE_STEP) * GRAPH_TABLE_STEP
+                       for g in groups)
         key = (len(entries), widths)
         slot = self._graphs.pop(key, None)
         if slot is None:
@@ -143,12 +188,15 @@ class ModelRunner:
                 self._graphs.pop(next(iter(self._graphs)))
             slot = _DecodeGraph(len(entries), widths, self.device)
         self._graphs[key] = slot   # most recently used last
-        bound = max(widths, default=GRAPH_TABLE_STEP) * self.block_size
         slot.copied.synchronize()          # the pinned buffer is free to be rewritten
-        batch = build_batch(entries, before, [r.state_slot for r in records], tables, self.device,
-                            widths=widths, static=(slot.host, slot.dev), max_ctx=bound)
+        slot.fill(tokens, before, records)
+        slot.dev.copy_(slot.host, non_blocking=True)
         slot.copied.record(torch.cuda.current_stream(self.device))
         if slot.graph is None:
+            bound = max(widths, default=GRAPH_TABLE_STEP) * self.block_size
+            tables = [[record.tables[g] for record in records] for g in groups]
+            batch = build_batch(entries, before, [r.state_slot for r in records], tables, self.device,
+                                widths=widths, static=(slot.host, slot.dev), max_ctx=bound)
             views = self.cache_views(batch)
             side = torch.cuda.Stream(device=self.device)
             side.wait_stream(torch.cuda.current_stream(self.device))
@@ -158,11 +206,10 @@ class ModelRunner:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 slot.logits = self.model.forward(batch, views)
-            slot.graph, slot.views = graph, views
+            slot.graph, slot.views, slot.batch = graph, views, batch
         slot.graph.replay()
         self.graph_replays += 1
-        for i, entry in enumerate(entries):
-            self.cache.commit(entry.request_id, before[i] + 1)
+        cache.commit_single_tokens(records)
         self.steps_run += 1
         return slot.logits
 

@@ -159,13 +159,16 @@ def gemm_nt_f32(a: Tensor, b: Tensor, bias: Tensor | None = None, out: Tensor | 
     return out
 
 
-SKINNY_MAX_ROWS = 64       # the decode product takes up to this many tokens
+# The weight-streaming kernel takes up to 64 rows; measured on MI355X it beats the matrix library up
+# to 16 rows (one MFMA row tile) and loses beyond, so the policy below stops there.
+SKINNY_KERNEL_ROWS = 64
+SKINNY_MAX_ROWS = 16
 _EPI_F32, _EPI_BF16, _EPI_SWIGLU = 0, 1, 2
 
 
-def _skinny_fits(x: Tensor, weight: Tensor) -> bool:
+def _skinny_fits(x: Tensor, weight: Tensor, rows: int = SKINNY_MAX_ROWS) -> bool:
     return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2
-            and x.shape[0] <= SKINNY_MAX_ROWS and x.is_contiguous() and x.shape[1] % 8 == 0
+            and x.shape[0] <= rows and x.is_contiguous() and x.shape[1] % 8 == 0
             and weight.stride(1) == 1 and weight.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
@@ -177,7 +180,7 @@ def gemm_skinny(x: Tensor, weight: Tensor, epilogue: str = "bf16", tiles: int = 
     [2I, K] with the gate rows first and y = silu(x Wg^T) * (x Wu^T) in bfloat16."""
     _gpu(x, "x", torch.bfloat16)
     _gpu(weight, "weight", torch.bfloat16, contiguous=False)
-    if not _skinny_fits(x, weight):
+    if not _skinny_fits(x, weight, SKINNY_KERNEL_ROWS):
         raise KernelError("the skinny product takes at most 64 contiguous bfloat16 rows with K a multiple of 8")
     m, k = x.shape
     rows = weight.shape[0]
@@ -391,8 +394,9 @@ def argmax_rows(logits: Tensor, tokens: Tensor, status: Tensor) -> None:
     rows, vocab = logits.shape
     if tokens.numel() != rows or status.numel() != rows:
         raise KernelError("tokens and status need one entry per row")
+    scratch = torch.empty(rows * 32 * 3, dtype=torch.int32, device=logits.device)
     _call("sample", "fe_argmax_rows", _ptr(logits), c_longlong(logits.stride(0)), c_int(rows),
-          c_int(vocab), _ptr(tokens), _ptr(status), _stream())
+          c_int(vocab), _ptr(tokens), _ptr(status), _ptr(scratch), _stream())
 
 
 def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index: Tensor,

@@ -471,3 +471,37 @@ def test_toy_architecture_registered_from_a_test(dtype):
         scale = float(want[k].abs().max())
         bound = 1e-4 * scale + 1e-5 if dtype == "float32" else ru.BF16_FRACTION * scale
         assert float((rows - want[k]).abs().max()) <= bound, k
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_batched_decode_through_graphs_matches_eager(dtype, folders):
+    """Twenty requests decode together (more than 16 rows: the matrix library's products sit
+    inside the captured graph); every replay is compared with the eager step, with eager
+    prompt portions of a late request between the replays."""
+    name = "C"
+    config = TINY[name]
+    requests = ru.make_requests(config, 23, tuple(range(17, 57, 2)))        # 20 requests of 17..55 tokens
+    late = ru.make_requests(config, 24, (50,))["r0"]
+    _, model = load_model(folders[name], dtype=dtype, device=DEV)
+    rows = {}
+    for graphs in (True, False):
+        runner = ModelRunner(model, block_size=16, block_capacity=120, num_state_slots=24, use_graphs=graphs)
+        for k, tokens in requests.items():
+            runner.begin(k)
+            runner.step([StepEntry(k, tokens[:-14], [])])
+        runner.begin("late")
+        collected = []
+        for step in range(14):
+            entries = [StepEntry(k, [tokens[len(tokens) - 14 + step]], [0]) for k, tokens in requests.items()]
+            collected.append(runner.step(entries).clone())
+            if step % 3 == 0:
+                runner.step([StepEntry("late", late[step * 3:step * 3 + 9], [0])])
+        rows[graphs] = torch.stack(collected).cpu()
+        assert (runner.graph_replays == 14) == graphs
+        for k in list(requests) + ["late"]:
+            runner.end(k)
+    want = torch.stack([plain.forward(folder_weights(folders[name]), config, tokens)[-14:] for tokens in requests.values()], dim=1)
+    scale = float(want.abs().max())
+    bound = 1e-4 * scale if dtype == "float32" else ru.BF16_FRACTION * scale
+    assert float((rows[True] - rows[False]).abs().max()) <= bound * 0.5
+    assert float((rows[True] - want).abs().max()) <= bound

@@ -364,7 +364,10 @@ def test_gemm_skinny_swiglu(ops, m, inter, k):
     want = refs.linear_swiglu(x, w).float()
     got = ops.gemm_skinny(x.to(DEV), w.to(DEV), "swiglu").cpu().float()
     torch.testing.assert_close(got, want, atol=1e-2 * float(want.abs().max()) + 1e-6, rtol=1e-2)
-    assert torch.equal(ops.linear_swiglu(x.to(DEV), w.to(DEV)).cpu().float(), got)
+    routed = ops.linear_swiglu(x.to(DEV), w.to(DEV)).cpu().float()   # up to 16 rows: this kernel; more: library + SwiGLU kernel
+    if m <= 16:
+        assert torch.equal(routed, got)
+    torch.testing.assert_close(routed, want, atol=1e-2 * float(want.abs().max()) + 1e-6, rtol=1e-2)
 
 
 def test_linear_routes_by_rows_and_dtype(ops):
