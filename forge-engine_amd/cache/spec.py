@@ -35,8 +35,8 @@ class CacheNeeds:
 class CacheView:
     """What one layer call sees of the cache in one step.
 
-    ``key_pages``/``value_pages``: [blocks, kv_heads, block_size, head_dim] of
-    this call's cache slot; ``block_table``: int32 [sequences, max_blocks] of the
+    ``key_pages`` [blocks, kv_heads, block_size, head_dim] and ``value_pages``
+    (transposed) [blocks, kv_heads, head_dim, block_size] of this call's cache slot; ``block_table``: int32 [sequences, max_blocks] of the
     slot's group (entry -1: no page); ``state``: [slots, *shape] of this call's
     fixed-size state, indexed by ``StepBatch.state_slots``.
     """

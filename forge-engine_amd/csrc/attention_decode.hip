@@ -1,51 +1,50 @@
 // Paged grouped-query attention for single decoded tokens, bfloat16 cache.
 //
 // For every sequence of the batch that brings exactly one query token (others
-// are skipped: they belong to the prefill kernel), the G query heads that share
-// a kv head read that head's keys and values once.  The kernel is bound by the
-// cache's bytes, so the work is laid out for streaming:
+// are skipped: another kernel serves them), the G query heads that share a kv
+// head read that head's keys and values once.  The kernel is bound by the
+// cache's bytes; everything between the loads and the output stays in
+// registers:
 //   * grid (key split, kv head, sequence); with few sequences the keys of one
 //     (sequence, head) are split over several blocks so that the chip is full,
 //     and a second small kernel merges the splits;
-//   * inside a block, the four waves take 16-key tiles in turn; a tile of keys
-//     is 16 rows of D contiguous bfloat16 in its page;
-//   * scores: MFMA 16x16x32 (A = the G query rows padded to 16, B = keys);
-//     softmax statistics in float32, online over tiles;
-//   * values: plain FMAs (the reduction runs over keys, which are not
-//     contiguous per lane in the page layout, and there is bandwidth to spare).
-// Exactness: scores, max, sum and the weighted value sum are float32; one
-// rounding at the final store.
+//   * inside a block the four waves take 32-key blocks in turn;
+//   * scores transposed, S^T = K Q^T: MFMA 16x16x32 with A = 16 keys (rows) and
+//     B = the G query rows padded to 16 (columns).  The 32 keys of a block feed
+//     two MFMA tiles whose rows interleave in groups of four, so that lane
+//     group lq ends up with the scores of the 8 consecutive keys 8lq .. 8lq+7 of
+//     its query row: exactly the B operand of the second product;
+//   * softmax statistics per query row in float32 (a row's keys sit in four
+//     lanes: two shuffles), base-2 exponent with the scale folded in;
+//   * output transposed, O^T = V^T P^T: A = 16 dims x 32 keys from the value
+//     pages, which are stored transposed ([D][slot]) for this, B = P^T.
+// Exactness: scores, max, sum and the weighted value sum are float32; P is
+// rounded to bfloat16 for the second product; one rounding at the final store.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 
-#define TILE 16          // keys per tile
+#define KEYS 32          // keys per block of work
 #define WAVES 4
+#define GMAX 8           // largest group size served
 
-__device__ __forceinline__ void unpack8(const uintx4 v, float* f) {
-  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
-  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
-  f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
-  f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+__device__ __forceinline__ unsigned int pack_bf16(float lo, float hi) {
+  return (unsigned int)float_to_bf16(lo) | ((unsigned int)float_to_bf16(hi) << 16);
 }
 
-// D: head size (64, 128, 256); GT: upper bound of the group size handled (1, 2, 4, 8).
-template <int D, int GT>
+template <int D>
 __global__ __launch_bounds__(256) void paged_decode_kernel(
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     float* __restrict__ part_o, float* __restrict__ part_ml, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const int* __restrict__ block_table, int table_stride,
-    int kv_heads, int groups, int block_size, int num_blocks, int window, float scale) {
-  constexpr int KC = D / 32;        // MFMA k-steps over the head dim
-  constexpr int LPK = D / 8;        // lanes that cover one value row with 16-byte loads
-  constexpr int KPI = 64 / LPK;     // value rows per load instruction
-  __shared__ float Ps[WAVES][16][TILE + 1];
-  __shared__ float Cs[WAVES][16];
-  __shared__ float Ow[WAVES][GT][D];
-  __shared__ float Ms[WAVES][GT], Ls[WAVES][GT];
+    int kv_heads, int groups, int block_size, int num_blocks, int window, float scale_log2) {
+  constexpr int KC = D / 32;        // MFMA k-steps over the head dim (scores)
+  constexpr int DT = D / 16;        // 16-dim tiles of the output
+  __shared__ float Ow[WAVES][GMAX][D];
+  __shared__ float Ms[WAVES][GMAX], Ls[WAVES][GMAX];
 
   const int split = blockIdx.x, splits = gridDim.x;
   const int hk = blockIdx.y, seq = blockIdx.z;
@@ -53,210 +52,190 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(
   if (cu_q[seq + 1] - q0 != 1) return;
   const int ctx = ctx_len[seq];
   const int k_begin = window > 0 ? max(0, ctx - window) : 0;
-  const int tile_first = k_begin / TILE;
-  const int tile_last = (ctx + TILE - 1) / TILE;          // exclusive
-  const int per_split = (tile_last - tile_first + splits - 1) / splits;
-  const int my_first = tile_first + split * per_split;
-  const int my_last = min(tile_last, my_first + per_split);
+  const int first = k_begin / KEYS;
+  const int last = (ctx + KEYS - 1) / KEYS;               // exclusive
+  const int per_split = (last - first + splits - 1) / splits;
+  const int my_first = first + split * per_split;
+  const int my_last = min(last, my_first + per_split);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 15, lq = lane >> 4;
-  const int kq = lane / LPK, dl = lane % LPK;
 
-  // query rows as the A operand: lane (lr = row, lq) holds q[row][32*c + 8*lq .. +8]
-  bf16x8 qa[KC];
+  // query rows as the B operand: lane (lr = row g, lq) holds q[g][32c + 8lq .. +8]
+  bf16x8 qb[KC];
   {
     const bf16_t* qrow = q + (size_t)q0 * q_stride + (size_t)(hk * groups + (lr < groups ? lr : 0)) * D;
 #pragma unroll
     for (int c = 0; c < KC; ++c) {
       uintx4 v = uintx4{0u, 0u, 0u, 0u};
       if (lr < groups) v = *(const uintx4*)(qrow + c * 32 + lq * 8);
-      qa[c] = __builtin_bit_cast(bf16x8, v);
+      qb[c] = __builtin_bit_cast(bf16x8, v);
     }
   }
 
-  float m_run[4], l_run[4];   // rows 4*lq + i, replicated over the 16 lanes of the group
+  float m_run = -INFINITY, l_run = 0.f;   // of query row lr (the same in the four lanes that share it)
+  floatx4 o[DT];                          // O^T: dims 16t + 4lq + i of query row lr
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { m_run[i] = -INFINITY; l_run[i] = 0.f; }
-  float acc[GT][8];           // this lane's keys (kq) x its 8 dims (dl), all rows
-#pragma unroll
-  for (int g = 0; g < GT; ++g)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+  for (int t = 0; t < DT; ++t) o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   const int* table = block_table + (size_t)seq * table_stride;
-  for (int t = my_first + wave; t < my_last; t += WAVES) {
-    const int key0 = t * TILE;
-    const int block = table[key0 / block_size];
-    const bool page_ok = block >= 0 && block < num_blocks;
-    const size_t tile_off = (((size_t)(page_ok ? block : 0) * kv_heads + hk) * block_size + (key0 % block_size)) * D;
-    // issue this tile's loads: keys (MFMA B operand) and values (16 bytes per lane)
-    uintx4 kb[KC];
+  // MFMA row r of key tile h (h = 0, 1) is key 8*(r/4) + 4h + r%4 of the block
+  const int krow = 8 * (lr >> 2) + (lr & 3);
+  uintx4 ka[2][KC], ka_next[2][KC];
+  auto fetch_keys = [&](int b, uintx4 (*dst)[KC]) {
 #pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      kb[c] = uintx4{0u, 0u, 0u, 0u};
-      if (page_ok) kb[c] = *(const uintx4*)(key_pages + tile_off + (size_t)lr * D + c * 32 + lq * 8);
-    }
-    uintx4 vb[TILE / KPI];
+    for (int h = 0; h < 2; ++h) {
+      const int key = b * KEYS + krow + 4 * h;
+      const int block = key < ctx ? table[key / block_size] : -1;
+      const bool ok = block >= 0 && block < num_blocks;
+      const bf16_t* row = key_pages + (((size_t)(ok ? block : 0) * kv_heads + hk) * block_size + key % block_size) * D;
 #pragma unroll
-    for (int j = 0; j < TILE / KPI; ++j) {
-      vb[j] = uintx4{0u, 0u, 0u, 0u};
-      if (page_ok) vb[j] = *(const uintx4*)(value_pages + tile_off + (size_t)(j * KPI + kq) * D + dl * 8);
-    }
-    floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int c = 0; c < KC; ++c)
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[c], __builtin_bit_cast(bf16x8, kb[c]), s, 0, 0, 0);
-    // lane holds s[i] = score(row 4*lq + i, key key0 + lr)
-    const int key = key0 + lr;
-    const bool visible = page_ok && key >= k_begin && key < ctx;
-    float p[4], corr[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float v = visible ? s[i] * scale : -INFINITY;
-      float mx = v;
-#pragma unroll
-      for (int offset = 8; offset > 0; offset >>= 1) mx = fmaxf(mx, __shfl_xor(mx, offset, FE_WAVE));
-      const float m_new = fmaxf(m_run[i], mx);
-      if (m_new > -INFINITY) {
-        corr[i] = __expf(m_run[i] - m_new);
-        p[i] = __expf(v - m_new);
-      } else {
-        corr[i] = 1.f;
-        p[i] = 0.f;
-      }
-      float sum = p[i];
-#pragma unroll
-      for (int offset = 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset, FE_WAVE);
-      l_run[i] = l_run[i] * corr[i] + sum;
-      m_run[i] = m_new;
-    }
-    // hand the probabilities and corrections to the value lanes through LDS
-#pragma unroll
-    for (int i = 0; i < 4; ++i) Ps[wave][lq * 4 + i][lr] = p[i];
-    if (lr == 0) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) Cs[wave][lq * 4 + i] = corr[i];
-    }
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
-#pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      const float cg = Cs[wave][g];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[g][e] *= cg;
-    }
-#pragma unroll
-    for (int j = 0; j < TILE / KPI; ++j) {
-      float v[8];
-      unpack8(vb[j], v);
-#pragma unroll
-      for (int g = 0; g < GT; ++g) {
-        const float pg = Ps[wave][g][j * KPI + kq];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pg, v[e], acc[g][e]);
+      for (int c = 0; c < KC; ++c) {
+        dst[h][c] = uintx4{0u, 0u, 0u, 0u};
+        if (ok) dst[h][c] = *(const uintx4*)(row + c * 32 + lq * 8);
       }
     }
-    __builtin_amdgcn_wave_barrier();
+  };
+  if (my_first + wave < my_last) fetch_keys(my_first + wave, ka_next);
+  for (int b = my_first + wave; b < my_last; b += WAVES) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int c = 0; c < KC; ++c) ka[h][c] = ka_next[h][c];
+    // this block's values (A operand of the second product): lane (lr = dim, lq) reads the 8
+    // consecutive keys 8lq .. 8lq+7 of dims 16t + lr from the transposed page
+    const int vkey = b * KEYS + 8 * lq;
+    const int vblock = vkey < ctx ? table[vkey / block_size] : -1;
+    const bool v_ok = vblock >= 0 && vblock < num_blocks;
+    const bf16_t* vbase = value_pages + ((size_t)(v_ok ? vblock : 0) * kv_heads + hk) * D * block_size + vkey % block_size;
+    uintx4 va[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      va[t] = uintx4{0u, 0u, 0u, 0u};
+      if (v_ok) va[t] = *(const uintx4*)(vbase + (size_t)(t * 16 + lr) * block_size);
+    }
+    if (b + WAVES < my_last) fetch_keys(b + WAVES, ka_next);   // flies while this block is worked on
+
+    floatx4 st[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      st[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < KC; ++c)
+        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[h][c]), qb[c], st[h], 0, 0, 0);
+    }
+    // lane (lr = query row, lq): st[h][i] = score of key b*32 + 8lq + 4h + i
+    float s[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int key = b * KEYS + 8 * lq + j;
+      const float v = st[j >> 2][j & 3] * scale_log2;
+      s[j] = (key >= k_begin && key < ctx) ? v : -INFINITY;
+      mx = fmaxf(mx, s[j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, FE_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, FE_WAVE));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = m_new > -INFINITY ? m_new : 0.f;
+    const float corr = __builtin_amdgcn_exp2f(m_run - m_use);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      s[j] = __builtin_amdgcn_exp2f(s[j] - m_use);
+      sum += s[j];
+    }
+    sum += __shfl_xor(sum, 16, FE_WAVE);
+    sum += __shfl_xor(sum, 32, FE_WAVE);
+    l_run = l_run * corr + sum;
+    m_run = m_new;
+    uintx4 pw;
+    pw.x = pack_bf16(s[0], s[1]); pw.y = pack_bf16(s[2], s[3]);
+    pw.z = pack_bf16(s[4], s[5]); pw.w = pack_bf16(s[6], s[7]);
+    const bf16x8 pb = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[t][i] *= corr;
+      o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, va[t]), pb, o[t], 0, 0, 0);
+    }
   }
 
-  // add up the key groups of the wave (lanes that differ in kq hold the same dims)
+  // lane (lr = query row, lq) holds O^T[16t + 4lq + i][lr]; the four waves meet in LDS
+  if (lr < groups) {
 #pragma unroll
-  for (int g = 0; g < GT; ++g)
+    for (int t = 0; t < DT; ++t)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float v = acc[g][e];
-#pragma unroll
-      for (int offset = LPK; offset < 64; offset <<= 1) v += __shfl_xor(v, offset, FE_WAVE);
-      acc[g][e] = v;
-    }
-  if (kq == 0) {
-#pragma unroll
-    for (int g = 0; g < GT; ++g)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) Ow[wave][g][dl * 8 + e] = acc[g][e];
-  }
-  if (lr == 0) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (lq * 4 + i < GT) { Ms[wave][lq * 4 + i] = m_run[i]; Ls[wave][lq * 4 + i] = l_run[i]; }
+      for (int i = 0; i < 4; ++i) Ow[wave][lr][t * 16 + lq * 4 + i] = o[t][i];
+    if (lq == 0) { Ms[wave][lr] = m_run; Ls[wave][lr] = l_run; }
   }
   __syncthreads();
 
-  // merge the four waves; write the result, or this split's partial result
   for (int e = tid; e < groups * D; e += 256) {
     const int g = e / D, d = e - g * D;
     float m_tot = -INFINITY;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) m_tot = fmaxf(m_tot, Ms[w][g]);
-    float o = 0.f, l = 0.f;
+    float ov = 0.f, l = 0.f;
     if (m_tot > -INFINITY) {
 #pragma unroll
       for (int w = 0; w < WAVES; ++w) {
-        const float f = __expf(Ms[w][g] - m_tot);
-        o += f * Ow[w][g][d];
+        const float f = __builtin_amdgcn_exp2f(Ms[w][g] - m_tot);
+        ov += f * Ow[w][g][d];
         l += f * Ls[w][g];
       }
     }
     if (splits == 1) {
-      out[(size_t)q0 * out_stride + (size_t)(hk * groups + g) * D + d] = float_to_bf16(l > 0.f ? o / l : 0.f);
+      out[(size_t)q0 * out_stride + (size_t)(hk * groups + g) * D + d] = float_to_bf16(l > 0.f ? ov / l : 0.f);
     } else {
       const size_t slot = ((size_t)seq * kv_heads + hk) * splits + split;
-      part_o[(slot * groups + g) * D + d] = o;
+      part_o[(slot * groups + g) * D + d] = ov;
       if (d == 0) {
-        part_ml[(slot * groups + g) * 2] = m_tot;
+        part_ml[(slot * groups + g) * 2] = m_tot;        // base-2 exponent units
         part_ml[(slot * groups + g) * 2 + 1] = l;
       }
     }
   }
 }
 
-// Merge the splits of one (sequence, kv head): grid (kv head, sequence).
+// Merge the splits of one (sequence, kv head): grid (kv head, sequence).  One thread per output
+// element; the splits' maxima and sums are read once into LDS.
 __global__ __launch_bounds__(256) void paged_decode_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
     long long out_stride, const int* __restrict__ cu_q, int kv_heads, int groups, int head_dim,
     int splits) {
+  __shared__ float scale_s[GMAX][64];   // weight of each split per query row
+  __shared__ float inv_l[GMAX];
   const int hk = blockIdx.x, seq = blockIdx.y;
   const int q0 = cu_q[seq];
   if (cu_q[seq + 1] - q0 != 1) return;
   const size_t first = ((size_t)seq * kv_heads + hk) * splits;
-  for (int e = threadIdx.x; e < groups * head_dim; e += blockDim.x) {
-    const int g = e / head_dim, d = e - g * head_dim;
+  if (threadIdx.x < groups) {
+    const int g = threadIdx.x;
     float m_tot = -INFINITY;
     for (int s = 0; s < splits; ++s) m_tot = fmaxf(m_tot, part_ml[((first + s) * groups + g) * 2]);
-    float o = 0.f, l = 0.f;
-    if (m_tot > -INFINITY) {
-      for (int s = 0; s < splits; ++s) {
-        const float f = __expf(part_ml[((first + s) * groups + g) * 2] - m_tot);
-        o += f * part_o[((first + s) * groups + g) * head_dim + d];
-        l += f * part_ml[((first + s) * groups + g) * 2 + 1];
-      }
+    float l = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float f = m_tot > -INFINITY ? __builtin_amdgcn_exp2f(part_ml[((first + s) * groups + g) * 2] - m_tot) : 0.f;
+      scale_s[g][s] = f;
+      l += f * part_ml[((first + s) * groups + g) * 2 + 1];
     }
-    out[(size_t)q0 * out_stride + (size_t)(hk * groups + g) * head_dim + d] = float_to_bf16(l > 0.f ? o / l : 0.f);
+    inv_l[g] = l > 0.f ? 1.f / l : 0.f;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < groups * head_dim; e += blockDim.x) {
+    const int g = e / head_dim, d = e - g * head_dim;
+    float o = 0.f;
+    for (int s = 0; s < splits; ++s) o += scale_s[g][s] * part_o[((first + s) * groups + g) * head_dim + d];
+    out[(size_t)q0 * out_stride + (size_t)(hk * groups + g) * head_dim + d] = float_to_bf16(o * inv_l[g]);
   }
 }
 
-template <int D>
-static int launch_decode(int gt, dim3 grid, const void* q, long long q_stride, const void* kp, const void* vp,
-                         void* out, long long out_stride, float* part_o, float* part_ml, const int* cu_q,
-                         const int* ctx_len, const int* table, int table_stride, int kv_heads, int groups,
-                         int block_size, int num_blocks, int window, float scale, hipStream_t stream) {
-#define FE_GO(GT)                                                                                          \
-  paged_decode_kernel<D, GT><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)kp,        \
-      (const bf16_t*)vp, (bf16_t*)out, out_stride, part_o, part_ml, cu_q, ctx_len, table, table_stride,      \
-      kv_heads, groups, block_size, num_blocks, window, scale)
-  if (gt <= 1) FE_GO(1);
-  else if (gt <= 2) FE_GO(2);
-  else if (gt <= 4) FE_GO(4);
-  else FE_GO(8);
-#undef FE_GO
-  return fe_check_launch();
-}
-
-// Sequences with one query token only; others are left untouched.  splits > 1
-// needs part_o [num_seqs * kv_heads * splits * groups * head_dim] and part_ml
-// [num_seqs * kv_heads * splits * groups * 2] floats.
+// Sequences with one query token only; others are left untouched.  Pages: keys
+// [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size].
+// splits > 1 (at most 64) needs part_o [num_seqs * kv_heads * splits * groups * head_dim] and
+// part_ml [num_seqs * kv_heads * splits * groups * 2] floats.
 extern "C" int fe_paged_attention_decode(const void* q, long long q_stride, const void* key_pages,
                                          const void* value_pages, void* out, long long out_stride,
                                          float* part_o, float* part_ml, const int* cu_q,
@@ -266,18 +245,21 @@ extern "C" int fe_paged_attention_decode(const void* q, long long q_stride, cons
                                          int splits, hipStream_t stream) {
   if (num_seqs <= 0) return FE_OK;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256) return FE_BAD_ARGUMENT;
-  if (groups < 1 || groups > 8 || kv_heads < 1 || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
-  if (block_size < TILE || block_size % TILE || num_blocks < 1 || table_stride < 1) return FE_BAD_ARGUMENT;
-  if (q_stride % 8 || splits < 1 || splits > 1024) return FE_BAD_ARGUMENT;
+  if (groups < 1 || groups > GMAX || kv_heads < 1 || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
+  if (block_size < 16 || block_size % 16 || num_blocks < 1 || table_stride < 1) return FE_BAD_ARGUMENT;
+  if (q_stride % 8 || splits < 1 || splits > 64) return FE_BAD_ARGUMENT;
   if (splits > 1 && (!part_o || !part_ml)) return FE_BAD_ARGUMENT;
   dim3 grid(splits, kv_heads, num_seqs);
-  int status;
-  if (head_dim == 64)
-    status = launch_decode<64>(groups, grid, q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, cu_q, ctx_len, block_table, table_stride, kv_heads, groups, block_size, num_blocks, window, scale, stream);
-  else if (head_dim == 128)
-    status = launch_decode<128>(groups, grid, q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, cu_q, ctx_len, block_table, table_stride, kv_heads, groups, block_size, num_blocks, window, scale, stream);
-  else
-    status = launch_decode<256>(groups, grid, q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, cu_q, ctx_len, block_table, table_stride, kv_heads, groups, block_size, num_blocks, window, scale, stream);
+  const float scale_log2 = scale * 1.4426950408889634f;
+#define FE_GO(DD)                                                                                          \
+  paged_decode_kernel<DD><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages,    \
+      (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, cu_q, ctx_len, block_table,     \
+      table_stride, kv_heads, groups, block_size, num_blocks, window, scale_log2)
+  if (head_dim == 64) FE_GO(64);
+  else if (head_dim == 128) FE_GO(128);
+  else FE_GO(256);
+#undef FE_GO
+  int status = fe_check_launch();
   if (status != FE_OK || splits == 1) return status;
   dim3 merge_grid(kv_heads, num_seqs);
   paged_decode_merge_kernel<<<merge_grid, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, out_stride, cu_q,

@@ -50,8 +50,8 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
   const int kstride = D + 1;
   float* Qs = smem;                   // [ROWS][D + 1]
   float* Ks = Qs + ROWS * kstride;    // [TK][D + 1]
-  float* Vs = Ks + TK * kstride;      // [TK][D]
-  float* Ps = Vs + TK * D;            // [ROWS][TK]
+  float* Vs = Ks + TK * kstride;      // [TK][D + 1]
+  float* Ps = Vs + TK * kstride;      // [ROWS][TK]
 
   const int seq = blockIdx.z;
   const int hk = blockIdx.y;
@@ -106,20 +106,26 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
       const int d4 = (e - kk * chunks) * 4;
       const int kp = kt + kk;
       float kv[4] = {0.f, 0.f, 0.f, 0.f};
-      float vv[4] = {0.f, 0.f, 0.f, 0.f};
       if (kp >= k_begin && kp < k_end) {
         const int block = table[kp / block_size];
-        if (block >= 0 && block < num_blocks) {
-          const size_t off = (((size_t)block * kv_heads + hk) * block_size + (kp % block_size)) * D + d4;
-          Vec4<T>::load(key_pages + off, kv);
-          Vec4<T>::load(value_pages + off, vv);
-        }
+        if (block >= 0 && block < num_blocks)
+          Vec4<T>::load(key_pages + (((size_t)block * kv_heads + hk) * block_size + (kp % block_size)) * D + d4, kv);
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        Ks[kk * kstride + d4 + i] = kv[i];
-        Vs[kk * D + d4 + i] = vv[i];
+      for (int i = 0; i < 4; ++i) Ks[kk * kstride + d4 + i] = kv[i];
+    }
+    // values live transposed in their pages ([D][slot]): consecutive threads take consecutive keys
+    for (int e = tid; e < TK * D; e += 256) {
+      const int d = e / TK;
+      const int kk = e - d * TK;
+      const int kp = kt + kk;
+      float v = 0.f;
+      if (kp >= k_begin && kp < k_end) {
+        const int block = table[kp / block_size];
+        if (block >= 0 && block < num_blocks)
+          v = load_as_float(value_pages + (((size_t)block * kv_heads + hk) * D + d) * block_size + (kp % block_size));
       }
+      Vs[kk * kstride + d] = v;
     }
     __syncthreads();
 
@@ -169,7 +175,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     const float* prow = Ps + r * TK;
     for (int kk = 0; kk < TK; ++kk) {
       const float p = prow[kk];
-      const float* vrow = Vs + kk * D;
+      const float* vrow = Vs + kk * kstride;
 #pragma unroll
       for (int i = 0; i < DPT; ++i)
         if (c + 16 * i < D) acc[i] = fmaf(p, vrow[c + 16 * i], acc[i]);
@@ -193,7 +199,7 @@ static int launch_generic(const void* q, long long q_stride, const void* key_pag
                           int window, float scale, int min_q_len, int max_q_served, hipStream_t stream) {
   const long long tiles = ((long long)max_q_len * groups + ROWS - 1) / ROWS;
   if (tiles > 0x7fffffffLL || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
-  const size_t smem = sizeof(float) * ((size_t)(ROWS + TK) * (head_dim + 1) + (size_t)TK * head_dim + ROWS * TK);
+  const size_t smem = sizeof(float) * ((size_t)(ROWS + 2 * TK) * (head_dim + 1) + ROWS * TK);
   dim3 grid((unsigned)tiles, kv_heads, num_seqs);
   paged_attention_generic_kernel<T, DMAX, TK, FAST_EXP><<<grid, 256, smem, stream>>>(
       (const T*)q, q_stride, (const T*)key_pages, (const T*)value_pages, (T*)out, out_stride, cu_q,

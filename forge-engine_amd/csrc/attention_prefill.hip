@@ -1,54 +1,72 @@
 // Paged grouped-query attention for portions of prompts (two or more query
 // tokens of one sequence in a step), bfloat16 cache, on the matrix cores.
 //
-// Block = 64 query tokens of one query head of one sequence (grid: query tile,
-// query head, sequence); its four waves take 16 query rows each.  Keys and
-// values are walked in tiles of 64 (whole 16-key runs of pages), loaded once
-// per block into LDS and shared by the four waves:
-//   S = Q K^T   MFMA 16x16x32, A = query rows (registers, loaded once),
-//               B = keys from LDS, row-major [key][D + pad];
-//   softmax     float32, online over tiles, base-2 exponent with the scale
-//               folded in; the causal (and window) mask only where a tile
-//               crosses a row's limits;
-//   O += P V    MFMA 16x16x32 with keys as the k dim: A = P (bfloat16, through
-//               a per-wave LDS tile to change from the score layout to the
-//               operand layout), B = values from LDS stored transposed
-//               [d][key + pad] so that each lane reads 8 consecutive keys.
+// Block = 64 or 128 query tokens of one query head of one sequence; its four
+// waves take 16 or 32 query rows each.  Keys and values are walked in tiles of
+// 64, loaded once per block into LDS and shared by the four waves; keys as
+// stored ([key][D]), values as stored too: their pages are transposed
+// ([D][slot]), which is the operand layout of the second product.
+//   S^T = K Q^T    MFMA 16x16x32, A = 16 keys from LDS, B = 16 query rows held
+//                  in registers for the whole kernel.  The 32 keys of a block
+//                  feed two MFMA tiles whose rows interleave in groups of four,
+//                  so lane group lq gets the scores of keys 8lq .. 8lq+7 of
+//                  its query row: already the B operand of the next product;
+//   softmax        float32, online over tiles, base-2 exponent with the scale
+//                  folded in; a row's keys sit in four lanes (two shuffles);
+//                  the causal (and window) mask only on tiles that cross it;
+//   O^T += V^T P^T MFMA 16x16x32, A = 16 dims x 32 keys from LDS, B = P^T
+//                  (bfloat16, straight from the score registers).
 // Query token i of the step sits at position ctx_before + i and sees keys
 // max(0, p - window + 1) .. p.  Sequences with fewer than two query tokens are
-// skipped (the decode kernel serves them).  Sums and statistics are float32;
-// P is rounded to bfloat16 for the second product, as the reference rounds its
+// skipped (the decode kernel serves them).  Sums and statistics are float32; P
+// is rounded to bfloat16 for the second product, as the reference rounds its
 // probabilities (src/forge_engine/qwen3.py:200).
+//
+// The grid is one-dimensional and aware of the eight XCDs: consecutive block
+// ids land on different XCDs, so block id l works on item (l % 8) * n/8 + l / 8
+// of a list ordered by (sequence, head, query tile): one XCD, with its own L2,
+// gets neighbouring heads, which share keys and values.  Within a head the
+// last query tile, the longest, comes first.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 
-#define BM 64        // query rows per block
 #define BN 64        // keys per tile
 #define KPAD 8       // bf16 padding of a key row in LDS
-#define VPAD 8       // bf16 padding of a transposed value row in LDS
-#define PPAD 8
+#define VPAD 8       // bf16 padding of a value row (one dim, 64 keys) in LDS
+#define XCDS 8
 
-template <int D>
+__device__ __forceinline__ unsigned int pack_bf16(float lo, float hi) {
+  return (unsigned int)float_to_bf16(lo) | ((unsigned int)float_to_bf16(hi) << 16);
+}
+
+template <int D, int RT>
 __global__ __launch_bounds__(256) void paged_prefill_kernel(
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int table_stride, int kv_heads, int groups, int block_size, int num_blocks, int window,
-    float scale_log2) {
+    float scale_log2, int q_tiles, int items_per_xcd, int total_items) {
+  constexpr int BM = 64 * RT;     // query rows per block
   constexpr int KC = D / 32;      // MFMA k-steps over the head dim (scores)
-  constexpr int DT = D / 16;      // 16-wide tiles of the head dim (output)
-  constexpr int CH = D / 8;       // 16-byte chunks per key row
+  constexpr int DT = D / 16;      // 16-dim tiles of the output
+  constexpr int CH = D / 8;       // 16-byte pieces per key row
   __shared__ __attribute__((aligned(16))) bf16_t Ks[BN][D + KPAD];
   __shared__ __attribute__((aligned(16))) bf16_t Vt[D][BN + VPAD];
-  __shared__ __attribute__((aligned(16))) bf16_t Ps[4][16][BN + PPAD];
 
-  const int seq = blockIdx.z, head = blockIdx.y, hk = head / groups;
+  const int heads = kv_heads * groups;
+  const int item = (blockIdx.x % XCDS) * items_per_xcd + blockIdx.x / XCDS;
+  if (item >= total_items) return;   // the list is padded to a multiple of the XCD count
+  const int seq = item / (heads * q_tiles);
+  const int rest = item - seq * heads * q_tiles;
+  const int head = rest / q_tiles;
+  const int q_tile = q_tiles - 1 - (rest - head * q_tiles);
+  const int hk = head / groups;
   const int q0 = cu_q[seq];
   const int q_len = cu_q[seq + 1] - q0;
-  const int row0 = blockIdx.x * BM;
+  const int row0 = q_tile * BM;
   if (q_len < 2 || row0 >= q_len) return;
   const int ctx = ctx_len[seq];
   const int before = ctx - q_len;
@@ -56,38 +74,40 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 15, lq = lane >> 4;
 
-  // this wave's 16 query rows as the A operand: lane (lr = row, lq) holds q[row][32c + 8lq .. +8]
-  const int my_row = row0 + wave * 16 + lr;          // A-operand row of this lane
-  bf16x8 qa[KC];
-  {
-    const bf16_t* qrow = q + (size_t)(q0 + min(my_row, q_len - 1)) * q_stride + (size_t)head * D;
+  // this wave's query rows as B operands: lane (lr = row, lq) holds q[row][32c + 8lq .. +8]
+  bf16x8 qb[RT][KC];
+  int row_pos[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = row0 + (wave * RT + rt) * 16 + lr;
+    row_pos[rt] = before + row;
+    const bf16_t* qrow = q + (size_t)(q0 + min(row, q_len - 1)) * q_stride + (size_t)head * D;
 #pragma unroll
     for (int c = 0; c < KC; ++c) {
       uintx4 v = uintx4{0u, 0u, 0u, 0u};
-      if (my_row < q_len) v = *(const uintx4*)(qrow + c * 32 + lq * 8);
-      qa[c] = __builtin_bit_cast(bf16x8, v);
+      if (row < q_len) v = *(const uintx4*)(qrow + c * 32 + lq * 8);
+      qb[rt][c] = __builtin_bit_cast(bf16x8, v);
     }
   }
-  // score/output layout: lane (lr, lq) holds rows 4lq + i (i < 4) at column lr
-  int row_pos[4];
+  float m_run[RT], l_run[RT];
+  floatx4 o[RT][DT];     // O^T: dims 16t + 4lq + i of query row lr
 #pragma unroll
-  for (int i = 0; i < 4; ++i) row_pos[i] = before + row0 + wave * 16 + lq * 4 + i;
-  float m_run[4], l_run[4];
+  for (int rt = 0; rt < RT; ++rt) {
+    m_run[rt] = -INFINITY;
+    l_run[rt] = 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { m_run[i] = -INFINITY; l_run[i] = 0.f; }
-  floatx4 o[DT];
-#pragma unroll
-  for (int t = 0; t < DT; ++t) o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < DT; ++t) o[rt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
 
   const int last_row = min(q_len, row0 + BM) - 1;
   const int pos_lo = before + row0, pos_hi = before + last_row;
+  const int wave_lo = pos_lo + wave * RT * 16;      // position of this wave's first row
   const int k_first = window > 0 ? max(0, pos_lo - window + 1) : 0;
   const int tile_first = k_first / BN, tile_last = pos_hi / BN;   // inclusive
   const int* table = block_table + (size_t)seq * table_stride;
 
-  // loader mapping.  keys: chunk p -> (key p / CH, 16-byte piece p % CH): rows are read whole.
-  // values: chunk p -> (key p % BN, piece p / BN): a wave's 64 lanes hold 64 keys of one piece,
-  // so the transposed 2-byte stores of a piece land side by side.
+  // loaders: keys piece p -> (key p / CH, 16 bytes p % CH); values piece p -> (dim p / 8, the 8
+  // keys (p % 8) * 8 .. of the tile), read from the transposed page of those keys
   constexpr int LOADS = BN * CH / 256;
   uintx4 kreg[LOADS], vreg[LOADS];
   auto load_tile = [&](int tile) {
@@ -105,12 +125,12 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
         kreg[i] = v;
       }
       {
-        const int key = tile * BN + p % BN;
+        const int key = tile * BN + (p % 8) * 8;
         uintx4 v = uintx4{0u, 0u, 0u, 0u};
         if (key < ctx) {
           const int block = table[key / block_size];
           if (block >= 0 && block < num_blocks)
-            v = *(const uintx4*)(value_pages + (((size_t)block * kv_heads + hk) * block_size + key % block_size) * D + (p / BN) * 8);
+            v = *(const uintx4*)(value_pages + (((size_t)block * kv_heads + hk) * D + p / 8) * block_size + key % block_size);
         }
         vreg[i] = v;
       }
@@ -121,16 +141,11 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
     for (int i = 0; i < LOADS; ++i) {
       const int p = tid + i * 256;
       *(uintx4*)&Ks[p / CH][(p % CH) * 8] = kreg[i];
-      const int key = p % BN, d0 = (p / BN) * 8;
-      const unsigned int w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        Vt[d0 + 2 * e][key] = (bf16_t)(w[e] & 0xffffu);
-        Vt[d0 + 2 * e + 1][key] = (bf16_t)(w[e] >> 16);
-      }
+      *(uintx4*)&Vt[p / 8][(p % 8) * 8] = vreg[i];
     }
   };
 
+  const int krow = 8 * (lr >> 2) + (lr & 3);   // MFMA row r of key tile h is key 8*(r/4) + 4h + r%4 of its 32-key block
   load_tile(tile_first);
   for (int tile = tile_first; tile <= tile_last; ++tile) {
     __syncthreads();            // the previous tile's LDS reads are done
@@ -138,86 +153,100 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
     __syncthreads();
     if (tile < tile_last) load_tile(tile + 1);   // flies while this tile multiplies
 
-    // scores of this wave's 16 rows against the tile's 64 keys
-    floatx4 s[BN / 16];
-#pragma unroll
-    for (int st = 0; st < BN / 16; ++st) {
-      s[st] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int c = 0; c < KC; ++c) {
-        const bf16x8 kb = *(const bf16x8*)&Ks[st * 16 + lr][c * 32 + lq * 8];
-        s[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[c], kb, s[st], 0, 0, 0);
-      }
-    }
     const int key_base = tile * BN;
-    // mask only if the tile reaches beyond some row's position or before its window
-    const bool edge = key_base + BN - 1 > pos_lo + wave * 16 || (window > 0 && key_base < pos_hi - window + 1);
-    float corr[4];
+    if (key_base > wave_lo + RT * 16 - 1 && window <= 0) continue;   // every key of the tile lies after this wave's rows
+    floatx4 st[RT][2][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) st[rt][blk][h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+          const bf16x8 ka = *(const bf16x8*)&Ks[blk * 32 + krow + 4 * h][c * 32 + lq * 8];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            st[rt][blk][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[rt][c], st[rt][blk][h], 0, 0, 0);
+        }
+    // lane (lr = query row, lq): st[rt][blk][h][i] = score of key key_base + 32 blk + 8lq + 4h + i
+    const bool edge = key_base + BN - 1 > wave_lo || (window > 0 && key_base < pos_hi - window + 1);
+    bf16x8 pb[RT][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float s[16];
       float mx = -INFINITY;
 #pragma unroll
-      for (int st = 0; st < BN / 16; ++st) {
-        float v = s[st][i] * scale_log2;
+      for (int j = 0; j < 16; ++j) {
+        float v = st[rt][j >> 3][(j >> 2) & 1][j & 3] * scale_log2;
         if (edge) {
-          const int key = key_base + st * 16 + lr;
-          const bool visible = key <= row_pos[i] && (window <= 0 || key > row_pos[i] - window);
+          const int key = key_base + 32 * (j >> 3) + 8 * lq + (j & 7);
+          const bool visible = key <= row_pos[rt] && (window <= 0 || key > row_pos[rt] - window);
           v = visible ? v : -INFINITY;
         }
-        s[st][i] = v;
+        s[j] = v;
         mx = fmaxf(mx, v);
       }
-#pragma unroll
-      for (int offset = 8; offset > 0; offset >>= 1) mx = fmaxf(mx, __shfl_xor(mx, offset, FE_WAVE));
-      const float m_new = fmaxf(m_run[i], mx);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, FE_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, FE_WAVE));
+      const float m_new = fmaxf(m_run[rt], mx);
       const float m_use = m_new > -INFINITY ? m_new : 0.f;    // a row with nothing visible yet
-      corr[i] = __builtin_amdgcn_exp2f(m_run[i] - m_use);
+      const float corr = __builtin_amdgcn_exp2f(m_run[rt] - m_use);
       float sum = 0.f;
 #pragma unroll
-      for (int st = 0; st < BN / 16; ++st) {
-        const float p = __builtin_amdgcn_exp2f(s[st][i] - m_use);
-        s[st][i] = p;
-        sum += p;
+      for (int j = 0; j < 16; ++j) {
+        s[j] = __builtin_amdgcn_exp2f(s[j] - m_use);
+        sum += s[j];
+      }
+      sum += __shfl_xor(sum, 16, FE_WAVE);
+      sum += __shfl_xor(sum, 32, FE_WAVE);
+      l_run[rt] = l_run[rt] * corr + sum;
+      m_run[rt] = m_new;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        uintx4 pw;
+        pw.x = pack_bf16(s[8 * blk + 0], s[8 * blk + 1]); pw.y = pack_bf16(s[8 * blk + 2], s[8 * blk + 3]);
+        pw.z = pack_bf16(s[8 * blk + 4], s[8 * blk + 5]); pw.w = pack_bf16(s[8 * blk + 6], s[8 * blk + 7]);
+        pb[rt][blk] = __builtin_bit_cast(bf16x8, pw);
       }
 #pragma unroll
-      for (int offset = 8; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset, FE_WAVE);
-      l_run[i] = l_run[i] * corr[i] + sum;
-      m_run[i] = m_new;
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[rt][t][i] *= corr;
     }
-    // P: score layout -> LDS -> operand layout (rows = lr, 8 consecutive keys per lane)
-#pragma unroll
-    for (int st = 0; st < BN / 16; ++st)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) Ps[wave][lq * 4 + i][st * 16 + lr] = float_to_bf16(s[st][i]);
 #pragma unroll
     for (int t = 0; t < DT; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[t][i] *= corr[i];
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
+      for (int blk = 0; blk < 2; ++blk) {
+        const bf16x8 va = *(const bf16x8*)&Vt[t * 16 + lr][blk * 32 + lq * 8];
 #pragma unroll
-    for (int kk = 0; kk < BN / 32; ++kk) {
-      const bf16x8 pa = *(const bf16x8*)&Ps[wave][lr][kk * 32 + lq * 8];
-#pragma unroll
-      for (int t = 0; t < DT; ++t) {
-        const bf16x8 vb = *(const bf16x8*)&Vt[t * 16 + lr][kk * 32 + lq * 8];
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o[t], 0, 0, 0);
+        for (int rt = 0; rt < RT; ++rt)
+          o[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[rt][blk], o[rt][t], 0, 0, 0);
       }
-    }
   }
 
-  // lane holds O[row 4lq + i][d = 16t + lr]
+  // lane (lr = query row, lq) holds O^T[16t + 4lq + i][row]: four consecutive dims per store
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = row0 + wave * 16 + lq * 4 + i;
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = row0 + (wave * RT + rt) * 16 + lr;
     if (row >= q_len) continue;
-    const float inv = l_run[i] > 0.f ? 1.f / l_run[i] : 0.f;
+    const float inv = l_run[rt] > 0.f ? 1.f / l_run[rt] : 0.f;
     bf16_t* orow = out + (size_t)(q0 + row) * out_stride + (size_t)head * D;
 #pragma unroll
-    for (int t = 0; t < DT; ++t) orow[t * 16 + lr] = float_to_bf16(o[t][i] * inv);
+    for (int t = 0; t < DT; ++t) {
+      uint2 w;
+      w.x = pack_bf16(o[rt][t][0] * inv, o[rt][t][1] * inv);
+      w.y = pack_bf16(o[rt][t][2] * inv, o[rt][t][3] * inv);
+      *(uint2*)(orow + t * 16 + lq * 4) = w;
+    }
   }
 }
 
+// Pages: keys [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size].
 extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, const void* key_pages,
                                           const void* value_pages, void* out, long long out_stride,
                                           const int* cu_q, const int* ctx_len, const int* block_table,
@@ -226,16 +255,21 @@ extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, con
                                           int window, float scale, hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len < 2) return FE_OK;
   if (head_dim != 64 && head_dim != 128) return FE_BAD_ARGUMENT;
-  if (groups < 1 || kv_heads < 1 || (long long)kv_heads * groups > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
-  if (block_size < 16 || block_size % 16 || num_blocks < 1 || table_stride < 1 || q_stride % 8) return FE_BAD_ARGUMENT;
-  dim3 grid((max_q_len + BM - 1) / BM, kv_heads * groups, num_seqs);
+  if (groups < 1 || kv_heads < 1 || num_seqs > 65535) return FE_BAD_ARGUMENT;
+  if (block_size < 16 || block_size % 16 || num_blocks < 1 || table_stride < 1 || q_stride % 8 || out_stride % 4) return FE_BAD_ARGUMENT;
   const float scale_log2 = scale * 1.4426950408889634f;
-#define FE_GO(DD)                                                                                           \
-  paged_prefill_kernel<DD><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages,    \
-      (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,         \
-      kv_heads, groups, block_size, num_blocks, window, scale_log2)
-  if (head_dim == 64) FE_GO(64);
-  else FE_GO(128);
+  const int rt = max_q_len >= 512 ? 2 : 1;       // long portions: 128-row blocks halve the reads of keys and values
+  const int q_tiles = (max_q_len + 64 * rt - 1) / (64 * rt);
+  const long long items = (long long)num_seqs * kv_heads * groups * q_tiles;
+  const long long per_xcd = (items + XCDS - 1) / XCDS;
+  if (per_xcd * XCDS > 0x7fffffffLL) return FE_BAD_ARGUMENT;
+  const unsigned grid = (unsigned)(per_xcd * XCDS);
+#define FE_GO(DD, RR)                                                                                        \
+  paged_prefill_kernel<DD, RR><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+      (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,          \
+      kv_heads, groups, block_size, num_blocks, window, scale_log2, q_tiles, (int)per_xcd, (int)items)
+  if (head_dim == 64) { if (rt == 2) FE_GO(64, 2); else FE_GO(64, 1); }
+  else { if (rt == 2) FE_GO(128, 2); else FE_GO(128, 1); }
 #undef FE_GO
   return fe_check_launch();
 }

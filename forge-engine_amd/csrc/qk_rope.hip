@@ -9,9 +9,11 @@
 //   out[j + R/2] = y[j + R/2] * cos(angle) + y[j] * sin(angle)
 //   dims >= R pass through.  All arithmetic in float32, one rounding at the store.
 //
-// Cache layout per layer: pages[block][kv_head][slot][D] for keys and the same
-// for values; token at position p of sequence s lives in block
-// table[s][p / block_size], slot p % block_size.
+// Cache layout per layer: keys pages[block][kv_head][slot][D]; values transposed,
+// pages[block][kv_head][D][slot], so that the attention kernels read 8 consecutive
+// keys of one dim in one piece (the matrix cores reduce over keys there).  The
+// token at position p of sequence s lives in block table[s][p / block_size],
+// slot p % block_size.
 #include "common.h"
 
 template <typename T>
@@ -41,12 +43,13 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
     const int seq = token_seq[t];
     const int block = block_table[(size_t)seq * table_stride + pos / block_size];
     if (block < 0 || block >= num_blocks) return;  // host reserves pages before the launch
-    T* pages = is_k ? key_pages : value_pages;
-    dst = pages + (((size_t)block * kv_heads + kv_head) * block_size + (pos % block_size)) * head_dim;
-  }
-  if (!is_q && !is_k) {  // value: copy
-    for (int d = lane; d < head_dim; d += FE_WAVE) dst[d] = x[d];
-    return;
+    const size_t page = ((size_t)block * kv_heads + kv_head) * block_size * head_dim;
+    if (!is_k) {  // value: copy into the transposed page
+      T* vdst = value_pages + page + (pos % block_size);
+      for (int d = lane; d < head_dim; d += FE_WAVE) vdst[(size_t)d * block_size] = x[d];
+      return;
+    }
+    dst = key_pages + page + (size_t)(pos % block_size) * head_dim;
   }
 
   const float* w = is_q ? q_weight : k_weight;

@@ -87,12 +87,14 @@ class ModelRunner:
                                   num_state_slots=num_state_slots)
         if self.device.type == "cuda":
             library.ensure_built(sorted(model.kernel_libraries()))
-        # pages of a group: [slot in group, key|value, page, kv head, position in page, head dim]
-        self.pages = [
-            torch.zeros((len(g.slots), 2, block_capacity, g.kv_heads, block_size, g.head_dim),
-                        dtype=self.dtype, device=self.device)
-            for g in groups
-        ]
+        # pages of a group, per cache slot: keys [page, kv head, position in page, head dim],
+        # values transposed [page, kv head, head dim, position in page]
+        self.key_pages = [
+            torch.zeros((len(g.slots), block_capacity, g.kv_heads, block_size, g.head_dim),
+                        dtype=self.dtype, device=self.device) for g in groups]
+        self.value_pages = [
+            torch.zeros((len(g.slots), block_capacity, g.kv_heads, g.head_dim, block_size),
+                        dtype=self.dtype, device=self.device) for g in groups]
         self.states: list[Tensor | None] = []
         for need in needs:
             if need.state is None:
@@ -149,7 +151,7 @@ class ModelRunner:
             if call.cache in self._where:
                 g, j = self._where[call.cache]
                 group = self.cache.groups[g]
-                views.append(CacheView(self.pages[g][j, 0], self.pages[g][j, 1], batch.block_tables[g],
+                views.append(CacheView(self.key_pages[g][j], self.value_pages[g][j], batch.block_tables[g],
                                        self.block_size, group.window, state))
             elif state is not None:
                 views.append(CacheView(state=state))

@@ -246,7 +246,8 @@ def qk_norm_rope_write(qkv: Tensor, q_weight: Tensor | None, k_weight: Tensor | 
     """Per-head RMSNorm of q and k, rotation, and the write of k, v into pages.
 
     qkv [T, (Hq + 2 Hkv) D] is changed in place (q part); pages are
-    [blocks, Hkv, block_size, D]; block_table [B, max_blocks] int32.
+    keys [blocks, Hkv, block_size, D], values transposed [blocks, Hkv, D, block_size];
+    block_table [B, max_blocks] int32.
     """
     _gpu(qkv, "qkv")
     tokens = qkv.shape[0]
@@ -271,11 +272,11 @@ def qk_norm_rope_write(qkv: Tensor, q_weight: Tensor | None, k_weight: Tensor | 
     _gpu(value_pages, "value_pages", qkv.dtype)
     if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
         raise KernelError(f"pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
-    if value_pages.shape != key_pages.shape:
-        raise KernelError("key and value pages must have one shape")
+    num_blocks, _, block_size, _ = key_pages.shape
+    if value_pages.shape != (num_blocks, kv_heads, head_dim, block_size):
+        raise KernelError(f"value pages are transposed: [blocks, {kv_heads}, {head_dim}, block_size], got {tuple(value_pages.shape)}")
     if block_table.dim() != 2:
         raise KernelError("block_table must be [sequences, max_blocks]")
-    num_blocks, _, block_size, _ = key_pages.shape
     _call("qk_rope", "fe_qk_norm_rope_write", _ptr(qkv), c_int(_code(qkv.dtype)), _ptr(q_weight),
           _ptr(k_weight), _ptr(inv_freq if rotary_dim else None), _ptr(positions), _ptr(token_seq),
           _ptr(block_table), c_int(block_table.stride(0)), _ptr(key_pages), _ptr(value_pages),
@@ -293,9 +294,9 @@ def _decode_kernel_fits(q: Tensor, head_dim: int, groups: int, block_size: int) 
 
 def decode_splits(num_decode: int, kv_heads: int, max_ctx: int) -> int:
     """Key splits per (sequence, kv head) for the decode kernel: enough blocks to
-    fill the chip, at least four 16-key tiles (one per wave) in each."""
+    fill the chip, at least four 32-key blocks of work (one per wave) in each."""
     want = -(-DECODE_TARGET_BLOCKS // max(1, num_decode * kv_heads))
-    most = max(1, -(-max_ctx // 16) // 4)
+    most = max(1, -(-max_ctx // 32) // 4)
     return max(1, min(want, most, 64))
 
 
@@ -331,8 +332,8 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
         raise KernelError(f"head size {head_dim} is not a multiple of 16 in [16, 256]")
     if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
         raise KernelError(f"pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
-    if value_pages.shape != key_pages.shape:
-        raise KernelError("key and value pages must have one shape")
+    if value_pages.shape != (key_pages.shape[0], kv_heads, head_dim, key_pages.shape[2]):
+        raise KernelError(f"value pages are transposed: [blocks, {kv_heads}, {head_dim}, block_size], got {tuple(value_pages.shape)}")
     if cu_q.numel() != num_seqs + 1 or ctx_len.numel() != num_seqs or block_table.shape[0] < num_seqs:
         raise KernelError("cu_q, ctx_len and block_table do not match the number of sequences")
     if block_table.dim() != 2 or block_table.stride(1) != 1:

@@ -106,7 +106,7 @@ def qk_norm_rope_write(qkv, q_weight, k_weight, inv_freq, positions, token_seq, 
         page = int(block_table[int(token_seq[t]), pos // block_size])
         assert page >= 0, "token without a page"
         key_pages[page, :, pos % block_size] = k[t]
-        value_pages[page, :, pos % block_size] = v[t]
+        value_pages[page, :, :, pos % block_size] = v[t]     # values are stored transposed: [D][slot]
 
 
 def gather_pages(pages, table_row, length, block_size):
@@ -134,7 +134,7 @@ def paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, 
         q_len, ctx = q1 - q0, int(ctxs[s])
         before = ctx - q_len
         keys = gather_pages(key_pages, table[s], ctx, block_size)
-        values = gather_pages(value_pages, table[s], ctx, block_size)
+        values = gather_pages(value_pages.transpose(2, 3), table[s], ctx, block_size)
         queries = q_host[q0:q1, :q_heads * head_dim].reshape(q_len, q_heads, head_dim)
         for i in range(q_len):
             pos = before + i

@@ -145,12 +145,13 @@ def test_qk_norm_rope_write(ops, dtype, q_heads, kv_heads, head_dim, block_size,
     if rotary_dim:
         inv_freq = 1.0 / (10000.0 ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
     shape = (num_blocks, kv_heads, block_size, head_dim)
-    kp_ref, vp_ref = torch.zeros(shape, dtype=dtype), torch.zeros(shape, dtype=dtype)
+    vshape = (num_blocks, kv_heads, head_dim, block_size)      # values are stored transposed
+    kp_ref, vp_ref = torch.zeros(shape, dtype=dtype), torch.zeros(vshape, dtype=dtype)
     qkv_ref = qkv.clone()
     refs.qk_norm_rope_write(qkv_ref, qw, kw, inv_freq, positions, token_seq, table, kp_ref, vp_ref,
                             q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, rotary_dim=rotary_dim, eps=1e-6)
     qkv_dev = qkv.to(DEV)
-    kp, vp = torch.zeros(shape, dtype=dtype, device=DEV), torch.zeros(shape, dtype=dtype, device=DEV)
+    kp, vp = torch.zeros(shape, dtype=dtype, device=DEV), torch.zeros(vshape, dtype=dtype, device=DEV)
     ops.qk_norm_rope_write(qkv_dev, qw.to(DEV), kw.to(DEV), None if inv_freq is None else inv_freq.to(DEV),
                            positions.to(DEV), token_seq.to(DEV), table.to(DEV), kp, vp, q_heads=q_heads,
                            kv_heads=kv_heads, head_dim=head_dim, rotary_dim=rotary_dim, eps=1e-6)
@@ -167,7 +168,7 @@ def test_rotation_sign_and_pairing_on_device(ops):
     qkv[0, 0] = 1.0          # q
     qkv[0, 5] = 1.0          # k, dim 1
     inv_freq = torch.tensor([1.0, 0.01])
-    kp, vp = torch.zeros(2, 1, 2, 4, device=DEV), torch.zeros(2, 1, 2, 4, device=DEV)
+    kp, vp = torch.zeros(2, 1, 2, 4, device=DEV), torch.zeros(2, 1, 4, 2, device=DEV)
     dev = qkv.to(DEV)
     ops.qk_norm_rope_write(dev, None, None, inv_freq.to(DEV), torch.tensor([1], dtype=torch.int32, device=DEV),
                            torch.tensor([0], dtype=torch.int32, device=DEV),
@@ -190,7 +191,7 @@ def _attention_case(g, dtype, seqs, q_heads, kv_heads, head_dim, block_size, ext
         table[s, :n] = torch.tensor(perm[at:at + n], dtype=torch.int32)
         at += n
     shape = (num_blocks, kv_heads, block_size, head_dim)
-    kp, vp = rand(g, *shape, dtype=dtype), rand(g, *shape, dtype=dtype)
+    kp, vp = rand(g, *shape, dtype=dtype), rand(g, num_blocks, kv_heads, head_dim, block_size, dtype=dtype)   # values transposed
     q = rand(g, total_q, q_heads * head_dim + extra_width, dtype=dtype)
     cu = torch.tensor([0] + list(torch.tensor([q for _, q in seqs]).cumsum(0)), dtype=torch.int32)
     ctx = torch.tensor([b + q for b, q in seqs], dtype=torch.int32)
@@ -238,7 +239,7 @@ def test_paged_attention_is_library_attention(ops):
     q, kp, vp, cu, ctx, table = _attention_case(g, torch.float32, [(0, 21)], 6, 2, 32, 8)
     got, _ = _run_attention(ops, q, kp, vp, cu, ctx, table, q_heads=6, kv_heads=2, head_dim=32)
     keys = refs.gather_pages(kp, table[0], 21, 8)
-    values = refs.gather_pages(vp, table[0], 21, 8)
+    values = refs.gather_pages(vp.transpose(2, 3), table[0], 21, 8)
     lib = torch.nn.functional.scaled_dot_product_attention(
         q.view(21, 6, 32).transpose(0, 1).unsqueeze(0), keys.repeat_interleave(3, 0).unsqueeze(0),
         values.repeat_interleave(3, 0).unsqueeze(0), is_causal=True)[0]
@@ -261,7 +262,7 @@ def test_paged_attention_far_key_stands_out(ops, dtype):
     q[0, head_dim + 3] = 40.0
     got, want = _run_attention(ops, q, kp, vp, cu, ctx, table, q_heads=2, kv_heads=1, head_dim=head_dim)
     torch.testing.assert_close(got, want, **tol(dtype))
-    torch.testing.assert_close(got[0, :head_dim], vp[page, 0, slot].float(), **tol(dtype))
+    torch.testing.assert_close(got[0, :head_dim], vp[page, 0, :, slot].float(), **tol(dtype))
 
 
 def test_argmax_rows(ops):
@@ -436,7 +437,7 @@ def test_decode_attention_far_key_and_page_edges(ops):
                                       cu.to(DEV), ctx.to(DEV), table.to(DEV), num_seqs=1, max_q_len=1, q_heads=4, kv_heads=1,
                                       head_dim=head_dim, scale=head_dim ** -0.5, num_decode=1, max_ctx=ctx_len, splits=splits).cpu().float()
             for h in range(4):
-                torch.testing.assert_close(got[0, h * head_dim:(h + 1) * head_dim], vp[page, 0, slot].float(), atol=2e-2, rtol=2e-2)
+                torch.testing.assert_close(got[0, h * head_dim:(h + 1) * head_dim], vp[page, 0, :, slot].float(), atol=2e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [
@@ -489,7 +490,7 @@ def test_prefill_attention_far_key_and_tile_edges(ops):
                                   cu.to(DEV), ctx.to(DEV), table.to(DEV), num_seqs=1, max_q_len=length, q_heads=2, kv_heads=1,
                                   head_dim=head_dim, scale=head_dim ** -0.5, num_decode=0).cpu().float()
         for h in range(2):
-            torch.testing.assert_close(got[query, h * head_dim:(h + 1) * head_dim], vp[page, 0, slot].float(), atol=2e-2, rtol=2e-2)
+            torch.testing.assert_close(got[query, h * head_dim:(h + 1) * head_dim], vp[page, 0, :, slot].float(), atol=2e-2, rtol=2e-2)
     # a key after the query must stay invisible however large its score would be
     kq = kp.clone()
     page, slot = int(table[0, 578 // block_size]), 578 % block_size
@@ -499,4 +500,4 @@ def test_prefill_attention_far_key_and_tile_edges(ops):
     got = ops.paged_attention(qq.to(DEV), kq.to(DEV), vp.to(DEV), torch.empty(length, 2 * head_dim, dtype=q.dtype, device=DEV),
                               cu.to(DEV), ctx.to(DEV), table.to(DEV), num_seqs=1, max_q_len=length, q_heads=2, kv_heads=1,
                               head_dim=head_dim, scale=head_dim ** -0.5, num_decode=0).cpu().float()
-    assert float((got[query, :head_dim] - vp[page, 0, slot].float()).abs().max()) > 0.1
+    assert float((got[query, :head_dim] - vp[page, 0, :, slot].float()).abs().max()) > 0.1
