@@ -49,6 +49,8 @@ def parse_args():
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
     parser.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
     parser.add_argument("--points", default="1,64", help="other decode batch sizes to report")
+    parser.add_argument("--phase", choices=("all", "decode", "prefill"), default="all",
+                        help="run one phase only (for profiles); the record then holds that phase alone")
     parser.add_argument("--seed", type=int, default=0)
     return parser.parse_args()
 
@@ -88,6 +90,8 @@ def main() -> int:
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
     model = random_model(config, args.seed, dtype=dtype, device=device)
     batches = sorted({args.batch, *[int(b) for b in args.points.split(",") if b]})
+    if args.phase == "decode":
+        batches = [args.batch]
     spare = args.steps + args.warmup + 8
     per_request = -(-(args.prompt_len + spare) // args.block_size)
     capacity = max(args.batch * -(-args.context // args.block_size), max(batches) * per_request,
@@ -135,7 +139,10 @@ def main() -> int:
             runner.end(name)
         return seconds, sum(contexts) / batch - args.steps / 2.0
 
-    results = {b: decode_run(b) for b in batches}
+    if args.phase == "prefill":
+        results = {}
+    else:
+        results = {b: decode_run(b) for b in batches}
 
     # prefill: one whole prompt in one step, logits at its last token
     prompt = random_tokens(args.prefill_tokens)
@@ -149,7 +156,16 @@ def main() -> int:
         sampler.sample(logits, [greedy], [0], [0])
         runner.end(name)
 
+    if args.phase == "decode":
+        seconds = results[args.batch][0]
+        print(json.dumps({"phase": "decode", "batch": args.batch, "ms_per_step": round(seconds * 1e3, 4),
+                          "value": round(args.batch / seconds, 2), "unit": "tokens/s"}))
+        return 0
     prefill_seconds = timed(prefill_once, 2, max(3, min(10, args.steps)))
+    if args.phase == "prefill":
+        print(json.dumps({"phase": "prefill", "tokens": args.prefill_tokens, "ms": round(prefill_seconds * 1e3, 3),
+                          "value": round(args.prefill_tokens / prefill_seconds, 1), "unit": "tokens/s"}))
+        return 0
 
     layers = config.num_hidden_layers
     matrix_params = layers * (config.hidden_size * (config.q_size + 2 * config.kv_size)

@@ -30,8 +30,10 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 #define WAVES 4
 #define GMAX 8           // largest group size served
 
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 __device__ __forceinline__ unsigned int pack_bf16(float lo, float hi) {
-  return (unsigned int)float_to_bf16(lo) | ((unsigned int)float_to_bf16(hi) << 16);
+  const bf16x2 v = {(__bf16)lo, (__bf16)hi};   // the hardware's round-to-nearest-even conversion
+  return __builtin_bit_cast(unsigned int, v);
 }
 
 template <int D>
@@ -40,7 +42,8 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     float* __restrict__ part_o, float* __restrict__ part_ml, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const int* __restrict__ block_table, int table_stride,
-    int kv_heads, int groups, int block_size, int num_blocks, int window, float scale_log2) {
+    int kv_heads, int groups, int block_shift, int num_blocks, int window, float scale_log2) {
+  const int block_size = 1 << block_shift, block_mask = block_size - 1;
   constexpr int KC = D / 32;        // MFMA k-steps over the head dim (scores)
   constexpr int DT = D / 16;        // 16-dim tiles of the output
   __shared__ float Ow[WAVES][GMAX][D];
@@ -82,14 +85,20 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(
   const int* table = block_table + (size_t)seq * table_stride;
   // MFMA row r of key tile h (h = 0, 1) is key 8*(r/4) + 4h + r%4 of the block
   const int krow = 8 * (lr >> 2) + (lr & 3);
+  // Page ids are read two blocks ahead and keys one block ahead, so that no load has to wait
+  // for another load: a lane needs one key page (its key rows krow, krow + 4 share it) and one
+  // value page (keys 8lq .. 8lq+7) per block.
   uintx4 ka[2][KC], ka_next[2][KC];
-  auto fetch_keys = [&](int b, uintx4 (*dst)[KC]) {
+  auto page_id = [&](int key) -> int {
+    const int id = key < ctx ? table[key >> block_shift] : -1;
+    return (id >= 0 && id < num_blocks) ? id : -1;
+  };
+  auto fetch_keys = [&](int b, int block, uintx4 (*dst)[KC]) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int key = b * KEYS + krow + 4 * h;
-      const int block = key < ctx ? table[key / block_size] : -1;
-      const bool ok = block >= 0 && block < num_blocks;
-      const bf16_t* row = key_pages + (((size_t)(ok ? block : 0) * kv_heads + hk) * block_size + key % block_size) * D;
+      const bool ok = block >= 0 && key < ctx;
+      const bf16_t* row = key_pages + ((((size_t)(ok ? block : 0) * kv_heads + hk) << block_shift) + (key & block_mask)) * D;
 #pragma unroll
       for (int c = 0; c < KC; ++c) {
         dst[h][c] = uintx4{0u, 0u, 0u, 0u};
@@ -97,8 +106,17 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(
       }
     }
   };
-  if (my_first + wave < my_last) fetch_keys(my_first + wave, ka_next);
-  for (int b = my_first + wave; b < my_last; b += WAVES) {
+  const int b0 = my_first + wave;
+  int vpage = -1, vpage_next = -1, kpage_next = -1;
+  if (b0 < my_last) {
+    vpage = page_id(b0 * KEYS + 8 * lq);
+    fetch_keys(b0, page_id(b0 * KEYS + krow), ka_next);
+    if (b0 + WAVES < my_last) {
+      kpage_next = page_id((b0 + WAVES) * KEYS + krow);
+      vpage_next = page_id((b0 + WAVES) * KEYS + 8 * lq);
+    }
+  }
+  for (int b = b0; b < my_last; b += WAVES) {
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -106,16 +124,20 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(
     // this block's values (A operand of the second product): lane (lr = dim, lq) reads the 8
     // consecutive keys 8lq .. 8lq+7 of dims 16t + lr from the transposed page
     const int vkey = b * KEYS + 8 * lq;
-    const int vblock = vkey < ctx ? table[vkey / block_size] : -1;
-    const bool v_ok = vblock >= 0 && vblock < num_blocks;
-    const bf16_t* vbase = value_pages + ((size_t)(v_ok ? vblock : 0) * kv_heads + hk) * D * block_size + vkey % block_size;
+    const bool v_ok = vpage >= 0 && vkey < ctx;
+    const bf16_t* vbase = value_pages + ((((size_t)(v_ok ? vpage : 0) * kv_heads + hk) * D) << block_shift) + (vkey & block_mask);
     uintx4 va[DT];
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
       va[t] = uintx4{0u, 0u, 0u, 0u};
-      if (v_ok) va[t] = *(const uintx4*)(vbase + (size_t)(t * 16 + lr) * block_size);
+      if (v_ok) va[t] = *(const uintx4*)(vbase + ((size_t)(t * 16 + lr) << block_shift));
     }
-    if (b + WAVES < my_last) fetch_keys(b + WAVES, ka_next);   // flies while this block is worked on
+    if (b + WAVES < my_last) fetch_keys(b + WAVES, kpage_next, ka_next);   // flies while this block is worked on
+    vpage = vpage_next;
+    if (b + 2 * WAVES < my_last) {
+      kpage_next = page_id((b + 2 * WAVES) * KEYS + krow);
+      vpage_next = page_id((b + 2 * WAVES) * KEYS + 8 * lq);
+    }
 
     floatx4 st[2];
 #pragma unroll
@@ -233,8 +255,8 @@ __global__ __launch_bounds__(256) void paged_decode_merge_kernel(
 }
 
 // Sequences with one query token only; others are left untouched.  Pages: keys
-// [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size].
-// splits > 1 (at most 64) needs part_o [num_seqs * kv_heads * splits * groups * head_dim] and
+// [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size];
+// block_size a power of two >= 16.  splits > 1 (at most 64) needs part_o [num_seqs * kv_heads * splits * groups * head_dim] and
 // part_ml [num_seqs * kv_heads * splits * groups * 2] floats.
 extern "C" int fe_paged_attention_decode(const void* q, long long q_stride, const void* key_pages,
                                          const void* value_pages, void* out, long long out_stride,
@@ -246,7 +268,9 @@ extern "C" int fe_paged_attention_decode(const void* q, long long q_stride, cons
   if (num_seqs <= 0) return FE_OK;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256) return FE_BAD_ARGUMENT;
   if (groups < 1 || groups > GMAX || kv_heads < 1 || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
-  if (block_size < 16 || block_size % 16 || num_blocks < 1 || table_stride < 1) return FE_BAD_ARGUMENT;
+  if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1) return FE_BAD_ARGUMENT;
+  int block_shift = 0;
+  while ((1 << block_shift) < block_size) ++block_shift;
   if (q_stride % 8 || splits < 1 || splits > 64) return FE_BAD_ARGUMENT;
   if (splits > 1 && (!part_o || !part_ml)) return FE_BAD_ARGUMENT;
   dim3 grid(splits, kv_heads, num_seqs);
@@ -254,7 +278,7 @@ extern "C" int fe_paged_attention_decode(const void* q, long long q_stride, cons
 #define FE_GO(DD)                                                                                          \
   paged_decode_kernel<DD><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages,    \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, cu_q, ctx_len, block_table,     \
-      table_stride, kv_heads, groups, block_size, num_blocks, window, scale_log2)
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2)
   if (head_dim == 64) FE_GO(64);
   else if (head_dim == 128) FE_GO(128);
   else FE_GO(256);

@@ -38,8 +38,10 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 #define VPAD 8       // bf16 padding of a value row (one dim, 64 keys) in LDS
 #define XCDS 8
 
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 __device__ __forceinline__ unsigned int pack_bf16(float lo, float hi) {
-  return (unsigned int)float_to_bf16(lo) | ((unsigned int)float_to_bf16(hi) << 16);
+  const bf16x2 v = {(__bf16)lo, (__bf16)hi};   // the hardware's round-to-nearest-even conversion
+  return __builtin_bit_cast(unsigned int, v);
 }
 
 template <int D, int RT>
@@ -47,8 +49,9 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
-    int table_stride, int kv_heads, int groups, int block_size, int num_blocks, int window,
+    int table_stride, int kv_heads, int groups, int block_shift, int num_blocks, int window,
     float scale_log2, int q_tiles, int items_per_xcd, int total_items) {
+  const int block_size = 1 << block_shift, block_mask = block_size - 1;
   constexpr int BM = 64 * RT;     // query rows per block
   constexpr int KC = D / 32;      // MFMA k-steps over the head dim (scores)
   constexpr int DT = D / 16;      // 16-dim tiles of the output
@@ -109,29 +112,46 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
   // loaders: keys piece p -> (key p / CH, 16 bytes p % CH); values piece p -> (dim p / 8, the 8
   // keys (p % 8) * 8 .. of the tile), read from the transposed page of those keys
   constexpr int LOADS = BN * CH / 256;
+  constexpr int MAXP = BN / 16;              // a tile spans at most this many pages
   uintx4 kreg[LOADS], vreg[LOADS];
+  int page_ids[MAXP];                        // pages of the tile that load_tile reads next
+  const int pages_per_tile = BN >> block_shift > 0 ? BN >> block_shift : 1;
+  auto load_pages = [&](int tile) {          // uniform addresses: scalar loads
+#pragma unroll
+    for (int j = 0; j < MAXP; ++j) {
+      const int key = tile * BN + (j << block_shift);
+      int id = -1;
+      if (j < pages_per_tile && key < ctx) id = table[key >> block_shift];
+      page_ids[j] = (id >= 0 && id < num_blocks) ? id : -1;
+    }
+  };
+  auto page_of = [&](int key_in_tile) -> int {
+    const int j = key_in_tile >> block_shift;
+    int id = page_ids[0];
+#pragma unroll
+    for (int k = 1; k < MAXP; ++k) id = j == k ? page_ids[k] : id;
+    return id;
+  };
   auto load_tile = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int p = tid + i * 256;
       {
-        const int key = tile * BN + p / CH;
+        const int kk = p / CH;
+        const int key = tile * BN + kk;
+        const int block = page_of(kk);
         uintx4 v = uintx4{0u, 0u, 0u, 0u};
-        if (key < ctx) {
-          const int block = table[key / block_size];
-          if (block >= 0 && block < num_blocks)
-            v = *(const uintx4*)(key_pages + (((size_t)block * kv_heads + hk) * block_size + key % block_size) * D + (p % CH) * 8);
-        }
+        if (block >= 0 && key < ctx)
+          v = *(const uintx4*)(key_pages + ((((size_t)block * kv_heads + hk) << block_shift) + (key & block_mask)) * D + (p % CH) * 8);
         kreg[i] = v;
       }
       {
-        const int key = tile * BN + (p % 8) * 8;
+        const int kk = (p % 8) * 8;
+        const int key = tile * BN + kk;
+        const int block = page_of(kk);
         uintx4 v = uintx4{0u, 0u, 0u, 0u};
-        if (key < ctx) {
-          const int block = table[key / block_size];
-          if (block >= 0 && block < num_blocks)
-            v = *(const uintx4*)(value_pages + (((size_t)block * kv_heads + hk) * D + p / 8) * block_size + key % block_size);
-        }
+        if (block >= 0 && key < ctx)
+          v = *(const uintx4*)(value_pages + ((((size_t)block * kv_heads + hk) * D + p / 8) << block_shift) + (key & block_mask));
         vreg[i] = v;
       }
     }
@@ -146,15 +166,20 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
   };
 
   const int krow = 8 * (lr >> 2) + (lr & 3);   // MFMA row r of key tile h is key 8*(r/4) + 4h + r%4 of its 32-key block
+  load_pages(tile_first);
   load_tile(tile_first);
+  if (tile_first < tile_last) load_pages(tile_first + 1);
   for (int tile = tile_first; tile <= tile_last; ++tile) {
     __syncthreads();            // the previous tile's LDS reads are done
     store_tile();
     __syncthreads();
-    if (tile < tile_last) load_tile(tile + 1);   // flies while this tile multiplies
+    if (tile < tile_last) {
+      load_tile(tile + 1);                       // flies while this tile multiplies
+      if (tile + 1 < tile_last) load_pages(tile + 2);
+    }
 
     const int key_base = tile * BN;
-    if (key_base > wave_lo + RT * 16 - 1 && window <= 0) continue;   // every key of the tile lies after this wave's rows
+    if (key_base > wave_lo + RT * 16 - 1) continue;   // every key of the tile lies after this wave's rows
     floatx4 st[RT][2][2];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
@@ -246,19 +271,25 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
   }
 }
 
-// Pages: keys [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size].
+// Pages: keys [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size];
+// block_size a power of two >= 16.  rows_per_block: 0 (the default, 64), 64 or 128.
 extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, const void* key_pages,
                                           const void* value_pages, void* out, long long out_stride,
                                           const int* cu_q, const int* ctx_len, const int* block_table,
                                           int table_stride, int num_seqs, int max_q_len, int kv_heads,
                                           int groups, int head_dim, int block_size, int num_blocks,
-                                          int window, float scale, hipStream_t stream) {
+                                          int window, float scale, int rows_per_block,
+                                          hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len < 2) return FE_OK;
   if (head_dim != 64 && head_dim != 128) return FE_BAD_ARGUMENT;
   if (groups < 1 || kv_heads < 1 || num_seqs > 65535) return FE_BAD_ARGUMENT;
-  if (block_size < 16 || block_size % 16 || num_blocks < 1 || table_stride < 1 || q_stride % 8 || out_stride % 4) return FE_BAD_ARGUMENT;
+  if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1 || q_stride % 8 || out_stride % 4) return FE_BAD_ARGUMENT;
   const float scale_log2 = scale * 1.4426950408889634f;
-  const int rt = max_q_len >= 512 ? 2 : 1;       // long portions: 128-row blocks halve the reads of keys and values
+  if (rows_per_block != 0 && rows_per_block != 64 && rows_per_block != 128) return FE_BAD_ARGUMENT;
+  // long portions: 128-row blocks halve the reads of keys and values
+  const int rt = rows_per_block ? rows_per_block / 64 : 1;   // 64-row blocks keep two blocks on a unit
+  int block_shift = 0;
+  while ((1 << block_shift) < block_size) ++block_shift;
   const int q_tiles = (max_q_len + 64 * rt - 1) / (64 * rt);
   const long long items = (long long)num_seqs * kv_heads * groups * q_tiles;
   const long long per_xcd = (items + XCDS - 1) / XCDS;
@@ -267,7 +298,7 @@ extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, con
 #define FE_GO(DD, RR)                                                                                        \
   paged_prefill_kernel<DD, RR><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,          \
-      kv_heads, groups, block_size, num_blocks, window, scale_log2, q_tiles, (int)per_xcd, (int)items)
+      kv_heads, groups, block_shift, num_blocks, window, scale_log2, q_tiles, (int)per_xcd, (int)items)
   if (head_dim == 64) { if (rt == 2) FE_GO(64, 2); else FE_GO(64, 1); }
   else { if (rt == 2) FE_GO(128, 2); else FE_GO(128, 1); }
 #undef FE_GO

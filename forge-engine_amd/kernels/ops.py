@@ -287,11 +287,6 @@ def qk_norm_rope_write(qkv: Tensor, q_weight: Tensor | None, k_weight: Tensor | 
 DECODE_TARGET_BLOCKS = 512   # blocks the decode attention kernel aims at (key splits fill the chip)
 
 
-def _decode_kernel_fits(q: Tensor, head_dim: int, groups: int, block_size: int) -> bool:
-    return (q.dtype == torch.bfloat16 and head_dim in (64, 128, 256) and groups <= 8
-            and block_size % 16 == 0)
-
-
 def decode_splits(num_decode: int, kv_heads: int, max_ctx: int) -> int:
     """Key splits per (sequence, kv head) for the decode kernel: enough blocks to
     fill the chip, at least four 32-key blocks of work (one per wave) in each."""
@@ -304,7 +299,7 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                     ctx_len: Tensor, block_table: Tensor, *, num_seqs: int, max_q_len: int,
                     q_heads: int, kv_heads: int, head_dim: int, scale: float,
                     window: int | None = None, num_decode: int | None = None,
-                    max_ctx: int | None = None, splits: int | None = None) -> Tensor:
+                    max_ctx: int | None = None, splits: int | None = None, prefill_rows: int = 0) -> Tensor:
     """Attention of every query token of a mixed batch over its paged keys.
 
     q: [T, >= Hq*D] (row stride may exceed Hq*D: the q part of a fused qkv
@@ -347,7 +342,7 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
         any_single, any_longer, num_decode = True, max_q_len > 1, num_seqs
     else:
         any_single, any_longer = num_decode > 0, num_decode < num_seqs
-    bf16_pages = q.dtype == torch.bfloat16 and block_size % 16 == 0
+    bf16_pages = q.dtype == torch.bfloat16 and block_size >= 16 and block_size & (block_size - 1) == 0
     fast_decode = bf16_pages and head_dim in (64, 128, 256) and groups <= 8
     fast_prefill = bf16_pages and head_dim in (64, 128)
 
@@ -376,7 +371,7 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
               _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
               c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), c_float(scale), _stream())
+              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(prefill_rows), _stream())
     # whatever the two fast kernels did not take goes to the general kernel
     single_left = any_single and not fast_decode
     longer_left = any_longer and not fast_prefill
