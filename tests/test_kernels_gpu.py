@@ -371,6 +371,41 @@ def test_gemm_skinny_swiglu(ops, m, inter, k):
     torch.testing.assert_close(routed, want, atol=1e-2 * float(want.abs().max()) + 1e-6, rtol=1e-2)
 
 
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("n,k", [(8200, 264), (9003, 1000), (8209, 2560), (8195, 4096)])
+def test_gemm_skinny_resident(ops, m, n, k):
+    """Weights with more than 512 row tiles take the variant whose blocks stay and keep x in
+    registers: same bits as the one-tile-per-block kernel, also for the gated product."""
+    g = torch.Generator().manual_seed(23)
+    x = rand(g, m, k, dtype=torch.bfloat16).to(DEV)
+    w = rand(g, n, k, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    want = x.float().cpu() @ w.float().cpu().T
+    plain = ops.gemm_skinny(x, w, "f32", tiles=1, waves=8).cpu()
+    bound = 2e-6 * float(want.abs().max()) * math.sqrt(k) + 1e-6
+    assert float((plain - want).abs().max()) <= bound
+    assert torch.equal(ops.gemm_skinny(x, w, "f32", tiles=-1).cpu(), plain)
+    assert torch.equal(ops.gemm_skinny(x, w, "f32").cpu(), plain)
+    assert torch.equal(ops.gemm_skinny(x, w, "bf16").cpu(), ops.gemm_skinny(x, w, "bf16", tiles=1, waves=8).cpu())
+    if n % 2:
+        w = w[:n - 1]
+    gated = ops.gemm_skinny(x, w, "swiglu", tiles=-1).cpu()
+    assert torch.equal(gated, ops.gemm_skinny(x, w, "swiglu", tiles=1, waves=8).cpu())
+    want = refs.linear_swiglu(x.cpu(), w.cpu()).float()
+    torch.testing.assert_close(gated.float(), want, atol=1e-2 * float(want.abs().max()) + 1e-6, rtol=1e-2)
+
+
+def test_gemm_skinny_resident_refuses(ops):
+    from forge_engine_amd.kernels.ops import KernelError
+    x = torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelError):
+        ops.gemm_skinny(x, w, "f32", tiles=-1)          # more than 16 rows
+    x = torch.zeros(4, 4104, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 4104, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelError):
+        ops.gemm_skinny(x, w, "f32", tiles=-1)          # K beyond what the registers hold
+
+
 def test_linear_routes_by_rows_and_dtype(ops):
     g = torch.Generator().manual_seed(22)
     w = rand(g, 136, 200, dtype=torch.bfloat16, scale=0.05)
