@@ -88,56 +88,43 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(
   // Page ids are read two blocks ahead and keys one block ahead, so that no load has to wait
   // for another load: a lane needs one key page (its key rows krow, krow + 4 share it) and one
   // value page (keys 8lq .. 8lq+7) per block.
-  uintx4 ka[2][KC], ka_next[2][KC];
-  auto page_id = [&](int key) -> int {
-    const int id = key < ctx ? table[key >> block_shift] : -1;
-    return (id >= 0 && id < num_blocks) ? id : -1;
-  };
+  // Every load below is unconditional (out-of-range keys read a valid address and are masked
+  // afterwards), so the loop body is straight-line code and the loads stay where they are issued.
+  const int table_last = table_stride - 1;
+  // Raw table entries are loaded two blocks ahead and checked only where they are used, so that
+  // nothing waits for them while the block's own loads are in flight.
+  auto raw_page = [&](int key) -> int { return table[min(key >> block_shift, table_last)]; };
+  auto checked = [&](int id, int key) -> int { return (key < ctx && id >= 0 && id < num_blocks) ? id : 0; };
   auto fetch_keys = [&](int b, int block, uintx4 (*dst)[KC]) {
+    const bool mine = b < my_last;      // past this block's share: read page 0 again (cached) instead
+    block = mine ? block : 0;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const int key = b * KEYS + krow + 4 * h;
-      const bool ok = block >= 0 && key < ctx;
-      const bf16_t* row = key_pages + ((((size_t)(ok ? block : 0) * kv_heads + hk) << block_shift) + (key & block_mask)) * D;
+      const int key = mine ? b * KEYS + krow + 4 * h : krow + 4 * h;
+      const bf16_t* row = key_pages + ((((size_t)block * kv_heads + hk) << block_shift) + (key & block_mask)) * D;
 #pragma unroll
-      for (int c = 0; c < KC; ++c) {
-        dst[h][c] = uintx4{0u, 0u, 0u, 0u};
-        if (ok) dst[h][c] = *(const uintx4*)(row + c * 32 + lq * 8);
-      }
+      for (int c = 0; c < KC; ++c) dst[h][c] = *(const uintx4*)(row + c * 32 + lq * 8);
     }
   };
-  const int b0 = my_first + wave;
-  int vpage = -1, vpage_next = -1, kpage_next = -1;
-  if (b0 < my_last) {
-    vpage = page_id(b0 * KEYS + 8 * lq);
-    fetch_keys(b0, page_id(b0 * KEYS + krow), ka_next);
-    if (b0 + WAVES < my_last) {
-      kpage_next = page_id((b0 + WAVES) * KEYS + krow);
-      vpage_next = page_id((b0 + WAVES) * KEYS + 8 * lq);
-    }
-  }
-  for (int b = b0; b < my_last; b += WAVES) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int c = 0; c < KC; ++c) ka[h][c] = ka_next[h][c];
-    // this block's values (A operand of the second product): lane (lr = dim, lq) reads the 8
-    // consecutive keys 8lq .. 8lq+7 of dims 16t + lr from the transposed page
+  // One block of 32 keys: its keys are in kcur (loaded a step ago), vraw is its value page; the
+  // step issues its value loads, then the next block's key loads into knext (page knext_raw) and
+  // the raw page ids of the block after that (into vraw and knext_raw2).  Two steps alternate the
+  // roles of the register sets, so nothing is copied.
+  auto step = [&](int b, uintx4 (*kcur)[KC], uintx4 (*knext)[KC], int& vraw, int knext_raw, int& knext_raw2) {
+    // values (A operand of the second product): lane (lr = dim, lq) reads the 8 consecutive keys
+    // 8lq .. 8lq+7 of dims 16t + lr from the transposed page
     const int vkey = b * KEYS + 8 * lq;
-    const bool v_ok = vpage >= 0 && vkey < ctx;
-    const bf16_t* vbase = value_pages + ((((size_t)(v_ok ? vpage : 0) * kv_heads + hk) * D) << block_shift) + (vkey & block_mask);
+    const bool v_ok = vkey < ctx;
+    const int vpage = checked(vraw, vkey);
+    const bf16_t* vbase = value_pages + ((((size_t)vpage * kv_heads + hk) * D) << block_shift) + (vkey & block_mask);
     uintx4 va[DT];
 #pragma unroll
-    for (int t = 0; t < DT; ++t) {
-      va[t] = uintx4{0u, 0u, 0u, 0u};
-      if (v_ok) va[t] = *(const uintx4*)(vbase + ((size_t)(t * 16 + lr) << block_shift));
-    }
-    if (b + WAVES < my_last) fetch_keys(b + WAVES, kpage_next, ka_next);   // flies while this block is worked on
-    vpage = vpage_next;
-    if (b + 2 * WAVES < my_last) {
-      kpage_next = page_id((b + 2 * WAVES) * KEYS + krow);
-      vpage_next = page_id((b + 2 * WAVES) * KEYS + 8 * lq);
-    }
+    for (int t = 0; t < DT; ++t) va[t] = *(const uintx4*)(vbase + ((size_t)(t * 16 + lr) << block_shift));
+    __builtin_amdgcn_sched_barrier(0);
+    fetch_keys(b + WAVES, checked(knext_raw, (b + WAVES) * KEYS + krow), knext);
+    vraw = raw_page((b + 2 * WAVES) * KEYS + 8 * lq);
+    knext_raw2 = raw_page((b + 2 * WAVES) * KEYS + krow);
+    __builtin_amdgcn_sched_barrier(0);
 
     floatx4 st[2];
 #pragma unroll
@@ -145,7 +132,7 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(
       st[h] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < KC; ++c)
-        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[h][c]), qb[c], st[h], 0, 0, 0);
+        st[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kcur[h][c]), qb[c], st[h], 0, 0, 0);
     }
     // lane (lr = query row, lq): st[h][i] = score of key b*32 + 8lq + 4h + i
     float s[8];
@@ -180,8 +167,24 @@ __global__ __launch_bounds__(256) void paged_decode_kernel(
     for (int t = 0; t < DT; ++t) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[t][i] *= corr;
-      o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, va[t]), pb, o[t], 0, 0, 0);
+      const uintx4 vt = v_ok ? va[t] : uintx4{0u, 0u, 0u, 0u};
+      o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vt), pb, o[t], 0, 0, 0);
     }
+  };
+
+  uintx4 k0[2][KC], k1[2][KC];
+  const int b0 = my_first + wave;
+  int v0 = 0, v1 = 0, kr0 = 0, kr1 = 0;      // raw page ids: values of this / the next block, keys of the next two
+  if (b0 < my_last) {
+    v0 = raw_page(b0 * KEYS + 8 * lq);
+    fetch_keys(b0, checked(raw_page(b0 * KEYS + krow), b0 * KEYS + krow), k0);
+    kr1 = raw_page((b0 + WAVES) * KEYS + krow);
+    v1 = raw_page((b0 + WAVES) * KEYS + 8 * lq);
+  }
+  for (int b = b0; b < my_last; b += 2 * WAVES) {
+    step(b, k0, k1, v0, kr1, kr0);
+    if (b + WAVES >= my_last) break;
+    step(b + WAVES, k1, k0, v1, kr0, kr1);
   }
 
   // lane (lr = query row, lq) holds O^T[16t + 4lq + i][lr]; the four waves meet in LDS

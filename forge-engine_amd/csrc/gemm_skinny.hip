@@ -44,9 +44,11 @@ struct StepRegs {
 // tiles), WAVES waves per block sharing K.
 template <int MT, int NT, int EPI, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
-    int K, long long ldw, long long ldo, int second_offset) {
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out_base, int M, int N,
+    int K, long long ldw, long long ldo, int second_offset, int steps_per_split, long long part_stride) {
   constexpr int NW = EPI == EPI_SWIGLU ? 2 * NT : NT;   // weight tiles per wave
+  // blockIdx.y: which part of K this block sums (float32 epilogue only); its sums go to a part of their own
+  void* out = EPI == EPI_F32 ? (void*)((float*)out_base + (size_t)blockIdx.y * part_stride) : out_base;
   __shared__ __attribute__((aligned(16))) float red[WAVES][64][4];
 
   const int tid = threadIdx.x;
@@ -112,9 +114,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
   };
 
   // steps wave, wave + WAVES, ...: two register sets, the next step's loads fly while this one multiplies
-  const int steps = (K + KSTEP - 1) / KSTEP;
+  const int all_steps = (K + KSTEP - 1) / KSTEP;
+  const int first_step = blockIdx.y * steps_per_split;
+  const int steps = min(all_steps, first_step + steps_per_split);
   StepRegs<MT, NW> ra, rb;
-  int step = wave;
+  int step = first_step + wave;
   if (step < steps) load(ra, step);
   while (step < steps) {
     const int next = step + WAVES;
@@ -161,12 +165,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     }
 }
 
+struct SkinnyCall {
+  const void* x;
+  const void* w;
+  void* out;
+  int M, N, K;
+  long long ldw, ldo;
+  int second_offset;      // rows between a gate row and its up row
+  int splits;             // parts of K, each summed by blocks of its own (float32 epilogue)
+  long long part_stride;  // floats between the parts' outputs
+  hipStream_t stream;
+};
+
 template <int MT, int NT, int EPI, int WAVES>
-static int launch_skinny(const void* x, const void* w, void* out, int M, int N, int K, long long ldw,
-                         long long ldo, int second_offset, hipStream_t stream) {
-  const int blocks = (N + ROWS * NT - 1) / (ROWS * NT);
-  gemm_skinny_kernel<MT, NT, EPI, WAVES><<<blocks, WAVES * 64, 0, stream>>>(
-      (const bf16_t*)x, (const bf16_t*)w, out, M, N, K, ldw, ldo, second_offset);
+static int launch_skinny(const SkinnyCall& c) {
+  const int blocks = (c.N + ROWS * NT - 1) / (ROWS * NT);
+  const int steps = (c.K + KSTEP - 1) / KSTEP;
+  const int splits = EPI == EPI_F32 ? c.splits : 1;
+  const int per_split = (steps + splits - 1) / splits;
+  gemm_skinny_kernel<MT, NT, EPI, WAVES><<<dim3(blocks, splits), WAVES * 64, 0, c.stream>>>(
+      (const bf16_t*)c.x, (const bf16_t*)c.w, c.out, c.M, c.N, c.K, c.ldw, c.ldo, c.second_offset, per_split,
+      c.part_stride);
   return fe_check_launch();
 }
 
@@ -296,35 +315,32 @@ static int clamp_tiles(int mt, int epilogue, int tiles) {
 }
 
 template <int MT, int NT, int EPI>
-static int dispatch_waves(int waves, const void* x, const void* w, void* out, int M, int N, int K,
-                          long long ldw, long long ldo, int second_offset, hipStream_t stream) {
+static int dispatch_waves(int waves, const SkinnyCall& c) {
   constexpr int WT = NT * (EPI == EPI_SWIGLU ? 2 : 1);
   if constexpr (shape_fits(MT, WT, 16)) {
-    if (waves == 16) return launch_skinny<MT, NT, EPI, 16>(x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+    if (waves == 16) return launch_skinny<MT, NT, EPI, 16>(c);
   }
-  if (waves >= 8) return launch_skinny<MT, NT, EPI, 8>(x, w, out, M, N, K, ldw, ldo, second_offset, stream);
-  return launch_skinny<MT, NT, EPI, 4>(x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+  if (waves >= 8) return launch_skinny<MT, NT, EPI, 8>(c);
+  return launch_skinny<MT, NT, EPI, 4>(c);
 }
 
 template <int MT, int EPI>
-static int dispatch_tiles(int nt, int waves, const void* x, const void* w, void* out, int M, int N, int K,
-                          long long ldw, long long ldo, int second_offset, hipStream_t stream) {
+static int dispatch_tiles(int nt, int waves, const SkinnyCall& c) {
   constexpr int PAIR = EPI == EPI_SWIGLU ? 2 : 1;
   if constexpr (shape_fits(MT, 4 * PAIR, 8)) {
-    if (nt == 4) return dispatch_waves<MT, 4, EPI>(waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+    if (nt == 4) return dispatch_waves<MT, 4, EPI>(waves, c);
   }
   if constexpr (shape_fits(MT, 2 * PAIR, 8)) {
-    if (nt >= 2) return dispatch_waves<MT, 2, EPI>(waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+    if (nt >= 2) return dispatch_waves<MT, 2, EPI>(waves, c);
   }
-  return dispatch_waves<MT, 1, EPI>(waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+  return dispatch_waves<MT, 1, EPI>(waves, c);
 }
 
 template <int EPI>
-static int dispatch(int mt, int nt, int waves, const void* x, const void* w, void* out, int M, int N,
-                    int K, long long ldw, long long ldo, int second_offset, hipStream_t stream) {
-  if (mt == 1) return dispatch_tiles<1, EPI>(nt, waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
-  if (mt == 2) return dispatch_tiles<2, EPI>(nt, waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
-  return dispatch_tiles<4, EPI>(nt, waves, x, w, out, M, N, K, ldw, ldo, second_offset, stream);
+static int dispatch(int mt, int nt, int waves, const SkinnyCall& c) {
+  if (mt == 1) return dispatch_tiles<1, EPI>(nt, waves, c);
+  if (mt == 2) return dispatch_tiles<2, EPI>(nt, waves, c);
+  return dispatch_tiles<4, EPI>(nt, waves, c);
 }
 
 // x [M, K] bf16 contiguous; w [N, K] (epilogue 0, 1) or [2N, K] with the gate
@@ -333,18 +349,23 @@ static int dispatch(int mt, int nt, int waves, const void* x, const void* w, voi
 // 16-row tiles a wave takes (1, 2, 4: more tiles share each read of x) and how
 // many waves share a block's K (4, 8, 16), aiming at a few thousand waves.  tiles -1 asks for
 // the resident variant (refused where it does not apply); 0 uses it wherever it applies.
+// splits > 1 (float32 epilogue, at most 16): K is cut into that many parts of whole 128-steps,
+// each summed by blocks of its own into out + part * part_stride; the caller adds the parts up
+// (in a fixed order, so the result stays deterministic).
 extern "C" int fe_gemm_skinny(const void* x, const void* w, void* out, int M, int N, int K,
                               long long ldw, long long ldo, int epilogue, int tiles, int waves,
-                              hipStream_t stream) {
+                              int splits, long long part_stride, hipStream_t stream) {
   if (M < 1) return FE_OK;
+  if (splits < 1 || splits > 16 || (splits > 1 && (epilogue != EPI_F32 || part_stride < (long long)M * ldo)))
+    return FE_BAD_ARGUMENT;
   if (M > 64 || N < 1 || K < 8 || K % 8 || ldw < K || ldw % 8 || ldo < N) return FE_BAD_ARGUMENT;
   if ((((uintptr_t)x) & 15) || (((uintptr_t)w) & 15)) return FE_BAD_ARGUMENT;
   if (epilogue < 0 || epilogue > 2) return FE_BAD_ARGUMENT;
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   const int steps = (K + KSTEP - 1) / KSTEP;
   const int weight_rows = epilogue == EPI_SWIGLU ? 2 * N : N;
-  if (tiles == -1 || (tiles == 0 && waves == 0 && resident_fits(M, N, K))) {
-    if (M > 16 || steps > 4 * RESIDENT_WAVES) return FE_BAD_ARGUMENT;
+  if (tiles == -1 || (tiles == 0 && waves == 0 && splits == 1 && resident_fits(M, N, K))) {
+    if (M > 16 || steps > 4 * RESIDENT_WAVES || splits != 1) return FE_BAD_ARGUMENT;
     if (epilogue == EPI_SWIGLU) return launch_resident<EPI_SWIGLU>(x, w, out, M, N, K, ldw, ldo, N, stream);
     if (epilogue == EPI_F32) return launch_resident<EPI_F32>(x, w, out, M, N, K, ldw, ldo, 0, stream);
     return launch_resident<EPI_BF16>(x, w, out, M, N, K, ldw, ldo, 0, stream);
@@ -359,11 +380,12 @@ extern "C" int fe_gemm_skinny(const void* x, const void* w, void* out, int M, in
   tiles = clamp_tiles(mt, epilogue, tiles);
   if (waves == 0) {
     waves = 8;
-    while (waves > 4 && waves > steps) waves >>= 1;
+    while (waves > 4 && waves > (steps + splits - 1) / splits) waves >>= 1;
   }
   if (waves != 4 && waves != 8 && waves != 16) return FE_BAD_ARGUMENT;
   if (waves == 16 && !shape_fits(mt, tiles * (epilogue == EPI_SWIGLU ? 2 : 1), 16)) waves = 8;
-  if (epilogue == EPI_SWIGLU) return dispatch<EPI_SWIGLU>(mt, tiles, waves, x, w, out, M, N, K, ldw, ldo, N, stream);
-  if (epilogue == EPI_F32) return dispatch<EPI_F32>(mt, tiles, waves, x, w, out, M, N, K, ldw, ldo, 0, stream);
-  return dispatch<EPI_BF16>(mt, tiles, waves, x, w, out, M, N, K, ldw, ldo, 0, stream);
+  const SkinnyCall call = {x, w, out, M, N, K, ldw, ldo, epilogue == EPI_SWIGLU ? N : 0, splits, part_stride, stream};
+  if (epilogue == EPI_SWIGLU) return dispatch<EPI_SWIGLU>(mt, tiles, waves, call);
+  if (epilogue == EPI_F32) return dispatch<EPI_F32>(mt, tiles, waves, call);
+  return dispatch<EPI_BF16>(mt, tiles, waves, call);
 }

@@ -173,11 +173,14 @@ def _skinny_fits(x: Tensor, weight: Tensor, rows: int = SKINNY_MAX_ROWS) -> bool
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(x: Tensor, weight: Tensor, epilogue: str = "bf16", tiles: int = 0, waves: int = 0) -> Tensor:
+def gemm_skinny(x: Tensor, weight: Tensor, epilogue: str = "bf16", tiles: int = 0, waves: int = 0,
+                splits: int = 1) -> Tensor:
     """y = x @ weight^T for up to 64 rows of bfloat16 x, float32 accumulation.
 
     epilogue ``f32``/``bf16``: y [M, N] in that dtype; ``swiglu``: weight is
-    [2I, K] with the gate rows first and y = silu(x Wg^T) * (x Wu^T) in bfloat16."""
+    [2I, K] with the gate rows first and y = silu(x Wg^T) * (x Wu^T) in bfloat16.
+    ``splits`` > 1 (``f32`` only): K is summed in that many parts by blocks of their own
+    and the result is the parts [splits, M, N], to be added up by the consumer."""
     _gpu(x, "x", torch.bfloat16)
     _gpu(weight, "weight", torch.bfloat16, contiguous=False)
     if not _skinny_fits(x, weight, SKINNY_KERNEL_ROWS):
@@ -190,9 +193,13 @@ def gemm_skinny(x: Tensor, weight: Tensor, epilogue: str = "bf16", tiles: int = 
     if code == _EPI_SWIGLU and rows % 2:
         raise KernelError("a gated weight needs an even number of rows")
     n = rows // 2 if code == _EPI_SWIGLU else rows
-    out = torch.empty((m, n), dtype=torch.float32 if code == _EPI_F32 else torch.bfloat16, device=x.device)
+    if splits != 1 and (code != _EPI_F32 or not 1 <= splits <= 16):
+        raise KernelError("parts of K need the float32 epilogue and at most 16 parts")
+    shape = (m, n) if splits == 1 else (splits, m, n)
+    out = torch.empty(shape, dtype=torch.float32 if code == _EPI_F32 else torch.bfloat16, device=x.device)
     _call("gemm_skinny", "fe_gemm_skinny", _ptr(x), _ptr(weight), _ptr(out), c_int(m), c_int(n), c_int(k),
-          c_longlong(weight.stride(0)), c_longlong(n), c_int(code), c_int(tiles), c_int(waves), _stream())
+          c_longlong(weight.stride(0)), c_longlong(n), c_int(code), c_int(tiles), c_int(waves), c_int(splits),
+          c_longlong(m * n), _stream())
     return out
 
 
