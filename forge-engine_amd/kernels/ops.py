@@ -294,6 +294,20 @@ def qk_norm_rope_write(qkv: Tensor, q_weight: Tensor | None, k_weight: Tensor | 
 DECODE_TARGET_BLOCKS = 512   # blocks the decode attention kernel aims at (key splits fill the chip)
 
 
+_SPLIT_COUNTERS: dict = {}
+
+
+def _split_counters(device, count: int) -> Tensor:
+    """Arrival counters of the decode kernel's key splits, one per (sequence, kv head): zero
+    between launches (the kernel leaves them so), shared by all launches of a device's stream."""
+    key = (device.type, device.index)
+    have = _SPLIT_COUNTERS.get(key)
+    if have is None or have.numel() < count:
+        have = torch.zeros(max(count, 4096), dtype=torch.int32, device=device)
+        _SPLIT_COUNTERS[key] = have
+    return have
+
+
 def decode_splits(num_decode: int, kv_heads: int, max_ctx: int) -> int:
     """Key splits per (sequence, kv head) for the decode kernel: enough blocks to
     fill the chip, at least four 32-key blocks of work (one per wave) in each."""
@@ -364,13 +378,14 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
     if any_single and fast_decode:
         if splits is None:
             splits = decode_splits(num_decode, kv_heads, max_ctx if max_ctx is not None else 16 * 4 * 8)
-        part_o = part_ml = None
+        part_o = part_ml = counters = None
         if splits > 1:
             part_o = torch.empty(num_seqs * kv_heads * splits * groups * head_dim, dtype=torch.float32, device=q.device)
             part_ml = torch.empty(num_seqs * kv_heads * splits * groups * 2, dtype=torch.float32, device=q.device)
+            counters = _split_counters(q.device, num_seqs * kv_heads)
         _call("attention_decode", "fe_paged_attention_decode", _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(part_o),
-              _ptr(part_ml), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)),
+              _ptr(part_ml), _ptr(counters), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)),
               c_int(num_seqs), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
               c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(splits), _stream())
     if any_longer and fast_prefill:

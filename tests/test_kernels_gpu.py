@@ -439,6 +439,18 @@ def test_decode_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size, s
                               torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
                               cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=7, max_ctx=700, splits=splits, **kw).cpu().float()
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+    # the splits' arrival counters are left at zero: further launches (other values, same pages) agree too
+    dev = [t.to(DEV) for t in (kp, vp, cu, ctx, table)]
+    for factor in (0.5, -2.0, 1.0):
+        out = torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV)
+        again = ops.paged_attention((q * factor).to(DEV), dev[0], dev[1], out, dev[2], dev[3], dev[4],
+                                    num_decode=7, max_ctx=700, splits=splits, **kw).cpu().float()
+        if factor == 1.0:
+            assert torch.equal(again, got)
+        else:
+            expect = refs.paged_attention(q * factor, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype),
+                                          cu, ctx, table, **kw).float()
+            torch.testing.assert_close(again, expect, atol=2e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("window", [1, 16, 37, 300])
