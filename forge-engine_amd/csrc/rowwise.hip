@@ -37,14 +37,23 @@ extern "C" int fe_embed_rows(const int* ids, const void* table, int table_dtype,
 // For output row r (source row s = rows ? rows[r] : r):
 //   sum = h[s] + delta[s]          (float32; written back to h[s] if store_sum)
 //   out[r] = sum * rsqrt(mean(sum^2) + eps) * w
+// delta may come in `parts` pieces `part_stride` elements apart (the partial sums of a product
+// whose K was split over blocks); they are added in order before anything else.
 // Statistics, scaling and the weight product are float32; one rounding at the
 // store.  One block per row; the row is re-read from h/delta in the second
 // pass (it is cache-resident), so any width works.
+template <typename TD>
+__device__ __forceinline__ float delta_sum(const TD* p, int parts, size_t part_stride) {
+  float d = load_as_float(p);
+  for (int k = 1; k < parts; ++k) d += load_as_float(p + k * part_stride);
+  return d;
+}
+
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                    const float* __restrict__ w, TO* __restrict__ out,
                                    const int* __restrict__ rows, int hidden, float eps,
-                                   int store_sum) {
+                                   int store_sum, int parts, size_t part_stride) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int s = rows ? rows[r] : r;
@@ -54,7 +63,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float v = hrow[i];
     if (drow) {
-      v += load_as_float(drow + i);
+      v += delta_sum(drow + i, parts, part_stride);
       if (store_sum) hrow[i] = v;
     }
     sumsq += v * v;
@@ -64,7 +73,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   TO* orow = out + (size_t)r * hidden;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float v = hrow[i];
-    if (drow && !store_sum) v += load_as_float(drow + i);
+    if (drow && !store_sum) v += delta_sum(drow + i, parts, part_stride);
     store_from_float(orow + i, v * inv * w[i]);
   }
 }
@@ -88,7 +97,8 @@ __device__ __forceinline__ void store4_from_float(bf16_t* p, float4 v) {
 template <typename TD, typename TO, int VEC>
 __global__ __launch_bounds__(256) void add_rmsnorm_regs_kernel(
     float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ w,
-    TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps, int store_sum) {
+    TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps, int store_sum,
+    int parts, size_t part_stride) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int s = rows ? rows[r] : r;
@@ -103,7 +113,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_regs_kernel(
     if (i < hidden) {
       v[j] = load4_as_float(hrow + i);
       if (drow) {
-        const float4 d = load4_as_float(drow + i);
+        float4 d = load4_as_float(drow + i);
+        for (int k = 1; k < parts; ++k) {
+          const float4 e = load4_as_float(drow + k * part_stride + i);
+          d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
+        }
         v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
         if (store_sum) *(float4*)(hrow + i) = v[j];
       }
@@ -126,63 +140,70 @@ __global__ __launch_bounds__(256) void add_rmsnorm_regs_kernel(
 
 template <typename TD, typename TO>
 static void launch_add_rmsnorm_typed(float* h, const TD* delta, const float* w, TO* out, const int* rows,
-                                     int n_rows, int hidden, float eps, int store_sum, hipStream_t stream) {
-  const bool aligned = hidden % 4 == 0 && (((uintptr_t)h | (uintptr_t)delta | (uintptr_t)w | (uintptr_t)out) & 15) == 0;
+                                     int n_rows, int hidden, float eps, int store_sum, int parts,
+                                     size_t part_stride, hipStream_t stream) {
+  const bool aligned = hidden % 4 == 0 && part_stride % 4 == 0 && (((uintptr_t)h | (uintptr_t)delta | (uintptr_t)w | (uintptr_t)out) & 15) == 0;
   if (aligned && hidden <= 1024)
-    add_rmsnorm_regs_kernel<TD, TO, 1><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum);
+    add_rmsnorm_regs_kernel<TD, TO, 1><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
   else if (aligned && hidden <= 4096)
-    add_rmsnorm_regs_kernel<TD, TO, 4><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum);
+    add_rmsnorm_regs_kernel<TD, TO, 4><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
   else if (aligned && hidden <= 8192)
-    add_rmsnorm_regs_kernel<TD, TO, 8><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum);
+    add_rmsnorm_regs_kernel<TD, TO, 8><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
   else {
     const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
-    add_rmsnorm_kernel<TD, TO><<<n_rows, threads, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum);
+    add_rmsnorm_kernel<TD, TO><<<n_rows, threads, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
   }
 }
 
 template <typename TD>
 static int launch_add_rmsnorm(float* h, const TD* delta, const float* w, void* out, int out_dtype,
                               const int* rows, int n_rows, int hidden, float eps, int store_sum,
-                              hipStream_t stream) {
+                              int parts, size_t part_stride, hipStream_t stream) {
   if (out_dtype == FE_F32)
-    launch_add_rmsnorm_typed<TD, float>(h, delta, w, (float*)out, rows, n_rows, hidden, eps, store_sum, stream);
+    launch_add_rmsnorm_typed<TD, float>(h, delta, w, (float*)out, rows, n_rows, hidden, eps, store_sum, parts, part_stride, stream);
   else if (out_dtype == FE_BF16)
-    launch_add_rmsnorm_typed<TD, bf16_t>(h, delta, w, (bf16_t*)out, rows, n_rows, hidden, eps, store_sum, stream);
+    launch_add_rmsnorm_typed<TD, bf16_t>(h, delta, w, (bf16_t*)out, rows, n_rows, hidden, eps, store_sum, parts, part_stride, stream);
   else
     return FE_BAD_ARGUMENT;
   return fe_check_launch();
 }
 
 // delta may be null (plain RMSNorm).  rows may be null (all n_rows rows in order).
-// With rows given, store_sum must be 0 unless the rows are distinct.
+// With rows given, store_sum must be 0 unless the rows are distinct.  delta_parts >= 1 pieces of
+// delta lie part_stride elements apart.
 extern "C" int fe_add_rmsnorm(float* h, const void* delta, int delta_dtype, const float* w,
                               void* out, int out_dtype, const int* rows, int n_rows, int hidden,
-                              float eps, int store_sum, hipStream_t stream) {
+                              float eps, int store_sum, int delta_parts, long long part_stride,
+                              hipStream_t stream) {
   if (n_rows <= 0) return FE_OK;
-  if (hidden <= 0 || !(eps > 0.f)) return FE_BAD_ARGUMENT;
+  if (hidden <= 0 || !(eps > 0.f) || delta_parts < 1 || delta_parts > 64 || part_stride < 0) return FE_BAD_ARGUMENT;
   if (delta == nullptr || delta_dtype == FE_F32)
-    return launch_add_rmsnorm<float>(h, (const float*)delta, w, out, out_dtype, rows, n_rows, hidden, eps, store_sum, stream);
+    return launch_add_rmsnorm<float>(h, (const float*)delta, w, out, out_dtype, rows, n_rows, hidden, eps, store_sum, delta_parts, (size_t)part_stride, stream);
   if (delta_dtype == FE_BF16)
-    return launch_add_rmsnorm<bf16_t>(h, (const bf16_t*)delta, w, out, out_dtype, rows, n_rows, hidden, eps, store_sum, stream);
+    return launch_add_rmsnorm<bf16_t>(h, (const bf16_t*)delta, w, out, out_dtype, rows, n_rows, hidden, eps, store_sum, delta_parts, (size_t)part_stride, stream);
   return FE_BAD_ARGUMENT;
 }
 
-// h[t] += delta[t] for all rows (flushes a pending update without a norm).
+// h[t] += delta[t] for all rows (flushes a pending update without a norm); delta in `parts`
+// pieces `part_stride` elements apart, added in order.
 template <typename TD>
-__global__ void add_rows_kernel(float* __restrict__ h, const TD* __restrict__ delta, size_t count) {
+__global__ void add_rows_kernel(float* __restrict__ h, const TD* __restrict__ delta, size_t count, int parts,
+                                size_t part_stride) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
-    h[i] += load_as_float(delta + i);
+    h[i] += delta_sum(delta + i, parts, part_stride);
 }
 
-extern "C" int fe_add_rows(float* h, const void* delta, int delta_dtype, long long count, hipStream_t stream) {
+extern "C" int fe_add_rows(float* h, const void* delta, int delta_dtype, long long count, int delta_parts,
+                           long long part_stride, hipStream_t stream) {
   if (count <= 0) return FE_OK;
+  if (delta_parts < 1 || delta_parts > 64 || part_stride < 0) return FE_BAD_ARGUMENT;
   const int threads = 256;
   long long want = (count + threads - 1) / threads;
   const int blocks = (int)(want < 4096 ? want : 4096);
   if (delta_dtype == FE_F32)
-    add_rows_kernel<float><<<blocks, threads, 0, stream>>>(h, (const float*)delta, (size_t)count);
+    add_rows_kernel<float><<<blocks, threads, 0, stream>>>(h, (const float*)delta, (size_t)count, delta_parts, (size_t)part_stride);
   else if (delta_dtype == FE_BF16)
-    add_rows_kernel<bf16_t><<<blocks, threads, 0, stream>>>(h, (const bf16_t*)delta, (size_t)count);
+    add_rows_kernel<bf16_t><<<blocks, threads, 0, stream>>>(h, (const bf16_t*)delta, (size_t)count, delta_parts, (size_t)part_stride);
   else
     return FE_BAD_ARGUMENT;
   return fe_check_launch();

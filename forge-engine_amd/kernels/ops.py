@@ -80,17 +80,18 @@ def embed_rows(ids: Tensor, table: Tensor, out: Tensor) -> Tensor:
 def add_rmsnorm(h: Tensor, delta: Tensor | None, weight: Tensor, eps: float, out: Tensor,
                 rows: Tensor | None = None, store_sum: bool = True) -> Tensor:
     """sum = h[s] + delta[s] (float32, written back to h if store_sum);
-    out[r] = sum * rsqrt(mean(sum^2) + eps) * weight, s = rows[r] or r."""
+    out[r] = sum * rsqrt(mean(sum^2) + eps) * weight, s = rows[r] or r.
+    delta may be [parts, rows, hidden]: the parts are added up in order first."""
     _gpu(h, "h", torch.float32)
     _gpu(weight, "weight", torch.float32)
     _gpu(out, "out")
     total_rows, hidden = h.shape
     if weight.shape != (hidden,):
         raise KernelError(f"weight must be [{hidden}], got {tuple(weight.shape)}")
+    parts = 1
     if delta is not None:
         _gpu(delta, "delta")
-        if delta.shape != h.shape:
-            raise KernelError(f"delta must be {tuple(h.shape)}, got {tuple(delta.shape)}")
+        parts = _delta_parts(h, delta)
     n_rows = total_rows
     if rows is not None:
         _gpu(rows, "rows", torch.int32)
@@ -104,18 +105,25 @@ def add_rmsnorm(h: Tensor, delta: Tensor | None, weight: Tensor, eps: float, out
     _call("rowwise", "fe_add_rmsnorm", _ptr(h), _ptr(delta),
           c_int(_code(delta.dtype) if delta is not None else FE_F32), _ptr(weight), _ptr(out),
           c_int(_code(out.dtype)), _ptr(rows), c_int(n_rows), c_int(hidden), c_float(eps),
-          c_int(1 if (store_sum and delta is not None) else 0), _stream())
+          c_int(1 if (store_sum and delta is not None) else 0), c_int(parts), c_longlong(h.numel()), _stream())
     return out
 
 
+def _delta_parts(h: Tensor, delta: Tensor) -> int:
+    if delta.shape == h.shape:
+        return 1
+    if delta.dim() == 3 and delta.shape[1:] == h.shape and 1 <= delta.shape[0] <= 64:
+        return delta.shape[0]
+    raise KernelError(f"delta must be {tuple(h.shape)} or [parts <= 64, {h.shape[0]}, {h.shape[1]}], got {tuple(delta.shape)}")
+
+
 def add_rows(h: Tensor, delta: Tensor) -> Tensor:
-    """h += delta, in float32."""
+    """h += delta, in float32; delta may be [parts, rows, hidden] (added up in order)."""
     _gpu(h, "h", torch.float32)
     _gpu(delta, "delta")
-    if delta.shape != h.shape:
-        raise KernelError(f"delta must be {tuple(h.shape)}, got {tuple(delta.shape)}")
+    parts = _delta_parts(h, delta)
     _call("rowwise", "fe_add_rows", _ptr(h), _ptr(delta), c_int(_code(delta.dtype)),
-          c_longlong(h.numel()), _stream())
+          c_longlong(h.numel()), c_int(parts), c_longlong(h.numel()), _stream())
     return h
 
 
@@ -230,6 +238,26 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
     if bias is not None:
         y += bias.to(y.dtype)
     return y
+
+
+# Measured on MI355X: a weight with few row tiles and a long K (the down projection: 160 tiles,
+# K = 9728) leaves CUs idle; four parts of K with blocks of their own take 14.7 instead of 18.4 us
+# at 8 rows.  The consumer (add_rmsnorm, add_rows) adds the parts in order.
+UPDATE_SPLIT_MAX_TILES = 256
+UPDATE_SPLIT_MIN_STEPS = 32
+UPDATE_SPLITS = 4
+
+
+def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
+    """The float32 product x @ weight^T (+ bias) as an update of the residual stream: [M, N], or
+    partial sums [parts, M, N] that ``add_rmsnorm`` / ``add_rows`` add up."""
+    _gpu(x, "x")
+    _gpu(weight, "weight", contiguous=False)
+    if (bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and _skinny_fits(x, weight)
+            and -(-weight.shape[0] // 16) <= UPDATE_SPLIT_MAX_TILES
+            and -(-weight.shape[1] // 128) >= UPDATE_SPLIT_MIN_STEPS):
+        return gemm_skinny(x, weight, "f32", tiles=1, waves=8, splits=UPDATE_SPLITS)
+    return linear(x, weight, bias, out_dtype=torch.float32)
 
 
 def linear_swiglu(x: Tensor, gate_up_weight: Tensor) -> Tensor:

@@ -131,7 +131,7 @@ class GroupedQueryAttention(Mixer):
             num_seqs=batch.num_seqs, max_q_len=batch.max_q_len, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
             num_decode=batch.num_decode, max_ctx=batch.max_ctx)
-        return ops.linear(attn, self.o_weight, self.o_bias, out_dtype=torch.float32)   # float32 update for the residual sum
+        return ops.linear_update(attn, self.o_weight, self.o_bias)   # float32 update for the residual sum
 
     def kernel_libraries(self):
         return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny"}

@@ -45,7 +45,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: Tensor, batch=None) -> Tensor:
         act = ops.linear_swiglu(x, self.gate_up_weight)
-        return ops.linear(act, self.down_weight, out_dtype=torch.float32)   # the update stays float32 for the residual sum
+        return ops.linear_update(act, self.down_weight)   # the update stays float32 for the residual sum
 
     def kernel_libraries(self):
         return {"rowwise", "gemm_f32", "gemm_skinny"}

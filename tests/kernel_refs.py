@@ -19,6 +19,8 @@ def embed_rows(ids, table, out):
 
 
 def add_rmsnorm(h, delta, weight, eps, out, rows=None, store_sum=True):
+    if delta is not None and delta.dim() == 3:
+        delta = delta.float().sum(0)
     if rows is not None:
         src = h[rows.long()]
         if delta is not None:
@@ -33,7 +35,7 @@ def add_rmsnorm(h, delta, weight, eps, out, rows=None, store_sum=True):
 
 
 def add_rows(h, delta):
-    h += delta.float()
+    h += delta.float().sum(0) if delta.dim() == 3 else delta.float()
     return h
 
 
@@ -70,7 +72,11 @@ def linear_swiglu(x, gate_up_weight):
     return (g / (1.0 + torch.exp(-g)) * u).to(x.dtype)
 
 
-def gemm_skinny(x, weight, epilogue="bf16", tiles=0, waves=0):
+def linear_update(x, weight, bias=None):
+    return linear(x, weight, bias, out_dtype=torch.float32)
+
+
+def gemm_skinny(x, weight, epilogue="bf16", tiles=0, waves=0, splits=1):
     if epilogue == "swiglu":
         return linear_swiglu(x, weight)
     return linear(x, weight, out_dtype=torch.float32 if epilogue == "f32" else torch.bfloat16)
@@ -204,7 +210,7 @@ def sample_rows(logits, temperatures, seeds, draw_index, tokens, status):
         tokens[r] = min(pick, logits.shape[1] - 1)
 
 
-NAMES = ("embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_swiglu", "gemm_skinny",
+NAMES = ("embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_update", "linear_swiglu", "gemm_skinny",
          "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_rows")
 
 

@@ -406,6 +406,50 @@ def test_gemm_skinny_resident_refuses(ops):
         ops.gemm_skinny(x, w, "f32", tiles=-1)          # K beyond what the registers hold
 
 
+@pytest.mark.parametrize("m,n,k,splits", [(1, 200, 1000, 3), (8, 2560, 9728, 4), (16, 330, 4096, 16), (5, 64, 264, 2)])
+def test_gemm_skinny_parts_and_their_consumers(ops, m, n, k, splits):
+    """K summed in parts by blocks of their own: the parts add up to the product, and the norm and
+    the plain add take them as they are (added in order, so repeated calls give the same bits)."""
+    g = torch.Generator().manual_seed(24)
+    x = rand(g, m, k, dtype=torch.bfloat16).to(DEV)
+    w = rand(g, n, k, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    whole = ops.gemm_skinny(x, w, "f32", tiles=1, waves=8)
+    parts = ops.gemm_skinny(x, w, "f32", tiles=1, waves=8, splits=splits)
+    assert parts.shape == (splits, m, n)
+    want = x.float().cpu() @ w.float().cpu().T
+    bound = 2e-6 * float(want.abs().max()) * math.sqrt(k) + 1e-6
+    assert float((parts.sum(0).cpu() - want).abs().max()) <= bound
+    assert float((whole.cpu() - want).abs().max()) <= bound
+    h = rand(g, m, n).to(DEV)
+    nw = rand(g, n).to(DEV)
+    summed = parts[0].clone()
+    for part in parts[1:]:
+        summed += part
+    for dtype in (torch.float32, torch.bfloat16):
+        h1, h2 = h.clone(), h.clone()
+        got = ops.add_rmsnorm(h1, parts, nw, 1e-6, torch.empty(m, n, dtype=dtype, device=DEV))
+        ref = ops.add_rmsnorm(h2, summed, nw, 1e-6, torch.empty(m, n, dtype=dtype, device=DEV))
+        assert torch.equal(got, ref) and torch.equal(h1, h2)
+    h1, h2 = h.clone(), h.clone()
+    assert torch.equal(ops.add_rows(h1, parts), ops.add_rows(h2, summed))
+    with pytest.raises(ops.KernelError):
+        ops.add_rows(h1, parts[:, :, :-1].contiguous())
+
+
+def test_linear_update_routes(ops):
+    g = torch.Generator().manual_seed(25)
+    x = rand(g, 8, 4096, dtype=torch.bfloat16).to(DEV)
+    few_rows = rand(g, 320, 4096, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    many_rows = rand(g, 8192, 4096, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    assert ops.linear_update(x, few_rows).dim() == 3              # few row tiles, long K: parts
+    assert ops.linear_update(x, many_rows).dim() == 2
+    assert ops.linear_update(x[:, :1024].contiguous(), few_rows[:, :1024]).dim() == 2
+    big = rand(g, 40, 4096, dtype=torch.bfloat16).to(DEV)
+    assert ops.linear_update(big, few_rows).shape == (40, 320)     # beyond 16 rows: the library
+    want = x.float().cpu() @ few_rows.float().cpu().T
+    torch.testing.assert_close(ops.linear_update(x, few_rows).sum(0).cpu(), want, atol=1e-3, rtol=1e-3)
+
+
 def test_linear_routes_by_rows_and_dtype(ops):
     g = torch.Generator().manual_seed(22)
     w = rand(g, 136, 200, dtype=torch.bfloat16, scale=0.05)
