@@ -16,6 +16,10 @@
 // slot p % block_size.
 #include "common.h"
 
+// One block serves `heads_per_block` heads of one token (4 waves, a head per wave at a time).
+// The cosines and sines of the token's angles are computed once per block into LDS: with many
+// tokens a block takes all heads of its token, so the (accurate, slow for large angles) sincosf
+// runs once per (token, frequency) instead of once per head.
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
     T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
@@ -23,101 +27,111 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
     const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_stride,
     T* __restrict__ key_pages, T* __restrict__ value_pages, int q_heads, int kv_heads,
     int head_dim, int rotary_dim, int block_size, int num_blocks, float eps, int write_kv,
-    int total_heads_work) {
+    int heads_per_block, int groups_per_token) {
+  __shared__ float cos_s[256], sin_s[256];
+  __shared__ float stage[4][512];
   const int lane = threadIdx.x & (FE_WAVE - 1);
   const int wave = threadIdx.x / FE_WAVE;
-  const int work = blockIdx.x * (blockDim.x / FE_WAVE) + wave;  // one (token, head) per wave
-  if (work >= total_heads_work) return;
+  const int t = blockIdx.x / groups_per_token;
+  const int group = blockIdx.x - t * groups_per_token;
   const int heads_all = q_heads + 2 * kv_heads;
-  const int t = work / heads_all;
-  const int head = work - t * heads_all;
-  T* x = qkv + ((size_t)t * heads_all + head) * head_dim;
-  const bool is_q = head < q_heads;
-  const bool is_k = !is_q && head < q_heads + kv_heads;
-  const int kv_head = is_q ? 0 : (is_k ? head - q_heads : head - q_heads - kv_heads);
+  const int head_end = min(heads_all, (group + 1) * heads_per_block);
   const int pos = positions[t];
-
-  T* dst = x;  // q stays in place
-  if (!is_q) {
-    if (!write_kv) return;
-    const int seq = token_seq[t];
-    const int block = block_table[(size_t)seq * table_stride + pos / block_size];
-    if (block < 0 || block >= num_blocks) return;  // host reserves pages before the launch
-    const size_t page = ((size_t)block * kv_heads + kv_head) * block_size * head_dim;
-    if (!is_k) {  // value: copy into the transposed page
-      T* vdst = value_pages + page + (pos % block_size);
-      for (int d = lane; d < head_dim; d += FE_WAVE) vdst[(size_t)d * block_size] = x[d];
-      return;
-    }
-    dst = key_pages + page + (size_t)(pos % block_size) * head_dim;
-  }
-
-  const float* w = is_q ? q_weight : k_weight;
   const int half = head_dim / 2;
   const int rhalf = rotary_dim / 2;
-  // Each lane owns pairs (j, j + half) for j = lane, lane + 64, ...; head_dim <= 512.
-  float lo[4], hi[4];
-  float sumsq = 0.f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int j = lane + i * FE_WAVE;
-    lo[i] = 0.f; hi[i] = 0.f;
-    if (j < half) {
-      lo[i] = load_as_float(x + j);
-      hi[i] = load_as_float(x + j + half);
-      sumsq += lo[i] * lo[i] + hi[i] * hi[i];
+  for (int j = threadIdx.x; j < rhalf; j += blockDim.x) {
+    float sn, cs;
+    sincosf((float)pos * inv_freq[j], &sn, &cs);
+    cos_s[j] = cs;
+    sin_s[j] = sn;
+  }
+  __syncthreads();
+
+  for (int head = group * heads_per_block + wave; head < head_end; head += 4) {
+    T* x = qkv + ((size_t)t * heads_all + head) * head_dim;
+    const bool is_q = head < q_heads;
+    const bool is_k = !is_q && head < q_heads + kv_heads;
+    const int kv_head = is_q ? 0 : (is_k ? head - q_heads : head - q_heads - kv_heads);
+
+    T* dst = x;  // q stays in place
+    if (!is_q) {
+      if (!write_kv) continue;
+      const int seq = token_seq[t];
+      const int block = block_table[(size_t)seq * table_stride + pos / block_size];
+      if (block < 0 || block >= num_blocks) continue;  // host reserves pages before the launch
+      const size_t page = ((size_t)block * kv_heads + kv_head) * block_size * head_dim;
+      if (!is_k) {  // value: copy into the transposed page
+        T* vdst = value_pages + page + (pos % block_size);
+        for (int d = lane; d < head_dim; d += FE_WAVE) vdst[(size_t)d * block_size] = x[d];
+        continue;
+      }
+      dst = key_pages + page + (size_t)(pos % block_size) * head_dim;
     }
-  }
-  float inv = 1.f;
-  if (w) {
-    sumsq = wave_sum(sumsq);
-    inv = rsqrtf(sumsq / (float)head_dim + eps);
-  }
+
+    const float* w = is_q ? q_weight : k_weight;
+    // Each lane owns pairs (j, j + half) for j = lane, lane + 64, ...; head_dim <= 512.
+    float lo[4], hi[4];
+    float sumsq = 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int j = lane + i * FE_WAVE;
-    if (j < half) {
-      if (w) {
-        lo[i] = lo[i] * inv * w[j];
-        hi[i] = hi[i] * inv * w[j + half];
+    for (int i = 0; i < 4; ++i) {
+      const int j = lane + i * FE_WAVE;
+      lo[i] = 0.f; hi[i] = 0.f;
+      if (j < half) {
+        lo[i] = load_as_float(x + j);
+        hi[i] = load_as_float(x + j + half);
+        sumsq += lo[i] * lo[i] + hi[i] * hi[i];
       }
     }
-  }
-  // Rotation pairs are (j, j + rhalf) for j < rhalf.  With rotary_dim == head_dim
-  // the partner of lo[i] is hi[i] and everything stays in registers.
-  if (rotary_dim == head_dim) {
+    float inv = 1.f;
+    if (w) {
+      sumsq = wave_sum(sumsq);
+      inv = rsqrtf(sumsq / (float)head_dim + eps);
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int j = lane + i * FE_WAVE;
       if (j < half) {
-        float s, c;
-        sincosf((float)pos * inv_freq[j], &s, &c);
-        const float a = lo[i], b = hi[i];
-        store_from_float(dst + j, a * c - b * s);
-        store_from_float(dst + j + half, b * c + a * s);
+        if (w) {
+          lo[i] = lo[i] * inv * w[j];
+          hi[i] = hi[i] * inv * w[j + half];
+        }
       }
     }
-  } else {
-    // Partial rotation: partners may sit in other lanes, so the normalised head
-    // goes through a per-wave LDS buffer (LDS operations of one wave are ordered).
-    __shared__ float stage[4][512];
-    float* buf = stage[wave];
+    // Rotation pairs are (j, j + rhalf) for j < rhalf.  With rotary_dim == head_dim
+    // the partner of lo[i] is hi[i] and everything stays in registers.
+    if (rotary_dim == head_dim) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int j = lane + i * FE_WAVE;
-      if (j < half) { buf[j] = lo[i]; buf[j + half] = hi[i]; }
-    }
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
-    for (int d = lane; d < head_dim; d += FE_WAVE) {
-      float v = buf[d];
-      if (d < rotary_dim) {
-        const int j = d < rhalf ? d : d - rhalf;
-        float s, c;
-        sincosf((float)pos * inv_freq[j], &s, &c);
-        v = d < rhalf ? buf[d] * c - buf[d + rhalf] * s : buf[d] * c + buf[d - rhalf] * s;
+      for (int i = 0; i < 4; ++i) {
+        const int j = lane + i * FE_WAVE;
+        if (j < half) {
+          const float sn = sin_s[j], cs = cos_s[j];
+          const float a = lo[i], b = hi[i];
+          store_from_float(dst + j, a * cs - b * sn);
+          store_from_float(dst + j + half, b * cs + a * sn);
+        }
       }
-      store_from_float(dst + d, v);
+    } else {
+      // Partial rotation: partners may sit in other lanes, so the normalised head
+      // goes through a per-wave LDS buffer (LDS operations of one wave are ordered).
+      float* buf = stage[wave];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = lane + i * FE_WAVE;
+        if (j < half) { buf[j] = lo[i]; buf[j + half] = hi[i]; }
+      }
+      __builtin_amdgcn_wave_barrier();
+      __threadfence_block();
+      for (int d = lane; d < head_dim; d += FE_WAVE) {
+        float v = buf[d];
+        if (d < rotary_dim) {
+          const int j = d < rhalf ? d : d - rhalf;
+          const float sn = sin_s[j], cs = cos_s[j];
+          v = d < rhalf ? buf[d] * cs - buf[d + rhalf] * sn : buf[d] * cs + buf[d - rhalf] * sn;
+        }
+        store_from_float(dst + d, v);
+      }
+      __builtin_amdgcn_wave_barrier();
+      __threadfence_block();      // the buffer is written again for the wave's next head
     }
   }
 }
@@ -135,19 +149,23 @@ extern "C" int fe_qk_norm_rope_write(void* qkv, int dtype, const float* q_weight
   if (write_kv && (block_size <= 0 || num_blocks <= 0 || !block_table || !key_pages || !value_pages)) return FE_BAD_ARGUMENT;
   const long long work = (long long)tokens * (q_heads + 2 * kv_heads);
   if (work <= 0 || work > 0x7fffffffLL) return FE_BAD_ARGUMENT;
-  const int waves_per_block = 4;
-  const long long blocks = (work + waves_per_block - 1) / waves_per_block;
+  // few tokens: four heads a block, so that the launch has many blocks; many tokens: a block per
+  // token, so that the angles' sines and cosines are computed once per token
+  const int heads_all = q_heads + 2 * kv_heads;
+  const int heads_per_block = tokens >= 256 ? heads_all : 4;
+  const int groups_per_token = (heads_all + heads_per_block - 1) / heads_per_block;
+  const long long blocks = (long long)tokens * groups_per_token;
   if (blocks > 0x7fffffffLL) return FE_BAD_ARGUMENT;
   if (dtype == FE_F32)
     qk_norm_rope_write_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>(
         (float*)qkv, q_weight, k_weight, inv_freq, positions, token_seq, block_table, table_stride,
         (float*)key_pages, (float*)value_pages, q_heads, kv_heads, head_dim, rotary_dim, block_size,
-        num_blocks, eps, write_kv, (int)work);
+        num_blocks, eps, write_kv, heads_per_block, groups_per_token);
   else if (dtype == FE_BF16)
     qk_norm_rope_write_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>(
         (bf16_t*)qkv, q_weight, k_weight, inv_freq, positions, token_seq, block_table, table_stride,
         (bf16_t*)key_pages, (bf16_t*)value_pages, q_heads, kv_heads, head_dim, rotary_dim, block_size,
-        num_blocks, eps, write_kv, (int)work);
+        num_blocks, eps, write_kv, heads_per_block, groups_per_token);
   else
     return FE_BAD_ARGUMENT;
   return fe_check_launch();

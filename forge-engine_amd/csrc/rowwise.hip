@@ -114,9 +114,14 @@ __global__ __launch_bounds__(256) void add_rmsnorm_regs_kernel(
       v[j] = load4_as_float(hrow + i);
       if (drow) {
         float4 d = load4_as_float(drow + i);
-        for (int k = 1; k < parts; ++k) {
-          const float4 e = load4_as_float(drow + k * part_stride + i);
-          d.x += e.x; d.y += e.y; d.z += e.z; d.w += e.w;
+        for (int k = 1; k < parts; k += 4) {     // four parts' loads fly together; added in order
+          float4 e[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            e[u] = k + u < parts ? load4_as_float(drow + (k + u) * part_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (k + u < parts) { d.x += e[u].x; d.y += e[u].y; d.z += e[u].z; d.w += e[u].w; }
         }
         v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
         if (store_sum) *(float4*)(hrow + i) = v[j];
@@ -224,11 +229,40 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
   }
 }
 
+// bfloat16 rows whose width is a multiple of 8: eight elements (16 bytes) of gate and of up per thread.
+__global__ __launch_bounds__(256) void swiglu_bf16x8_kernel(const bf16_t* __restrict__ gate_up,
+                                                            bf16_t* __restrict__ out, int inter8, size_t total8) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total8; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = i / inter8;
+    const int c = (int)(i - t * inter8);
+    const uint4* row = (const uint4*)gate_up + t * 2 * (size_t)inter8;
+    const uint4 g = row[c];
+    const uint4 u = row[inter8 + c];
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
+      const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
+      ow[k] = (uint32_t)float_to_bf16(g0 / (1.f + expf(-g0)) * u0) |
+              ((uint32_t)float_to_bf16(g1 / (1.f + expf(-g1)) * u1) << 16);
+    }
+    ((uint4*)out)[i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+  }
+}
+
 extern "C" int fe_swiglu(const void* gate_up, void* out, int dtype, int tokens, int inter, hipStream_t stream) {
   if (tokens <= 0) return FE_OK;
   if (inter <= 0) return FE_BAD_ARGUMENT;
   const size_t total = (size_t)tokens * inter;
   const int threads = 256;
+  if (dtype == FE_BF16 && inter % 8 == 0 && ((((uintptr_t)gate_up) | ((uintptr_t)out)) & 15) == 0) {
+    const size_t total8 = total / 8;
+    const size_t want8 = (total8 + threads - 1) / threads;
+    swiglu_bf16x8_kernel<<<(int)(want8 < 16384 ? want8 : 16384), threads, 0, stream>>>(
+        (const bf16_t*)gate_up, (bf16_t*)out, inter / 8, total8);
+    return fe_check_launch();
+  }
   size_t want = (total + threads - 1) / threads;
   const int blocks = (int)(want < 8192 ? want : 8192);
   if (dtype == FE_F32)

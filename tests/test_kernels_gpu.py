@@ -96,6 +96,11 @@ def test_add_rows_and_swiglu(ops, dtype):
     torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
     # the library expression of the reference's own test (tests/test_cute_swiglu.py:18-27)
     torch.testing.assert_close(got.float(), (torch.nn.functional.silu(gu[:, :328].float()) * gu[:, 328:].float()), **tol(dtype))
+    for inter in (100, 8, 9728):     # widths that are and are not a multiple of the 8-element pieces
+        gu = rand(g, 37, 2 * inter, dtype=dtype, scale=2.0)
+        want = refs.swiglu(gu, torch.empty(37, inter, dtype=dtype))
+        got = ops.swiglu(gu.to(DEV), torch.empty(37, inter, dtype=dtype, device=DEV)).cpu()
+        torch.testing.assert_close(got.float(), want.float(), **tol(dtype))
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 70, 50), (65, 129, 96), (130, 64, 2560), (17, 1003, 200), (5, 33, 7)])
@@ -137,9 +142,10 @@ def _qk_case(g, dtype, tokens, q_heads, kv_heads, head_dim, block_size, num_bloc
     (4, 2, 16, 4, 16), (6, 2, 32, 8, 32), (5, 1, 128, 16, 128), (3, 3, 64, 1, 32), (8, 2, 256, 32, 256),
     (2, 1, 48, 5, 0),
 ])
-def test_qk_norm_rope_write(ops, dtype, q_heads, kv_heads, head_dim, block_size, rotary_dim):
+@pytest.mark.parametrize("tokens", [11, 300])       # few tokens: four heads a block; many: a block per token
+def test_qk_norm_rope_write(ops, dtype, q_heads, kv_heads, head_dim, block_size, rotary_dim, tokens):
     g = torch.Generator().manual_seed(5)
-    tokens, num_blocks = 11, 40
+    num_blocks = 2 * ((tokens + 5) // block_size + 2)
     qkv, qw, kw, positions, token_seq, table = _qk_case(g, dtype, tokens, q_heads, kv_heads, head_dim, block_size, num_blocks)
     inv_freq = None
     if rotary_dim:
