@@ -50,7 +50,9 @@ def _ptr(tensor: Tensor | None) -> c_void_p:
 
 
 def _stream() -> c_void_p:
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the raw handle of the current stream of the current device (a plain C call; building a
+    # torch.cuda.Stream object for every launch costs more than the launch)
+    return c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
 
 
 def _call(lib_name: str, fn_name: str, *args) -> None:
