@@ -23,6 +23,7 @@ from forge_engine_amd.engine import (GenerationEngine, ModelRunner, StepEntry, b
                                      engine_from_folder, load_model)
 from forge_engine_amd.parts import (BuildContext, LayerCall, LayerSpec, Mixer, ModelPlan, ParamSpec, PartSpec,
                                     Residual, build_part)
+from forge_engine_amd.parts.base import Embedding, FeedForward
 from forge_engine_amd.registry import register_architecture, register_part
 from forge_engine_amd.sampling import SamplingParams
 from forge_engine_amd.weights import fill_random_weights, write_random_model
@@ -471,6 +472,202 @@ def test_toy_architecture_registered_from_a_test(dtype):
         scale = float(want[k].abs().max())
         bound = 1e-4 * scale + 1e-5 if dtype == "float32" else ru.BF16_FRACTION * scale
         assert float((rows - want[k]).abs().max()) <= bound, k
+
+
+# ------------------- a second toy: learned absolute positions, a feed-forward with routing
+
+class PositionedEmbedding(Embedding):
+    """Another position encoding: h0 = E[token] + P[position], a learned table (plain torch ops:
+    test code).  The attention layers of this toy rotate nothing."""
+
+    def __init__(self, ctx, prefix, *, vocab_size: int, hidden_size: int, max_positions: int) -> None:
+        super().__init__(ctx, prefix)
+        self.vocab_size, self.hidden_size, self.max_positions = vocab_size, hidden_size, max_positions
+        self.weight = self.positions = None
+
+    def param_specs(self):
+        return {self.name("weight"): ParamSpec((self.vocab_size, self.hidden_size)),
+                self.name("positions"): ParamSpec((self.max_positions, self.hidden_size))}
+
+    def set_param(self, name, tensor):
+        if name == self.name("weight"):
+            self.weight = tensor
+        else:
+            self.positions = tensor
+
+    def forward(self, batch) -> Residual:
+        h = self.weight[batch.token_ids.long()].float() + self.positions[batch.positions.long()].float()
+        return Residual(h.contiguous())
+
+
+class RoutedFeedForward(FeedForward):
+    """A feed-forward with routing: router logits in float32, the best expert of each token
+    (lowest index among equals) weighted by its softmax probability.  Every expert runs on every
+    token and a mask keeps the chosen one: nothing is decided on the host, so decode steps with
+    this part replay from captured graphs."""
+
+    def __init__(self, ctx, prefix, *, hidden_size: int, intermediate_size: int, experts: int) -> None:
+        super().__init__(ctx, prefix)
+        self.hidden_size, self.intermediate_size, self.experts = hidden_size, intermediate_size, experts
+        self.router = None
+        self.gate_up = [None] * experts
+        self.down = [None] * experts
+
+    def param_specs(self):
+        specs = {self.name("router.weight"): ParamSpec((self.experts, self.hidden_size))}
+        for e in range(self.experts):
+            specs[self.name(f"experts.{e}.gate_up.weight")] = ParamSpec((2 * self.intermediate_size, self.hidden_size))
+            specs[self.name(f"experts.{e}.down.weight")] = ParamSpec((self.hidden_size, self.intermediate_size))
+        return specs
+
+    def set_param(self, name, tensor):
+        local = name[len(self.prefix) + 1:]
+        if local == "router.weight":
+            self.router = tensor
+        else:
+            _, index, which, _ = local.split(".")
+            (self.gate_up if which == "gate_up" else self.down)[int(index)] = tensor
+
+    def forward(self, x, batch=None):
+        from forge_engine_amd.kernels import ops
+        logits = x.float() @ self.router.float().T
+        probs = torch.softmax(logits, dim=-1)
+        chosen = logits.argmax(dim=-1, keepdim=True)
+        update = torch.zeros((x.shape[0], self.hidden_size), dtype=torch.float32, device=x.device)
+        for e in range(self.experts):
+            out = ops.linear(ops.linear_swiglu(x, self.gate_up[e]), self.down[e], out_dtype=torch.float32)
+            update += out * (probs[:, e:e + 1] * (chosen == e))
+        return update
+
+
+@dataclass(frozen=True)
+class RoutedConfig(ModelConfig):
+    vocab_size: int
+    hidden_size: int
+    intermediate_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    experts: int
+    max_positions: int
+    rms_norm_eps: float
+    architecture: ClassVar[str] = "ToyRoutedLM"
+
+    @classmethod
+    def from_dict(cls, raw):
+        read = KeyReader(raw)
+        return cls(*(read.integer(k) for k in ("vocab_size", "hidden_size", "intermediate_size", "num_attention_heads",
+                                              "num_key_value_heads", "head_dim", "experts", "max_positions")),
+                   read.number("rms_norm_eps"))
+
+
+def routed_plan(config: RoutedConfig) -> ModelPlan:
+    def norm(prefix):
+        return PartSpec("rms_norm", {"size": config.hidden_size, "eps": config.rms_norm_eps}, prefix)
+
+    def layer(index, feed_forward):
+        prefix = f"model.layers.{index}"
+        attention = PartSpec("gqa_attention", {
+            "hidden_size": config.hidden_size, "num_heads": config.num_attention_heads,
+            "num_kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+            "position": PartSpec("none", {})}, f"{prefix}.self_attn")
+        return LayerSpec("pre_norm", attention, feed_forward,
+                         {"input": norm(f"{prefix}.input_layernorm"), "post_mixer": norm(f"{prefix}.post_attention_layernorm")})
+
+    sizes = {"hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size}
+    layers = (layer(0, PartSpec("toy_routed", dict(sizes, experts=config.experts), "model.layers.0.moe")),
+              layer(1, PartSpec("swiglu", dict(sizes), "model.layers.1.mlp")))
+    table = {"vocab_size": config.vocab_size, "hidden_size": config.hidden_size}
+    return ModelPlan(config.hidden_size, config.vocab_size,
+                     PartSpec("toy_positioned", dict(table, max_positions=config.max_positions), "model.embed_tokens"),
+                     layers, (LayerCall(0), LayerCall(1)), norm("model.norm"), PartSpec("lm_head", dict(table, tied=False), "lm_head"))
+
+
+def routed_plain_forward(w, config: RoutedConfig, tokens):
+    t = len(tokens)
+    eps = config.rms_norm_eps
+    heads, kv_heads, d = config.num_attention_heads, config.num_key_value_heads, config.head_dim
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)] + w["model.embed_tokens.positions"][:t]
+    for index in (0, 1):
+        p = f"model.layers.{index}"
+        x = plain.rms_norm(h, w[f"{p}.input_layernorm.weight"], eps)
+        q = (x @ w[f"{p}.self_attn.q_proj.weight"].T).view(t, heads, d).transpose(0, 1)
+        k = (x @ w[f"{p}.self_attn.k_proj.weight"].T).view(t, kv_heads, d).transpose(0, 1)
+        v = (x @ w[f"{p}.self_attn.v_proj.weight"].T).view(t, kv_heads, d).transpose(0, 1)
+        attn = plain.causal_attention(q, k, v, d ** -0.5).transpose(0, 1).reshape(t, heads * d)
+        h, y = plain.add_rms_norm(h, attn @ w[f"{p}.self_attn.o_proj.weight"].T, w[f"{p}.post_attention_layernorm.weight"], eps)
+        if index == 1:
+            h = h + plain.swiglu_mlp(y, w, f"{p}.mlp")
+            continue
+        logits = y @ w[f"{p}.moe.router.weight"].T
+        probs = torch.softmax(logits, dim=-1)
+        rows = []
+        for i in range(t):
+            e = int(logits[i].argmax())
+            gate_up = w[f"{p}.moe.experts.{e}.gate_up.weight"]
+            inter = config.intermediate_size
+            act = torch.nn.functional.silu(y[i] @ gate_up[:inter].T) * (y[i] @ gate_up[inter:].T)
+            rows.append(probs[i, e] * (act @ w[f"{p}.moe.experts.{e}.down.weight"].T))
+        h = h + torch.stack(rows)
+    return plain.rms_norm(h, w["model.norm.weight"], eps) @ w["lm_head.weight"].T
+
+
+def test_routed_feed_forward_and_learned_positions_registered_from_a_test(tmp_path):
+    """Parts of other kinds than Qwen3's (an embedding that adds learned positions, attention
+    without rotation, a feed-forward with routing in one layer and a dense one in the other) are
+    registered here, built from a model folder and stepped: portions, then decoding through
+    captured graphs, against a plain whole-sequence implementation."""
+    register_part("embedding", "toy_positioned", PositionedEmbedding, replace=True)
+    register_part("feed_forward", "toy_routed", RoutedFeedForward, replace=True)
+    register_architecture("ToyRoutedLM", RoutedConfig, routed_plan, replace=True)
+    raw = {"architectures": ["ToyRoutedLM"], "vocab_size": 77, "hidden_size": 48, "intermediate_size": 40,
+           "num_attention_heads": 3, "num_key_value_heads": 3, "head_dim": 16, "experts": 3, "max_positions": 64,
+           "rms_norm_eps": 1e-6}
+    config = load_model_config(raw)
+    folder = write_random_model(config, 11, tmp_path, dtype=torch.float32)
+    assert json.loads((folder / "config.json").read_text())["experts"] == 3
+    w = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
+    w["model.embed_tokens.positions"] *= 20.0     # positions that matter, and routing that is not uniform
+    w["model.layers.0.moe.router.weight"] *= 200.0
+    from safetensors.torch import save_file
+    save_file({k: v.contiguous() for k, v in w.items()}, str(folder / "model.safetensors"))
+    _, model = load_model(folder, dtype="float32", device=DEV)
+    assert model.graph_safe
+    requests = ru.make_requests(raw, 5, (29, 40, 17))
+    want = {k: routed_plain_forward(w, config, v) for k, v in requests.items()}
+    runner = ModelRunner(model, block_size=4, block_capacity=30, num_state_slots=3)
+    got = {k: [] for k in requests}
+    for k in requests:
+        runner.begin(k)
+    cut = {k: len(v) - 8 for k, v in requests.items()}
+    at = {k: 0 for k in requests}
+    step = 0
+    while any(at[k] < cut[k] for k in requests):          # prompts in portions of changing size, side by side
+        entries = []
+        for k in requests:
+            size = min((7, 2, 5, 3)[(step + len(requests[k])) % 4], cut[k] - at[k])
+            if size > 0:
+                entries.append(StepEntry(k, requests[k][at[k]:at[k] + size], list(range(size))))
+                at[k] += size
+        logits = runner.step(entries).cpu()
+        row = 0
+        for e in entries:
+            got[e.request_id].append(logits[row:row + len(e.tokens)])
+            row += len(e.tokens)
+        step += 1
+    for i in range(8):                                     # then single tokens: captured graphs
+        entries = [StepEntry(k, [requests[k][cut[k] + i]], [0]) for k in requests]
+        logits = runner.step(entries).cpu()
+        for row, e in enumerate(entries):
+            got[e.request_id].append(logits[row:row + 1])
+    assert runner.graph_replays >= 6
+    for k in requests:
+        rows = torch.cat(got[k])
+        scale = float(want[k].abs().max())
+        assert float((rows - want[k]).abs().max()) <= 1e-4 * scale + 1e-5, k
+    # the routing really spreads: every expert is some token's choice
+    y = plain.rms_norm(w["model.embed_tokens.weight"], w["model.norm.weight"], 1e-6)
+    assert len(set((y @ w["model.layers.0.moe.router.weight"].T).argmax(-1).tolist())) == 3
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
