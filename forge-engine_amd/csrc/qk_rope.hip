@@ -136,6 +136,94 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
   }
 }
 
+// The same for bfloat16 heads of 16 * 2^n elements that are rotated whole (rotary_dim == head_dim):
+// head_dim / 8 lanes share a head, each with 8 consecutive elements (one 16-byte load and store),
+// so a wave works on 512 / head_dim heads at once; the partner of element j, j + head_dim / 2,
+// sits in the lane head_dim / 16 further on (one shuffle per element).
+template <int LPH>    // lanes per head
+__global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
+    bf16_t* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+    const float* __restrict__ inv_freq, const int* __restrict__ positions,
+    const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_stride,
+    bf16_t* __restrict__ key_pages, bf16_t* __restrict__ value_pages, int q_heads, int kv_heads,
+    int block_size, int num_blocks, float eps, int write_kv, int heads_per_block, int groups_per_token) {
+  constexpr int D = LPH * 8;
+  constexpr int HALF = D / 2;
+  constexpr int HEADS_AT_ONCE = 256 / LPH;
+  __shared__ float cos_s[HALF], sin_s[HALF];
+  const int t = blockIdx.x / groups_per_token;
+  const int group = blockIdx.x - t * groups_per_token;
+  const int heads_all = q_heads + 2 * kv_heads;
+  const int head_end = min(heads_all, (group + 1) * heads_per_block);
+  const int pos = positions[t];
+  for (int j = threadIdx.x; j < HALF; j += blockDim.x) {
+    float sn, cs;
+    sincosf((float)pos * inv_freq[j], &sn, &cs);
+    cos_s[j] = cs;
+    sin_s[j] = sn;
+  }
+  __syncthreads();
+  const int sub = threadIdx.x % LPH;          // which 8 elements of the head
+  const int first = sub * 8;
+  const bool low = first < HALF;              // elements of the first half pair with the second
+  for (int head = group * heads_per_block + threadIdx.x / LPH; head < head_end; head += HEADS_AT_ONCE) {
+    bf16_t* x = qkv + ((size_t)t * heads_all + head) * D + first;
+    const bool is_q = head < q_heads;
+    const bool is_k = !is_q && head < q_heads + kv_heads;
+    if (!is_q && !write_kv) continue;
+    const uint4 raw = *(const uint4*)x;
+    size_t page = 0;
+    int slot = 0;
+    if (!is_q) {
+      const int kv_head = is_k ? head - q_heads : head - q_heads - kv_heads;
+      const int block = block_table[(size_t)token_seq[t] * table_stride + pos / block_size];
+      if (block < 0 || block >= num_blocks) continue;  // host reserves pages before the launch
+      page = ((size_t)block * kv_heads + kv_head) * block_size * D;
+      slot = pos % block_size;
+      if (!is_k) {   // value: into the transposed page, element d at [d][slot]
+        const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+        bf16_t* vdst = value_pages + page + slot;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          vdst[(size_t)(first + e) * block_size] = (bf16_t)(e & 1 ? w4[e >> 1] >> 16 : w4[e >> 1] & 0xffffu);
+        continue;
+      }
+    }
+    float v[8];
+    {
+      const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[2 * e] = __uint_as_float(w4[e] << 16);
+        v[2 * e + 1] = __uint_as_float(w4[e] & 0xffff0000u);
+      }
+    }
+    const float* w = is_q ? q_weight : k_weight;
+    if (w) {
+      float sumsq = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sumsq += v[e] * v[e];
+#pragma unroll
+      for (int offset = LPH / 2; offset > 0; offset >>= 1) sumsq += __shfl_xor(sumsq, offset, FE_WAVE);
+      const float inv = rsqrtf(sumsq / (float)D + eps);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = v[e] * inv * w[first + e];
+    }
+    uint32_t o4[4];
+    float r[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float other = __shfl_xor(v[e], LPH / 2, FE_WAVE);     // element first + e -/+ HALF
+      const int j = (first + e) & (HALF - 1);
+      r[e] = low ? v[e] * cos_s[j] - other * sin_s[j] : v[e] * cos_s[j] + other * sin_s[j];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o4[e] = (uint32_t)float_to_bf16(r[2 * e]) | ((uint32_t)float_to_bf16(r[2 * e + 1]) << 16);
+    bf16_t* dst = is_q ? x : key_pages + page + (size_t)slot * D + first;
+    *(uint4*)dst = make_uint4(o4[0], o4[1], o4[2], o4[3]);
+  }
+}
+
 extern "C" int fe_qk_norm_rope_write(void* qkv, int dtype, const float* q_weight, const float* k_weight,
                                      const float* inv_freq, const int* positions, const int* token_seq,
                                      const int* block_table, int table_stride, void* key_pages,
@@ -152,10 +240,25 @@ extern "C" int fe_qk_norm_rope_write(void* qkv, int dtype, const float* q_weight
   // few tokens: four heads a block, so that the launch has many blocks; many tokens: a block per
   // token, so that the angles' sines and cosines are computed once per token
   const int heads_all = q_heads + 2 * kv_heads;
-  const int heads_per_block = tokens >= 256 ? heads_all : 4;
+  const bool vec = dtype == FE_BF16 && rotary_dim == head_dim && (head_dim == 64 || head_dim == 128 || head_dim == 256) &&
+                   ((((uintptr_t)qkv) | ((uintptr_t)key_pages)) & 15) == 0;
+  // the vector kernel works on 2048 / head_dim heads at once
+  const int heads_per_block = tokens >= 256 ? heads_all : (vec ? 2048 / head_dim : 4);
   const int groups_per_token = (heads_all + heads_per_block - 1) / heads_per_block;
   const long long blocks = (long long)tokens * groups_per_token;
   if (blocks > 0x7fffffffLL) return FE_BAD_ARGUMENT;
+  if (vec) {
+#define FE_GO(LPH)                                                                                          \
+  qk_norm_rope_write_vec_kernel<LPH><<<(unsigned)blocks, 256, 0, stream>>>(                                   \
+      (bf16_t*)qkv, q_weight, k_weight, inv_freq, positions, token_seq, block_table, table_stride,            \
+      (bf16_t*)key_pages, (bf16_t*)value_pages, q_heads, kv_heads, block_size, num_blocks, eps, write_kv,     \
+      heads_per_block, groups_per_token)
+    if (head_dim == 64) FE_GO(8);
+    else if (head_dim == 128) FE_GO(16);
+    else FE_GO(32);
+#undef FE_GO
+    return fe_check_launch();
+  }
   if (dtype == FE_F32)
     qk_norm_rope_write_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>(
         (float*)qkv, q_weight, k_weight, inv_freq, positions, token_seq, block_table, table_stride,
