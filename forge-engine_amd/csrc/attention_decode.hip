@@ -45,7 +45,7 @@ __device__ __forceinline__ float load_agent(const float* p) {
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void paged_decode_kernel(
+__global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     float* part_o, float* part_ml, int* __restrict__ counters, const int* __restrict__ cu_q,
