@@ -26,7 +26,7 @@ class StepBatch:
     num_wanted: int
     max_q_len: int
     max_ctx: int
-    num_decode: int         # sequences that bring exactly one token
+    num_decode: int | None  # sequences that bring exactly one token (None: not known on the host)
     token_ids: Tensor       # int32 [T]
     positions: Tensor       # int32 [T]   absolute position of each token in its request
     token_seq: Tensor       # int32 [T]   index of the token's request within the batch
@@ -108,6 +108,32 @@ def build_batch(entries, lengths_before, state_slots, tables_per_group, device, 
         q_lens=q_lens, ctx_before_host=list(lengths_before), state_slots_host=list(state_slots))
 
 
-def static_batch_size(num_seqs: int, widths) -> int:
-    """int32 entries of a single-token batch of ``num_seqs`` requests."""
-    return 8 * num_seqs + 1 + num_seqs * sum(widths)
+def static_batch_size(num_seqs: int, widths, num_tokens: int | None = None, num_wanted: int | None = None) -> int:
+    """int32 entries of a batch of ``num_seqs`` requests (by default with one token and one
+    wanted row each)."""
+    tokens = num_seqs if num_tokens is None else num_tokens
+    wanted = num_seqs if num_wanted is None else num_wanted
+    return 3 * tokens + 4 * num_seqs + 1 + wanted + num_seqs * sum(widths)
+
+
+def static_batch(flat: Tensor, *, num_tokens: int, num_seqs: int, num_wanted: int, widths, max_q_len: int,
+                 max_ctx: int) -> StepBatch:
+    """The batch of a captured step: views into a device buffer at fixed addresses, laid out as
+    ``build_batch`` lays a batch out, for ``num_seqs`` sequences of which some may be empty.
+    What the kernels cannot read from the buffer is a bound (``max_q_len``, ``max_ctx``) or
+    unknown (how many sequences bring one token); the host-side lists are not filled in, so a
+    model with a part that reads them is not captured."""
+    sizes = [num_tokens, num_tokens, num_tokens, num_seqs + 1, num_seqs, num_seqs, num_seqs, num_wanted]
+    views, offset = [], 0
+    for size in sizes:
+        views.append(flat[offset:offset + size])
+        offset += size
+    block_tables = []
+    for width in widths:
+        block_tables.append(flat[offset:offset + num_seqs * width].view(num_seqs, width))
+        offset += num_seqs * width
+    return StepBatch(
+        num_tokens=num_tokens, num_seqs=num_seqs, num_wanted=num_wanted, max_q_len=max_q_len, max_ctx=max_ctx,
+        num_decode=None, token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
+        ctx_len=views[4], ctx_before=views[5], state_slots=views[6], want_rows=views[7],
+        block_tables=block_tables, request_ids=[], q_lens=[], ctx_before_host=[], state_slots_host=[])

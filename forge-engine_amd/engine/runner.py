@@ -14,11 +14,14 @@ from torch import Tensor
 from ..cache import CacheCapacityError, CacheManager, CacheView, plan_groups
 from ..kernels import library
 from ..models.decoder import DecoderModel
-from .batch import StepBatch, StepEntry, build_batch, static_batch_size
+from .batch import StepBatch, StepEntry, build_batch, static_batch, static_batch_size
 
 GRAPH_MAX_REQUESTS = 64      # decode steps of up to this many requests replay a captured graph
 GRAPH_TABLE_STEP = 64        # block-table widths of graphs are multiples of this many pages
 GRAPH_LIMIT = 24             # captured graphs kept (least recently used goes first)
+PORTION_GRAPH_MAX_TOKENS = 1024   # steps with prompt portions of up to this many tokens may be captured
+PORTION_GRAPH_SEQ_STEP = 8        # ... for a number of sequences rounded up to a multiple of this
+PORTION_GRAPH_WANT_STEP = 8       # ... and of wanted rows likewise (none stays none)
 
 
 class _DecodeGraph:
@@ -71,13 +74,77 @@ class _DecodeGraph:
                     keys[i] = key
 
 
+class _PortionGraph:
+    """One captured step that holds prompt portions (beside single tokens or not): fixed token
+    count, sequence count and wanted-row count rounded up, block-table widths rounded up.
+    Sequences beyond the step's own are empty (no tokens, so every kernel skips them), wanted
+    rows beyond the step's own repeat row 0 and are cut off the result."""
+
+    def __init__(self, num_tokens: int, num_seqs: int, num_wanted: int, widths, device) -> None:
+        size = static_batch_size(num_seqs, widths, num_tokens, num_wanted)
+        self.host = torch.empty(size, dtype=torch.int32).pin_memory()
+        self.dev = torch.zeros(size, dtype=torch.int32, device=device)
+        self.np = self.host.numpy()
+        self.np[:] = 0
+        self.t, self.b, self.w, self.widths = num_tokens, num_seqs, num_wanted, list(widths)
+        self.table_at = []
+        offset = 3 * num_tokens + 4 * num_seqs + 1 + num_wanted
+        for width in self.widths:
+            self.table_at.append(offset)
+            self.np[offset:offset + num_seqs * width] = -1
+            offset += num_seqs * width
+        self.graph = None
+        self.logits = None
+        self.copied = torch.cuda.Event()
+
+    def fill(self, entries, before, records) -> None:
+        t, b, w, buf = self.t, self.b, self.w, self.np
+        n = len(entries)
+        at = 0
+        cu = buf[3 * t:3 * t + b + 1]
+        want = buf[3 * t + 4 * b + 1:3 * t + 4 * b + 1 + w]
+        rows = 0
+        for i, entry in enumerate(entries):
+            count = len(entry.tokens)
+            buf[at:at + count] = entry.tokens
+            buf[t + at:t + at + count] = np.arange(before[i], before[i] + count)
+            buf[2 * t + at:2 * t + at + count] = i
+            cu[i] = at
+            for place in entry.want:
+                want[rows] = at + place
+                rows += 1
+            at += count
+        cu[n:] = at                                                   # the other sequences are empty
+        want[rows:] = 0
+        ctx = buf[3 * t + b + 1:3 * t + 2 * b + 1]
+        ctx[:n] = [before[i] + len(e.tokens) for i, e in enumerate(entries)]
+        ctx[n:] = 0
+        start = buf[3 * t + 2 * b + 1:3 * t + 3 * b + 1]
+        start[:n] = before
+        start[n:] = 0
+        slots = buf[3 * t + 3 * b + 1:3 * t + 4 * b + 1]
+        slots[:n] = [r.state_slot for r in records]
+        slots[n:] = 0
+        for g, width in enumerate(self.widths):
+            base = self.table_at[g]
+            for i, record in enumerate(records):
+                table = record.tables[g]
+                row = buf[base + i * width:base + (i + 1) * width]
+                row[:len(table)] = table
+                row[len(table):] = -1
+            buf[base + n * width:base + b * width] = -1
+
+
 class ModelRunner:
     def __init__(self, model: DecoderModel, *, block_size: int, block_capacity: int,
                  num_state_slots: int, use_graphs: bool = True) -> None:
         self.model = model
         self.use_graphs = use_graphs and model.ctx.device.type == "cuda" and model.graph_safe
         self._graphs: dict[tuple, _DecodeGraph] = {}
+        self._portion_graphs: dict[tuple, _PortionGraph] = {}
+        self._portion_seen: dict[tuple, int] = {}
         self.graph_replays = 0
+        self.portion_graph_replays = 0
         self.device = model.ctx.device
         self.dtype = model.ctx.dtype
         self.block_size = block_size
@@ -215,6 +282,70 @@ class ModelRunner:
         self.steps_run += 1
         return slot.logits
 
+    def _portion_key(self, entries: list[StepEntry]):
+        """The shape under which a step with prompt portions may be captured, or None."""
+        if not self.use_graphs or len(entries) > GRAPH_MAX_REQUESTS:
+            return None
+        tokens = sum(len(e.tokens) for e in entries)
+        if tokens > PORTION_GRAPH_MAX_TOKENS:
+            return None
+        seqs = -(-len(entries) // PORTION_GRAPH_SEQ_STEP) * PORTION_GRAPH_SEQ_STEP
+        wanted = sum(len(e.want) for e in entries)
+        wanted = -(-wanted // PORTION_GRAPH_WANT_STEP) * PORTION_GRAPH_WANT_STEP
+        return tokens, seqs, wanted
+
+    def _portion_graph_step(self, entries: list[StepEntry], shape) -> Tensor | None:
+        """A step with prompt portions as a replay of a captured graph, once its shape (token
+        count, sequence and wanted-row counts rounded up, table widths rounded up) has come
+        before: a scheduler that fills its token budget repeats few shapes.  None if the step
+        is to run eagerly (first sighting of a shape)."""
+        cache = self.cache
+        self._check(entries)
+        records = [cache.request(e.request_id) for e in entries]
+        before = [r.length for r in records]
+        groups = range(len(cache.groups))
+        after = [b + len(e.tokens) for b, e in zip(before, entries)]
+        pages = -(-max(after) // self.block_size)
+        widths = tuple(-(-pages // GRAPH_TABLE_STEP) * GRAPH_TABLE_STEP for _ in groups)
+        key = (*shape, widths)
+        slot = self._portion_graphs.pop(key, None)
+        if slot is None:
+            seen = self._portion_seen.pop(key, 0)
+            if len(self._portion_seen) >= 4 * GRAPH_LIMIT:
+                self._portion_seen.pop(next(iter(self._portion_seen)))
+            self._portion_seen[key] = seen + 1
+            if seen == 0:
+                return None
+            if len(self._portion_graphs) >= GRAPH_LIMIT:
+                self._portion_graphs.pop(next(iter(self._portion_graphs)))
+            slot = _PortionGraph(shape[0], shape[1], shape[2], widths, self.device)
+        self._portion_graphs[key] = slot
+        cache.reserve({e.request_id: n for e, n in zip(entries, after)})
+        records = [cache.request(e.request_id) for e in entries]
+        slot.copied.synchronize()
+        slot.fill(entries, before, records)
+        slot.dev.copy_(slot.host, non_blocking=True)
+        slot.copied.record(torch.cuda.current_stream(self.device))
+        if slot.graph is None:
+            batch = static_batch(slot.dev, num_tokens=shape[0], num_seqs=shape[1], num_wanted=shape[2],
+                                 widths=widths, max_q_len=shape[0], max_ctx=widths[0] * self.block_size if widths else 0)
+            views = self.cache_views(batch)
+            side = torch.cuda.Stream(device=self.device)
+            side.wait_stream(torch.cuda.current_stream(self.device))
+            with torch.cuda.stream(side):      # once eagerly: libraries load, scratch gets its size
+                self.model.forward(batch, views)
+            torch.cuda.current_stream(self.device).wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                slot.logits = self.model.forward(batch, views)
+            slot.graph, slot.views, slot.batch = graph, views, batch
+        slot.graph.replay()
+        self.portion_graph_replays += 1
+        for entry, length in zip(entries, after):
+            cache.commit(entry.request_id, length)
+        self.steps_run += 1
+        return slot.logits[:sum(len(e.want) for e in entries)]
+
     @torch.inference_mode()
     def step(self, entries: list[StepEntry]) -> Tensor:
         """Run the entries' tokens as one batch; float32 logits [wanted, vocab]
@@ -224,6 +355,11 @@ class ModelRunner:
         of the same shape overwrites."""
         if self._graphable(entries):
             return self._graph_step(entries)
+        shape = self._portion_key(entries) if entries else None
+        if shape is not None:
+            logits = self._portion_graph_step(entries, shape)
+            if logits is not None:
+                return logits
         batch = self.prepare(entries)
         logits = self.model.forward(batch, self.cache_views(batch))
         for i, entry in enumerate(entries):

@@ -137,6 +137,51 @@ def test_long_decoding_through_graphs_matches_eager_and_plain(dtype, folders):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_steps_with_portions_replay_captured_graphs(name, dtype, folders):
+    """A scheduler that fills its token budget repeats few step shapes; such steps (prompt portions
+    beside decoded tokens) are captured on their second sighting and replayed.  Requests come and go
+    (pages and sequence slots of the captured shape are reused, padded sequences stay empty), every
+    position's logits are wanted and compared with the plain implementation, with and without graphs."""
+    config = TINY[name]
+    block = BLOCK_SIZE[name]
+    requests = ru.make_requests(config, 41, (37, 52, 23, 44, 31, 18))
+    want = ru.plain_logits(folders[name], requests)
+    _, model = load_model(folders[name], dtype=dtype, device=DEV)
+    for graphs in (True, False):
+        runner = ModelRunner(model, block_size=block, block_capacity=3 * (60 // block + 2), num_state_slots=3,
+                             use_graphs=graphs)
+        waiting = list(requests)
+        live, at, got = [], {}, {}
+        while waiting or live:
+            while waiting and len(live) < 3:          # at most three live: pages are used again
+                k = waiting.pop(0)
+                runner.begin(k)
+                live.append(k)
+                at[k] = 0
+            entries = []
+            for k in live:
+                tokens = requests[k]
+                # portions of 6 tokens; the last 5 tokens of a request come one by one beside them
+                size = 6 if at[k] + 6 <= len(tokens) - 5 else (len(tokens) - 5 - at[k] if at[k] < len(tokens) - 5 else 1)
+                entries.append(StepEntry(k, tokens[at[k]:at[k] + size], list(range(size))))
+            logits = runner.step(entries).cpu()
+            row = 0
+            for e in entries:
+                for i in range(len(e.tokens)):
+                    got[(e.request_id, at[e.request_id] + i)] = logits[row + i].clone()
+                row += len(e.tokens)
+                at[e.request_id] += len(e.tokens)
+            for k in [k for k in live if at[k] == len(requests[k])]:
+                runner.end(k)
+                live.remove(k)
+        assert runner.cache.allocated_pages == 0
+        runner.cache.check_invariants()
+        assert (runner.portion_graph_replays >= 5) == graphs
+        ru.compare(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_first_tokens_of_a_sequence(name, dtype, folders):
     """Position 0 alone, then 1, 2, 3: the shortest contexts, one page, first slots."""
     config = TINY[name]
