@@ -35,9 +35,14 @@ typedef __attribute__((ext_vector_type(4))) float floatx4;
 typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 
 #define BN 64        // keys per tile
-#define KPAD 8       // bf16 padding of a key row in LDS
+#define KPAD 0       // key rows are not padded: their 16-byte chunks are swizzled instead (see key_swizzle)
 #define VPAD 8       // bf16 padding of a value row (one dim, 64 keys) in LDS
 #define XCDS 8
+
+// Chunk c (16 bytes) of key row r lives at chunk position c ^ swizzle(r) of the row.  The 16 lanes
+// that read one chunk index together hold rows 8a + b (+ 4h), a < 4, b < 4, which a padded row
+// stride cannot spread over all banks (rows 8 apart always collide); 4a + b is distinct for them.
+__device__ __forceinline__ int key_swizzle(int row, int chunks) { return (((row >> 3) & 3) * 4 + (row & 3)) & (chunks - 1); }
 
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 __device__ __forceinline__ unsigned int pack_bf16(float lo, float hi) {
@@ -46,7 +51,7 @@ __device__ __forceinline__ unsigned int pack_bf16(float lo, float hi) {
 }
 
 template <int D, int RT>
-__global__ __launch_bounds__(256) void paged_prefill_kernel(
+__global__ __launch_bounds__(256, RT == 1 ? 2 : 1) void paged_prefill_kernel(
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
@@ -116,7 +121,7 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
       {
         const int key = tile * BN + (p % 8) * 8;     // p % 8 == tid % 8: 256 is a multiple of 8
         const uintx4 v = *(const uintx4*)(value_pages + ((((size_t)ids.v * kv_heads + hk) * D + p / 8) << block_shift) + (key & block_mask));
-        vreg[i] = key < ctx ? v : uintx4{0u, 0u, 0u, 0u};
+        vreg[i] = (tile * BN + BN <= ctx || key < ctx) ? v : uintx4{0u, 0u, 0u, 0u};
       }
     }
   };
@@ -124,7 +129,7 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int p = tid + i * 256;
-      *(uintx4*)&Ks[stage][p / CH][(p % CH) * 8] = kreg[i];
+      *(uintx4*)&Ks[stage][p / CH][((p % CH) ^ key_swizzle(p / CH, CH)) * 8] = kreg[i];
       *(uintx4*)&Vt[stage][p / 8][(p % 8) * 8] = vreg[i];
     }
   };
@@ -180,21 +185,17 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(
       if (key_base > wave_lo + RT * 16 - 1) return;   // every key of the tile lies after this wave's rows
       floatx4 st[RT][2][2];
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-          for (int h = 0; h < 2; ++h) st[rt][blk][h] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
       for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
           for (int c = 0; c < KC; ++c) {
-            const bf16x8 ka = *(const bf16x8*)&Ks[stage][blk * 32 + krow + 4 * h][c * 32 + lq * 8];
+            const int row = blk * 32 + krow + 4 * h;
+            const bf16x8 ka = *(const bf16x8*)&Ks[stage][row][((c * 4 + lq) ^ key_swizzle(row, CH)) * 8];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
-              st[rt][blk][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qb[rt][c], st[rt][blk][h], 0, 0, 0);
+              st[rt][blk][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  ka, qb[rt][c], c == 0 ? floatx4{0.f, 0.f, 0.f, 0.f} : st[rt][blk][h], 0, 0, 0);
           }
       // lane (lr = query row, lq): st[rt][blk][h][i] = score of key key_base + 32 blk + 8lq + 4h + i
       const bool edge = key_base + BN - 1 > wave_lo || (window > 0 && key_base < pos_hi - window + 1);
