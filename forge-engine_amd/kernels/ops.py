@@ -250,15 +250,44 @@ UPDATE_SPLIT_MIN_STEPS = 32
 UPDATE_SPLITS = 4
 
 
+# Between 17 and 64 rows the product is still bound by the weight's bytes; the matrix library needs
+# 21 us for each of the two projections back to the hidden size at 64 rows (1 to 2.4 TB/s).  The
+# kernel below splits K over blocks of 64 weight rows, aiming at this many blocks.
+MID_ROWS = 64
+MID_TARGET_BLOCKS = 512
+
+
+def gemm_mid_parts(x: Tensor, weight: Tensor, parts: int) -> Tensor:
+    """Partial sums [parts, M, N] (float32) of x @ weight^T over ``parts`` runs of whole 128-steps
+    of K, for up to 64 rows of bfloat16 x."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(weight, "weight", torch.bfloat16, contiguous=False)
+    if not _skinny_fits(x, weight, MID_ROWS) or weight.shape[1] != x.shape[1] or not 1 <= parts <= 64:
+        raise KernelError("the product in parts takes at most 64 contiguous bfloat16 rows, K a multiple of 8, at most 64 parts")
+    m, k = x.shape
+    n = weight.shape[0]
+    out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
+    _call("gemm_mid", "fe_gemm_mid_parts", _ptr(x), _ptr(weight), _ptr(out), c_int(m), c_int(n), c_int(k),
+          c_longlong(weight.stride(0)), c_longlong(n), c_int(parts), c_longlong(m * n), _stream())
+    return out
+
+
 def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
     """The float32 product x @ weight^T (+ bias) as an update of the residual stream: [M, N], or
     partial sums [parts, M, N] that ``add_rmsnorm`` / ``add_rows`` add up."""
     _gpu(x, "x")
     _gpu(weight, "weight", contiguous=False)
-    if (bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and _skinny_fits(x, weight)
+    plain_bf16 = bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+    if (plain_bf16 and _skinny_fits(x, weight)
             and -(-weight.shape[0] // 16) <= UPDATE_SPLIT_MAX_TILES
             and -(-weight.shape[1] // 128) >= UPDATE_SPLIT_MIN_STEPS):
         return gemm_skinny(x, weight, "f32", tiles=1, waves=8, splits=UPDATE_SPLITS)
+    if plain_bf16 and x.shape[0] > SKINNY_MAX_ROWS and _skinny_fits(x, weight, MID_ROWS):
+        steps = -(-weight.shape[1] // 128)
+        blocks = -(-weight.shape[0] // 64)
+        parts = max(1, min(16, MID_TARGET_BLOCKS // blocks, steps // 2))
+        parts = -(-steps // -(-steps // parts))          # no part without steps
+        return gemm_mid_parts(x, weight, parts)
     return linear(x, weight, bias, out_dtype=torch.float32)
 
 
@@ -467,4 +496,4 @@ def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index:
           _stream())
 
 
-LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")
+LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")

@@ -48,7 +48,7 @@ class SwiGLU(FeedForward):
         return ops.linear_update(act, self.down_weight)   # the update stays float32 for the residual sum
 
     def kernel_libraries(self):
-        return {"rowwise", "gemm_f32", "gemm_skinny"}
+        return {"rowwise", "gemm_f32", "gemm_skinny", "gemm_mid"}
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

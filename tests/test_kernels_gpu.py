@@ -450,10 +450,50 @@ def test_linear_update_routes(ops):
     assert ops.linear_update(x, few_rows).dim() == 3              # few row tiles, long K: parts
     assert ops.linear_update(x, many_rows).dim() == 2
     assert ops.linear_update(x[:, :1024].contiguous(), few_rows[:, :1024]).dim() == 2
-    big = rand(g, 40, 4096, dtype=torch.bfloat16).to(DEV)
-    assert ops.linear_update(big, few_rows).shape == (40, 320)     # beyond 16 rows: the library
+    big = rand(g, 70, 4096, dtype=torch.bfloat16).to(DEV)
+    assert ops.linear_update(big, few_rows).shape == (70, 320)     # beyond 64 rows: the library
     want = x.float().cpu() @ few_rows.float().cpu().T
     torch.testing.assert_close(ops.linear_update(x, few_rows).sum(0).cpu(), want, atol=1e-3, rtol=1e-3)
+
+
+@pytest.mark.parametrize("m", [17, 33, 48, 64, 5])
+@pytest.mark.parametrize("n,k,parts", [(2560, 4096, 8), (2560, 9728, 9), (200, 264, 2), (1003, 1000, 3), (64, 128, 1), (70, 8, 1)])
+def test_gemm_mid_parts(ops, m, n, k, parts):
+    """17 to 64 rows: K in parts over blocks of 64 weight rows, x staged through LDS; the parts add
+    up to the product, each row independent of the rows beside it, the same bits every time."""
+    g = torch.Generator().manual_seed(26)
+    x = rand(g, m, k, dtype=torch.bfloat16).to(DEV)
+    w = rand(g, n, k, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    got = ops.gemm_mid_parts(x, w, parts)
+    assert got.shape == (parts, m, n)
+    want = x.float().cpu() @ w.float().cpu().T
+    bound = 2e-6 * float(want.abs().max()) * math.sqrt(k) + 1e-6
+    assert float((got.sum(0).cpu() - want).abs().max()) <= bound
+    assert torch.equal(ops.gemm_mid_parts(x, w, parts), got)
+    alone = ops.gemm_mid_parts(x[2:3].contiguous(), w, parts)
+    assert torch.equal(alone[:, 0], got[:, 2])
+    # a padded weight (row stride beyond K) and what the residual stream does with the parts
+    wide = torch.zeros(n, k + 8, dtype=torch.bfloat16, device=DEV)
+    wide[:, :k] = w
+    assert torch.equal(ops.gemm_mid_parts(x, wide[:, :k], parts), got)
+    h = rand(g, m, n).to(DEV)
+    h1, h2 = h.clone(), h.clone()
+    summed = got[0].clone()
+    for part in got[1:]:
+        summed += part
+    assert torch.equal(ops.add_rows(h1, got), ops.add_rows(h2, summed))
+
+
+def test_linear_update_takes_the_mid_kernel(ops):
+    g = torch.Generator().manual_seed(27)
+    w = rand(g, 2560, 4096, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    for rows in (17, 40, 64):
+        x = rand(g, rows, 4096, dtype=torch.bfloat16).to(DEV)
+        update = ops.linear_update(x, w)
+        assert update.dim() == 3 and update.shape[1:] == (rows, 2560)
+        want = x.float().cpu() @ w.float().cpu().T
+        torch.testing.assert_close(update.sum(0).cpu(), want, atol=2e-3, rtol=2e-3)
+    assert ops.linear_update(rand(g, 65, 4096, dtype=torch.bfloat16).to(DEV), w).dim() == 2
 
 
 def test_linear_routes_by_rows_and_dtype(ops):
