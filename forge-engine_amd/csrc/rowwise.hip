@@ -114,13 +114,13 @@ __global__ __launch_bounds__(256) void add_rmsnorm_regs_kernel(
       v[j] = load4_as_float(hrow + i);
       if (drow) {
         float4 d = load4_as_float(drow + i);
-        for (int k = 1; k < parts; k += 4) {     // four parts' loads fly together; added in order
-          float4 e[4];
+        for (int k = 1; k < parts; k += 8) {     // eight parts' loads fly together; added in order
+          float4 e[8];
 #pragma unroll
-          for (int u = 0; u < 4; ++u)
+          for (int u = 0; u < 8; ++u)
             e[u] = k + u < parts ? load4_as_float(drow + (k + u) * part_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-          for (int u = 0; u < 4; ++u)
+          for (int u = 0; u < 8; ++u)
             if (k + u < parts) { d.x += e[u].x; d.y += e[u].y; d.z += e[u].z; d.w += e[u].w; }
         }
         v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
