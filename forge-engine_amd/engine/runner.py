@@ -351,8 +351,8 @@ class ModelRunner:
         """Run the entries' tokens as one batch; float32 logits [wanted, vocab]
         in the order of the entries and of each entry's ``want``.  Raises
         ``CacheCapacityError`` (and changes nothing) if pages run out.  The
-        result of a decode-only step lives in a buffer that the next such step
-        of the same shape overwrites."""
+        result of a step that replays a captured graph lives in a buffer that
+        the next step of the same shape overwrites."""
         if self._graphable(entries):
             return self._graph_step(entries)
         shape = self._portion_key(entries) if entries else None

@@ -77,6 +77,32 @@ def test_greedy_generation_through_the_entry_point(name, dtype, folders):
     assert list(single.stream(prompts[1])) == outputs[1]
 
 
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_scheduler_under_page_pressure_on_the_gpu(name, folders):
+    """Twelve requests of random lengths through the scheduler with too few pages for all of them
+    (requests are preempted and recomputed), portions of prompts beside decoded tokens, decode and
+    portion graphs: in float32 every request generates what it generates alone in the plain
+    implementation, and every page comes back."""
+    import random
+    config, weights = TINY[name], folder_weights(folders[name])
+    rng = random.Random(51)
+    lengths = [rng.randrange(3, 40) for _ in range(12)]
+    prompts = list(ru.make_requests(config, 52, lengths).values())
+    new_tokens = [rng.randrange(4, 14) for _ in prompts]
+    block = BLOCK_SIZE[name]
+    capacity = 3 * (-(-(max(lengths) + 14) // block)) + 2        # room for about three requests
+    scheduler = SchedulerConfig(block_size=block, block_capacity=capacity, token_budget=24, max_batch_size=6,
+                                max_requests=16, prefill_chunk=16, admission="preempt")
+    engine = engine_from_folder(folders[name], scheduler_config=scheduler, dtype="float32")
+    ids = [engine.submit(p, sampling_params=SamplingParams(max_new_tokens=n)) for p, n in zip(prompts, new_tokens)]
+    engine.run_until_idle()
+    assert engine.snapshot().preemptions >= 1
+    assert engine.cache_pool.allocated_pages == 0
+    for request_id, prompt, n in zip(ids, prompts, new_tokens):
+        got = list(engine.request(request_id).output_token_ids)
+        assert got == plain.greedy_generate(weights, config, prompt, n), request_id
+
+
 def test_command_line_generates(folders, capsys):
     from forge_engine_amd.cli import main
     prompt = [5, 17, 3, 200, 9]
