@@ -94,8 +94,8 @@ __device__ __forceinline__ void store4_from_float(bf16_t* p, float4 v) {
   *(uint2*)p = u;
 }
 
-template <typename TD, typename TO, int VEC>
-__global__ __launch_bounds__(256) void add_rmsnorm_regs_kernel(
+template <typename TD, typename TO, int VEC, int THREADS>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_regs_kernel(
     float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ w,
     TO* __restrict__ out, const int* __restrict__ rows, int hidden, float eps, int store_sum,
     int parts, size_t part_stride) {
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_regs_kernel(
   float sumsq = 0.f;
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    const int i = (threadIdx.x + j * 256) * 4;
+    const int i = (threadIdx.x + j * THREADS) * 4;
     v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (i < hidden) {
       v[j] = load4_as_float(hrow + i);
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_regs_kernel(
   TO* orow = out + (size_t)r * hidden;
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    const int i = (threadIdx.x + j * 256) * 4;
+    const int i = (threadIdx.x + j * THREADS) * 4;
     if (i < hidden) {
       const float4 ww = *(const float4*)(w + i);
       store4_from_float(orow + i, make_float4(v[j].x * inv * ww.x, v[j].y * inv * ww.y,
@@ -148,12 +148,14 @@ static void launch_add_rmsnorm_typed(float* h, const TD* delta, const float* w, 
                                      int n_rows, int hidden, float eps, int store_sum, int parts,
                                      size_t part_stride, hipStream_t stream) {
   const bool aligned = hidden % 4 == 0 && part_stride % 4 == 0 && (((uintptr_t)h | (uintptr_t)delta | (uintptr_t)w | (uintptr_t)out) & 15) == 0;
-  if (aligned && hidden <= 1024)
-    add_rmsnorm_regs_kernel<TD, TO, 1><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
+  if (aligned && n_rows <= 16 && hidden > 1024 && hidden <= 4096)   // few rows: a whole row in flight at once
+    add_rmsnorm_regs_kernel<TD, TO, 1, 1024><<<n_rows, 1024, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
+  else if (aligned && hidden <= 1024)
+    add_rmsnorm_regs_kernel<TD, TO, 1, 256><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
   else if (aligned && hidden <= 4096)
-    add_rmsnorm_regs_kernel<TD, TO, 4><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
+    add_rmsnorm_regs_kernel<TD, TO, 4, 256><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
   else if (aligned && hidden <= 8192)
-    add_rmsnorm_regs_kernel<TD, TO, 8><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
+    add_rmsnorm_regs_kernel<TD, TO, 8, 256><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
   else {
     const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
     add_rmsnorm_kernel<TD, TO><<<n_rows, threads, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);

@@ -44,16 +44,17 @@ def test_embed_rows(ops, dtype, hidden):
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("delta_dtype", [None, torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hidden", [24, 200, 2560, 5000])
-def test_add_rmsnorm(ops, out_dtype, delta_dtype, hidden):
+@pytest.mark.parametrize("n", [7, 23])          # few rows of a wide stream take a kernel with more threads a row
+def test_add_rmsnorm(ops, out_dtype, delta_dtype, hidden, n):
     g = torch.Generator().manual_seed(1)
-    h = rand(g, 7, hidden, scale=3.0)
-    delta = None if delta_dtype is None else rand(g, 7, hidden, dtype=delta_dtype)
+    h = rand(g, n, hidden, scale=3.0)
+    delta = None if delta_dtype is None else rand(g, n, hidden, dtype=delta_dtype)
     w = 1.0 + rand(g, hidden, scale=0.1)
     h_ref = h.clone()
-    want = refs.add_rmsnorm(h_ref, delta, w, 1e-5, torch.empty(7, hidden, dtype=out_dtype))
+    want = refs.add_rmsnorm(h_ref, delta, w, 1e-5, torch.empty(n, hidden, dtype=out_dtype))
     h_dev = h.to(DEV)
     got = ops.add_rmsnorm(h_dev, None if delta is None else delta.to(DEV), w.to(DEV), 1e-5,
-                          torch.empty(7, hidden, dtype=out_dtype, device=DEV))
+                          torch.empty(n, hidden, dtype=out_dtype, device=DEV))
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol(out_dtype))
     torch.testing.assert_close(h_dev.cpu(), h_ref, atol=1e-6, rtol=1e-6)   # the sum went back into the stream
 
