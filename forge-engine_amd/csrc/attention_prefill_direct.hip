@@ -1,0 +1,291 @@
+// Paged grouped-query attention for portions of prompts, bfloat16 cache, with
+// keys and values loaded from global memory straight into LDS.
+//
+// Same arithmetic as the staged kernel (attention_prefill.hip): a block is 64
+// query rows of one head, four waves of 16 rows, keys walked in tiles of 64;
+// S^T = K Q^T and O^T = V^T P^T on MFMA 16x16x32, softmax statistics in
+// float32.  What differs is how a tile reaches LDS: `global_load_lds_dwordx4`
+// writes 64 lanes x 16 bytes at consecutive LDS addresses without passing
+// through registers, so the kernel needs no staging registers (a third and a
+// fourth wave fit a SIMD) and no LDS store instructions.  Which global bytes a
+// lane loads is free, which LDS address they land at is not; hence
+//   keys    LDS unit u = 16-byte chunk position u % CH of key row u / CH holds
+//           chunk (u % CH) ^ swizzle(row) of that row (conflict-free reads for the
+//           interleaved rows of the MFMA operand, coalesced 256-byte rows in memory);
+//   values  LDS unit u = dim u % D of key chunk u / D (8 keys): the 16 lanes that
+//           read one chunk of 16 dims hit 16 neighbouring units.
+// A wave loads the 16 keys 16w .. 16w+15 of a tile and their values: one page a
+// wave and tile (pages hold at least 16 keys), its id fetched a tile ahead by a
+// scalar load.  One LDS buffer for keys and one for values, two barriers a tile:
+// once every wave has its scores, the tile's values and the next tile's keys are
+// requested and fly during the softmax; they are waited for before the second
+// product.
+//
+// Keys at or beyond the context read the bytes of the last key instead (their
+// scores are masked; their probabilities are zero).  Pages must hold finite
+// values in every slot of a page in use (the engine's pages start as zeros).
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+#define BN 64        // keys per tile
+#define XCDS 8
+
+__device__ __forceinline__ unsigned int pack_bf16(float lo, float hi) {
+  const bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(unsigned int, v);
+}
+
+// rows 8a + b (+ 4h) are read together: 4a + b is distinct for them
+__device__ __forceinline__ int key_swizzle(int row, int chunks) { return (((row >> 3) & 3) * 4 + (row & 3)) & (chunks - 1); }
+
+// wait until at most n of this wave's vector memory operations are outstanding (n < 16)
+#define FE_WAIT_VMEM(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (0x7 << 4) | (0xF << 8))
+
+__device__ __forceinline__ void load_to_lds(const void* global, void* lds) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)global,
+                                   (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+}
+
+template <int D>
+__global__ __launch_bounds__(256, 4) void paged_prefill_direct_kernel(
+    const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
+    const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
+    const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
+    int table_stride, int kv_heads, int groups, int block_shift, int num_blocks, int window,
+    float scale_log2, int q_tiles, int pairs, int pairs_per_xcd) {
+  const int block_mask = (1 << block_shift) - 1;
+  constexpr int BM = 64;
+  constexpr int KC = D / 32;            // MFMA k-steps over the head dim (scores)
+  constexpr int DT = D / 16;            // 16-dim tiles of the output
+  constexpr int CH = D / 8;             // 16-byte chunks per key row
+  constexpr int KI = BN * CH / 256;     // key load instructions per wave and tile
+  constexpr int VI = 8 * D / 256;       // value load instructions per wave and tile
+  __shared__ __attribute__((aligned(16))) uintx4 Ks[BN * CH];
+  __shared__ __attribute__((aligned(16))) uintx4 Vs[8 * D];
+
+  // Block id b runs on XCD b % 8.  An XCD, with its own L2, takes a run of neighbouring (sequence,
+  // head) pairs, which share keys and values; within the XCD the blocks are ordered by row tile,
+  // the last (the longest walk over the keys) first, so that the blocks a CU holds at a time are
+  // a mix of long and short walks and the long ones start early.
+  const int heads = kv_heads * groups;
+  const int local = blockIdx.x / XCDS;
+  const int pair = (blockIdx.x % XCDS) * pairs_per_xcd + local % pairs_per_xcd;
+  if (pair >= pairs) return;
+  const int q_tile = q_tiles - 1 - local / pairs_per_xcd;
+  const int seq = pair / heads;
+  const int head = pair - seq * heads;
+  const int hk = head / groups;
+  const int q0 = cu_q[seq];
+  const int q_len = cu_q[seq + 1] - q0;
+  const int row0 = q_tile * BM;
+  if (q_len < 2 || row0 >= q_len) return;
+  const int ctx = ctx_len[seq];
+  const int before = ctx - q_len;
+  const int* table = block_table + (size_t)seq * table_stride;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, lq = lane >> 4;
+  const int krow = 8 * (lr >> 2) + (lr & 3);   // MFMA row r of key tile h is key 8*(r/4) + 4h + r%4 of its 32-key block
+
+  // this wave's query rows as B operands: lane (lr = row, lq) holds q[row][32c + 8lq .. +8]
+  bf16x8 qb[KC];
+  const int row = row0 + wave * 16 + lr;
+  const int row_pos = before + row;
+  {
+    const bf16_t* qrow = q + (size_t)(q0 + min(row, q_len - 1)) * q_stride + (size_t)head * D;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const uintx4 v = *(const uintx4*)(qrow + c * 32 + lq * 8);
+      qb[c] = __builtin_bit_cast(bf16x8, row < q_len ? v : uintx4{0u, 0u, 0u, 0u});
+    }
+  }
+  float m_run = -INFINITY, l_run = 0.f;
+  floatx4 o[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t) o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int last_row = min(q_len, row0 + BM) - 1;
+  const int pos_lo = before + row0, pos_hi = before + last_row;
+  const int wave_lo = pos_lo + wave * 16;
+  const int k_first = window > 0 ? max(0, pos_lo - window + 1) : 0;
+  const int tile_first = k_first / BN, tile_last = pos_hi / BN;   // inclusive
+  const int last_key = ctx - 1;
+
+  // the page of this wave's 16 keys of a tile (uniform over the wave)
+  auto page_of = [&](int tile) -> int {
+    const int key = min(tile * BN + 16 * wave, last_key);
+    const int id = table[key >> block_shift];
+    return (id >= 0 && id < num_blocks) ? id : 0;
+  };
+  // per-lane constants of the loaders
+  int k_row[KI], k_chunk[KI], v_dim[VI], v_first[VI];
+#pragma unroll
+  for (int i = 0; i < KI; ++i) {
+    const int u = (wave * KI + i) * 64 + lane;
+    k_row[i] = u / CH;
+    k_chunk[i] = (u % CH) ^ key_swizzle(u / CH, CH);
+  }
+#pragma unroll
+  for (int i = 0; i < VI; ++i) {
+    const int u = (wave * VI + i) * 64 + lane;
+    v_dim[i] = u % D;
+    v_first[i] = (u / D) * 8;         // first key of the chunk within the tile
+  }
+  auto load_keys = [&](int tile, int page) {
+    const size_t base = ((size_t)page * kv_heads + hk) << block_shift;
+#pragma unroll
+    for (int i = 0; i < KI; ++i) {
+      const int key = min(tile * BN + k_row[i], last_key);
+      load_to_lds(key_pages + (base + (key & block_mask)) * D + k_chunk[i] * 8, &Ks[(wave * KI + i) * 64]);
+    }
+  };
+  auto load_values = [&](int tile, int page) {
+    const size_t base = ((size_t)page * kv_heads + hk) * D;
+#pragma unroll
+    for (int i = 0; i < VI; ++i) {
+      const int key = min(tile * BN + v_first[i], last_key & ~7);
+      load_to_lds(value_pages + ((base + v_dim[i]) << block_shift) + (key & block_mask), &Vs[(wave * VI + i) * 64]);
+    }
+  };
+
+  int page = page_of(tile_first);
+  load_keys(tile_first, page);
+  int page_next = tile_first < tile_last ? page_of(tile_first + 1) : 0;
+  FE_WAIT_VMEM(0);
+  __syncthreads();               // the first tile's keys are in LDS
+  for (int tile = tile_first; tile <= tile_last; ++tile) {
+    const bool more = tile < tile_last;
+    const int key_base = tile * BN;
+    const bool mine = key_base <= wave_lo + 15;     // some key of the tile is visible to this wave's rows
+    floatx4 st[2][2];
+    if (mine) {
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int c = 0; c < KC; ++c) {
+            const int r = blk * 32 + krow + 4 * h;
+            const bf16x8 ka = __builtin_bit_cast(bf16x8, Ks[r * CH + ((c * 4 + lq) ^ key_swizzle(r, CH))]);
+            st[blk][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                ka, qb[c], c == 0 ? floatx4{0.f, 0.f, 0.f, 0.f} : st[blk][h], 0, 0, 0);
+          }
+    }
+    // Every wave has its scores, and multiplied the tile before: both buffers are free.  This
+    // tile's values and the next tile's keys are requested now and fly during the softmax.
+    __syncthreads();
+    load_values(tile, page);
+    if (more) {
+      load_keys(tile + 1, page_next);
+      page = page_next;
+      if (tile + 2 <= tile_last) page_next = page_of(tile + 2);
+    }
+    bf16x8 pb[2];
+    if (mine) {
+      // lane (lr = query row, lq): st[blk][h][i] = score of key key_base + 32 blk + 8lq + 4h + i
+      const bool edge = key_base + BN - 1 > wave_lo || (window > 0 && key_base < pos_hi - window + 1);
+      float s[16];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        float v = st[j >> 3][(j >> 2) & 1][j & 3];
+        if (edge) {
+          const int key = key_base + 32 * (j >> 3) + 8 * lq + (j & 7);
+          const bool visible = key <= row_pos && (window <= 0 || key > row_pos - window);
+          v = visible ? v : -INFINITY;
+        }
+        s[j] = v;
+        mx = fmaxf(mx, v);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, FE_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, FE_WAVE));
+      const float m_new = fmaxf(m_run, mx * scale_log2);   // the scale is positive
+      const float m_use = m_new > -INFINITY ? m_new : 0.f; // a row with nothing visible yet
+      const float corr = __builtin_amdgcn_exp2f(m_run - m_use);
+      float sum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        s[j] = __builtin_amdgcn_exp2f(fmaf(s[j], scale_log2, -m_use));
+        sum += s[j];
+      }
+      sum += __shfl_xor(sum, 16, FE_WAVE);
+      sum += __shfl_xor(sum, 32, FE_WAVE);
+      l_run = l_run * corr + sum;
+      m_run = m_new;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        uintx4 pw;
+        pw.x = pack_bf16(s[8 * blk + 0], s[8 * blk + 1]); pw.y = pack_bf16(s[8 * blk + 2], s[8 * blk + 3]);
+        pw.z = pack_bf16(s[8 * blk + 4], s[8 * blk + 5]); pw.w = pack_bf16(s[8 * blk + 6], s[8 * blk + 7]);
+        pb[blk] = __builtin_bit_cast(bf16x8, pw);
+      }
+      if (__any(corr != 1.f)) {
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[t][i] *= corr;
+      }
+    }
+    FE_WAIT_VMEM(0);
+    __syncthreads();             // the values (and the next keys) are in LDS
+    if (mine) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+          const bf16x8 va = __builtin_bit_cast(bf16x8, Vs[(blk * 4 + lq) * D + t * 16 + lr]);
+          o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[blk], o[t], 0, 0, 0);
+        }
+    }
+  }
+
+  // lane (lr = query row, lq) holds O^T[16t + 4lq + i][row]: four consecutive dims per store
+  if (row < q_len) {
+    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    bf16_t* orow = out + (size_t)(q0 + row) * out_stride + (size_t)head * D;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      uint2 w;
+      w.x = pack_bf16(o[t][0] * inv, o[t][1] * inv);
+      w.y = pack_bf16(o[t][2] * inv, o[t][3] * inv);
+      *(uint2*)(orow + t * 16 + lq * 4) = w;
+    }
+  }
+}
+
+// Pages: keys [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size];
+// block_size a power of two >= 16; head_dim 64 or 128.  Sequences with fewer than two query tokens
+// are skipped.
+extern "C" int fe_paged_attention_prefill_direct(const void* q, long long q_stride, const void* key_pages,
+                                                 const void* value_pages, void* out, long long out_stride,
+                                                 const int* cu_q, const int* ctx_len, const int* block_table,
+                                                 int table_stride, int num_seqs, int max_q_len, int kv_heads,
+                                                 int groups, int head_dim, int block_size, int num_blocks,
+                                                 int window, float scale, hipStream_t stream) {
+  if (num_seqs <= 0 || max_q_len < 2) return FE_OK;
+  if (head_dim != 64 && head_dim != 128) return FE_BAD_ARGUMENT;
+  if (groups < 1 || kv_heads < 1 || num_seqs > 65535) return FE_BAD_ARGUMENT;
+  if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1 || q_stride % 8 || out_stride % 4) return FE_BAD_ARGUMENT;
+  if ((((uintptr_t)key_pages) | ((uintptr_t)value_pages) | ((uintptr_t)q)) & 15) return FE_BAD_ARGUMENT;
+  const float scale_log2 = scale * 1.4426950408889634f;
+  int block_shift = 0;
+  while ((1 << block_shift) < block_size) ++block_shift;
+  const int q_tiles = (max_q_len + 63) / 64;
+  const long long pairs = (long long)num_seqs * kv_heads * groups;
+  const long long per_xcd = (pairs + XCDS - 1) / XCDS;
+  if (per_xcd * XCDS * q_tiles > 0x7fffffffLL) return FE_BAD_ARGUMENT;
+  const unsigned grid = (unsigned)(per_xcd * XCDS * q_tiles);
+#define FE_GO(DD)                                                                                                \
+  paged_prefill_direct_kernel<DD><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+      (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,            \
+      kv_heads, groups, block_shift, num_blocks, window, scale_log2, q_tiles, (int)pairs, (int)per_xcd)
+  if (head_dim == 64) FE_GO(64);
+  else FE_GO(128);
+#undef FE_GO
+  return fe_check_launch();
+}
