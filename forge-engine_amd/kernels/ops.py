@@ -382,7 +382,7 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
                     ctx_len: Tensor, block_table: Tensor, *, num_seqs: int, max_q_len: int,
                     q_heads: int, kv_heads: int, head_dim: int, scale: float,
                     window: int | None = None, num_decode: int | None = None,
-                    max_ctx: int | None = None, splits: int | None = None, prefill_rows: int = 0) -> Tensor:
+                    max_ctx: int | None = None, splits: int | None = None) -> Tensor:
     """Attention of every query token of a mixed batch over its paged keys.
 
     q: [T, >= Hq*D] (row stride may exceed Hq*D: the q part of a fused qkv
@@ -450,18 +450,12 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
               _ptr(part_ml), _ptr(counters), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)),
               c_int(num_seqs), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
               c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(splits), _stream())
-    if any_longer and fast_prefill and prefill_rows == 0:
-        _call("attention_prefill_direct", "fe_paged_attention_prefill_direct", _ptr(q), c_longlong(q_stride),
-              _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
-              _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
-              c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), c_float(scale), _stream())
-    elif any_longer and fast_prefill:
+    if any_longer and fast_prefill:
         _call("attention_prefill", "fe_paged_attention_prefill", _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
               _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
               c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(prefill_rows), _stream())
+              c_int(num_blocks), c_int(window or 0), c_float(scale), _stream())
     # whatever the two fast kernels did not take goes to the general kernel
     single_left = any_single and not fast_decode
     longer_left = any_longer and not fast_prefill
@@ -505,4 +499,4 @@ def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index:
           _stream())
 
 
-LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "attention_prefill_direct", "sample")
+LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")

@@ -134,7 +134,7 @@ class GroupedQueryAttention(Mixer):
         return ops.linear_update(attn, self.o_weight, self.o_bias)   # float32 update for the residual sum
 
     def kernel_libraries(self):
-        return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "attention_prefill_direct", "gemm_f32", "gemm_skinny", "gemm_mid"}
+        return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny", "gemm_mid"}
 
 
 register_part("mixer", "gqa_attention", GroupedQueryAttention)

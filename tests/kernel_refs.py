@@ -129,7 +129,7 @@ def gather_pages(pages, table_row, length, block_size):
 
 
 def paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, *, num_seqs, max_q_len,
-                    q_heads, kv_heads, head_dim, scale, window=None, num_decode=None, max_ctx=None, splits=None, prefill_rows=0):
+                    q_heads, kv_heads, head_dim, scale, window=None, num_decode=None, max_ctx=None, splits=None):
     block_size = key_pages.shape[2]
     groups = q_heads // kv_heads
     key_pages, value_pages = key_pages.cpu(), value_pages.cpu()
