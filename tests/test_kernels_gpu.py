@@ -544,6 +544,35 @@ def test_decode_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size, s
             torch.testing.assert_close(again, expect, atol=2e-2, rtol=2e-2)
 
 
+def test_attention_kernels_on_random_mixed_batches(ops):
+    """Random head counts, groups, page sizes, windows and mixtures of single tokens and portions
+    (with and without context before them): the fast kernels that a bfloat16 batch is routed to
+    against the plain reference."""
+    import random
+    rng = random.Random(77)
+    for case in range(24):
+        head_dim = rng.choice([64, 128])
+        kv_heads = rng.choice([1, 2, 3])
+        groups = rng.choice([1, 2, 4, 5, 8])
+        q_heads = kv_heads * groups
+        block_size = rng.choice([16, 32, 64])
+        window = rng.choice([None, None, 1, 17, 64, 100])
+        seqs = [(rng.choice([0, 0, 1, 15, 16, 63, 64, rng.randrange(0, 300)]),
+                 rng.choice([1, 1, 2, 3, 17, 63, 64, 65, 130, rng.randrange(2, 200)])) for _ in range(rng.randrange(1, 5))]
+        g = torch.Generator().manual_seed(100 + case)
+        q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                    extra_width=2 * kv_heads * head_dim)
+        kw = dict(num_seqs=len(seqs), max_q_len=max(n for _, n in seqs), q_heads=q_heads, kv_heads=kv_heads,
+                  head_dim=head_dim, scale=head_dim ** -0.5, window=window)
+        want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype), cu, ctx, table, **kw).float()
+        got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV),
+                                  torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
+                                  cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=sum(1 for _, n in seqs if n == 1),
+                                  max_ctx=max(b + n for b, n in seqs), **kw).cpu().float()
+        assert torch.isfinite(got).all(), (case, seqs)
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2, msg=lambda m: f"case {case} {seqs} window {window}: {m}")
+
+
 @pytest.mark.parametrize("window", [1, 16, 37, 300])
 def test_decode_attention_kernel_window(ops, window):
     g = torch.Generator().manual_seed(31)
