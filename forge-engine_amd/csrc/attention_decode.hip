@@ -20,7 +20,16 @@
 //     pages, which are stored transposed ([D][slot]) for this, B = P^T.
 // Exactness: scores, max, sum and the weighted value sum are float32; P is
 // rounded to bfloat16 for the second product; one rounding at the final store.
+//
+// The PREPARE variant takes the raw output of the fused q/k/v projection instead of finished
+// queries and does on the way what a kernel of its own would do before it: RMSNorm over each
+// q and k head, rotation by the token's position, and the write of the new key and value into
+// their pages.  The new token's own key never comes back from memory: the last key split
+// treats it as a fifth partial result (score q.k_new, weight 1, value v_new) beside those of
+// its four waves.  The arithmetic is the stand-alone kernel's (rope_math.h), so the cache
+// holds the same bits whichever kernel wrote them.
 #include "common.h"
+#include "rope_math.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
@@ -44,27 +53,39 @@ __device__ __forceinline__ float load_agent(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int D>
+// What the PREPARE variant needs beyond the plain one: the norms' weights (null: no norm), the
+// rotation's frequencies [D / 2], and the pages as writable memory.
+struct Prepare {
+  const float* q_weight;
+  const float* k_weight;
+  const float* inv_freq;
+  float eps;
+};
+
+template <int D, bool PREPARE>
 __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
-    const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
-    const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
+    const bf16_t* __restrict__ q, long long q_stride, const bf16_t* key_pages,
+    const bf16_t* value_pages, bf16_t* __restrict__ out, long long out_stride,
     float* part_o, float* part_ml, int* __restrict__ counters, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const int* __restrict__ block_table, int table_stride,
-    int kv_heads, int groups, int block_shift, int num_blocks, int window, float scale_log2) {
+    int kv_heads, int groups, int block_shift, int num_blocks, int window, float scale_log2,
+    Prepare prep) {
   const int block_size = 1 << block_shift, block_mask = block_size - 1;
   constexpr int KC = D / 32;        // MFMA k-steps over the head dim (scores)
   constexpr int DT = D / 16;        // 16-dim tiles of the output
-  __shared__ float Ow[WAVES][GMAX][D];
-  __shared__ float Ms[WAVES][GMAX], Ls[WAVES][GMAX];
+  constexpr int PARTS = WAVES + (PREPARE ? 1 : 0);   // partial results that meet in LDS
+  __shared__ float Ow[PARTS][GMAX][D];
+  __shared__ float Ms[PARTS][GMAX], Ls[PARTS][GMAX];
 
   const int split = blockIdx.x, splits = gridDim.x;
   const int hk = blockIdx.y, seq = blockIdx.z;
   const int q0 = cu_q[seq];
   if (cu_q[seq + 1] - q0 != 1) return;
   const int ctx = ctx_len[seq];
+  const int cached = PREPARE ? ctx - 1 : ctx;             // keys that the loop below reads from the pages
   const int k_begin = window > 0 ? max(0, ctx - window) : 0;
   const int first = k_begin / KEYS;
-  const int last = (ctx + KEYS - 1) / KEYS;               // exclusive
+  const int last = (cached + KEYS - 1) / KEYS;            // exclusive
   const int per_split = (last - first + splits - 1) / splits;
   const int my_first = first + split * per_split;
   const int my_last = min(last, my_first + per_split);
@@ -72,6 +93,15 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 15, lq = lane >> 4;
+
+  // The rotation's cosines and sines of this token, once per block.
+  __shared__ float cos_s[PREPARE ? D / 2 : 1], sin_s[PREPARE ? D / 2 : 1];
+  if (PREPARE && tid < D / 2) {
+    float sn, cs;
+    sincosf((float)(ctx - 1) * prep.inv_freq[tid], &sn, &cs);
+    cos_s[tid] = cs;
+    sin_s[tid] = sn;
+  }
 
   // query rows as the B operand: lane (lr = row g, lq) holds q[g][32c + 8lq .. +8]
   bf16x8 qb[KC];
@@ -102,7 +132,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   // Raw table entries are loaded two blocks ahead and checked only where they are used, so that
   // nothing waits for them while the block's own loads are in flight.
   auto raw_page = [&](int key) -> int { return table[min(key >> block_shift, table_last)]; };
-  auto checked = [&](int id, int key) -> int { return (key < ctx && id >= 0 && id < num_blocks) ? id : 0; };
+  auto checked = [&](int id, int key) -> int { return (key < cached && id >= 0 && id < num_blocks) ? id : 0; };
   auto fetch_keys = [&](int b, int block, uintx4 (*dst)[KC]) {
     const bool mine = b < my_last;      // past this block's share: read page 0 again (cached) instead
     block = mine ? block : 0;
@@ -122,7 +152,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     // values (A operand of the second product): lane (lr = dim, lq) reads the 8 consecutive keys
     // 8lq .. 8lq+7 of dims 16t + lr from the transposed page
     const int vkey = b * KEYS + 8 * lq;
-    const bool v_ok = vkey < ctx;
+    const bool v_ok = vkey < cached;
     const int vpage = checked(vraw, vkey);
     const bf16_t* vbase = value_pages + ((((size_t)vpage * kv_heads + hk) * D) << block_shift) + (vkey & block_mask);
     uintx4 va[DT];
@@ -149,7 +179,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     for (int j = 0; j < 8; ++j) {
       const int key = b * KEYS + 8 * lq + j;
       const float v = st[j >> 2][j & 3] * scale_log2;
-      s[j] = (key >= k_begin && key < ctx) ? v : -INFINITY;
+      s[j] = (key >= k_begin && key < cached) ? v : -INFINITY;
       mx = fmaxf(mx, s[j]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, FE_WAVE));
@@ -189,6 +219,134 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     kr1 = raw_page((b0 + WAVES) * KEYS + krow);
     v1 = raw_page((b0 + WAVES) * KEYS + 8 * lq);
   }
+
+  bool extra = false;       // this block also brings the new token's own key and value
+  if constexpr (PREPARE) {
+    __syncthreads();        // cos_s, sin_s
+    // Queries: chunk 4c + lq of head row lr sits in qb[c].  Norm, rotation and rounding as the
+    // stand-alone kernel does them: the butterfly over chunks runs over c first, then over lq.
+    float qv[KC][8];
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const uintx4 raw = __builtin_bit_cast(uintx4, qb[c]);
+      const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+      unpack_bf16x8(w4, qv[c]);
+    }
+    if (prep.q_weight) {
+      float total[KC];
+#pragma unroll
+      for (int c = 0; c < KC; ++c) total[c] = sum_squares8(qv[c]);
+#pragma unroll
+      for (int offset = KC / 2; offset > 0; offset >>= 1) {
+        float next[KC];
+#pragma unroll
+        for (int c = 0; c < KC; ++c) next[c] = total[c] + total[c ^ offset];
+#pragma unroll
+        for (int c = 0; c < KC; ++c) total[c] = next[c];
+      }
+      float sumsq = total[0];
+      sumsq += __shfl_xor(sumsq, 32, FE_WAVE);
+      sumsq += __shfl_xor(sumsq, 16, FE_WAVE);
+      const float inv = inverse_rms(sumsq, D, prep.eps);
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        const float4 wa = *(const float4*)(prep.q_weight + c * 32 + lq * 8);
+        const float4 wb = *(const float4*)(prep.q_weight + c * 32 + lq * 8 + 4);
+        const float w8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qv[c][e] = normalise(qv[c][e], inv, w8[e]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < KC / 2; ++c) {
+      float lo[8], hi[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float cs = cos_s[c * 32 + lq * 8 + e], sn = sin_s[c * 32 + lq * 8 + e];
+        lo[e] = rotate_low(qv[c][e], qv[c + KC / 2][e], cs, sn);
+        hi[e] = rotate_high(qv[c + KC / 2][e], qv[c][e], cs, sn);
+      }
+      uint32_t pl[4], ph[4];
+      pack_bf16x8(lo, pl);
+      pack_bf16x8(hi, ph);
+      qb[c] = __builtin_bit_cast(bf16x8, uintx4{pl[0], pl[1], pl[2], pl[3]});
+      qb[c + KC / 2] = __builtin_bit_cast(bf16x8, uintx4{ph[0], ph[1], ph[2], ph[3]});
+    }
+
+    // The new token's key and value: made by the last wave of the last split (the one with the
+    // least other work), written to their pages, and kept in LDS as a partial result of their
+    // own: score q.k_new, weight 1, value v_new.
+    extra = split == splits - 1;
+    if (extra && wave == WAVES - 1) {
+      constexpr int LPH = D / 8;                 // lanes that share a head, 8 elements each
+      __shared__ __attribute__((aligned(16))) bf16_t new_key[D];
+      const int sub = lane & (LPH - 1);
+      const int role = lane / LPH;               // 0: key, 1: value, others idle (they follow the key's path)
+      const int pos = ctx - 1;
+      const bf16_t* row = q + (size_t)q0 * q_stride;
+      const size_t k_at = (size_t)(kv_heads * groups + hk) * D, v_at = k_at + (size_t)kv_heads * D;
+      const uint4 raw = *(const uint4*)(row + (role == 1 ? v_at : k_at) + sub * 8);
+      const int block = table[min(pos >> block_shift, table_last)];
+      const bool writable = block >= 0 && block < num_blocks;     // the host reserves pages before the launch
+      const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+      float v[8];
+      unpack_bf16x8(w4, v);
+      if (prep.k_weight) {
+        float sumsq = sum_squares8(v);
+#pragma unroll
+        for (int offset = LPH / 2; offset > 0; offset >>= 1) sumsq += __shfl_xor(sumsq, offset, FE_WAVE);
+        const float inv = inverse_rms(sumsq, D, prep.eps);
+        const float4 wa = *(const float4*)(prep.k_weight + sub * 8);
+        const float4 wb = *(const float4*)(prep.k_weight + sub * 8 + 4);
+        const float w8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = normalise(v[e], inv, w8[e]);
+      }
+      const bool low = sub * 8 < D / 2;
+      float r[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float other = __shfl_xor(v[e], LPH / 2, FE_WAVE);
+        const int j = (sub * 8 + e) & (D / 2 - 1);
+        r[e] = low ? rotate_low(v[e], other, cos_s[j], sin_s[j]) : rotate_high(v[e], other, cos_s[j], sin_s[j]);
+      }
+      uint32_t k4[4];
+      pack_bf16x8(r, k4);
+      const size_t page = (size_t)(writable ? block : 0) * kv_heads + hk;
+      if (role == 0) {
+        *(uint4*)&new_key[sub * 8] = make_uint4(k4[0], k4[1], k4[2], k4[3]);
+        if (writable)
+          *(uint4*)(const_cast<bf16_t*>(key_pages) + ((page << block_shift) + (pos & block_mask)) * D + sub * 8) =
+              make_uint4(k4[0], k4[1], k4[2], k4[3]);
+      } else if (role == 1) {
+        bf16_t* vdst = const_cast<bf16_t*>(value_pages) + ((page * D) << block_shift) + (pos & block_mask);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const bf16_t bits = (bf16_t)(e & 1 ? w4[e >> 1] >> 16 : w4[e >> 1] & 0xffffu);
+          if (writable) vdst[(size_t)(sub * 8 + e) << block_shift] = bits;
+          for (int g = 0; g < groups; ++g) Ow[WAVES][g][sub * 8 + e] = bf16_to_float(bits);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      __threadfence_block();                     // new_key is read by other lanes of this wave
+      float dot = 0.f;
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        const uint4 kraw = *(const uint4*)&new_key[c * 32 + lq * 8];
+        const uintx4 qraw = __builtin_bit_cast(uintx4, qb[c]);
+        const uint32_t kw[4] = {kraw.x, kraw.y, kraw.z, kraw.w}, qw[4] = {qraw.x, qraw.y, qraw.z, qraw.w};
+        float kf[8], qf[8];
+        unpack_bf16x8(kw, kf);
+        unpack_bf16x8(qw, qf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dot = __fmaf_rn(qf[e], kf[e], dot);
+      }
+      dot += __shfl_xor(dot, 16, FE_WAVE);
+      dot += __shfl_xor(dot, 32, FE_WAVE);
+      if (lq == 0 && lr < groups) { Ms[WAVES][lr] = dot * scale_log2; Ls[WAVES][lr] = 1.f; }
+    }
+  }
+
   for (int b = b0; b < my_last; b += 2 * WAVES) {
     step(b, k0, k1, v0, kr1, kr0);
     if (b + WAVES >= my_last) break;
@@ -210,6 +368,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     float m_tot = -INFINITY;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) m_tot = fmaxf(m_tot, Ms[w][g]);
+    if (PREPARE && extra) m_tot = fmaxf(m_tot, Ms[PARTS - 1][g]);
     float ov = 0.f, l = 0.f;
     if (m_tot > -INFINITY) {
 #pragma unroll
@@ -217,6 +376,11 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
         const float f = __builtin_amdgcn_exp2f(Ms[w][g] - m_tot);
         ov += f * Ow[w][g][d];
         l += f * Ls[w][g];
+      }
+      if (PREPARE && extra) {
+        const float f = __builtin_amdgcn_exp2f(Ms[PARTS - 1][g] - m_tot);
+        ov += f * Ow[PARTS - 1][g][d];
+        l += f * Ls[PARTS - 1][g];
       }
     }
     if (splits == 1) {
@@ -271,6 +435,41 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   }
 }
 
+static int launch_decode(const void* q, long long q_stride, const void* key_pages, const void* value_pages,
+                         void* out, long long out_stride, float* part_o, float* part_ml, int* counters,
+                         const int* cu_q, const int* ctx_len, const int* block_table, int table_stride,
+                         int num_seqs, int kv_heads, int groups, int head_dim, int block_size,
+                         int num_blocks, int window, float scale, int splits, const Prepare* prep,
+                         hipStream_t stream) {
+  if (num_seqs <= 0) return FE_OK;
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256) return FE_BAD_ARGUMENT;
+  if (groups < 1 || groups > GMAX || kv_heads < 1 || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
+  if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1) return FE_BAD_ARGUMENT;
+  int block_shift = 0;
+  while ((1 << block_shift) < block_size) ++block_shift;
+  if (q_stride % 8 || splits < 1 || splits > 64) return FE_BAD_ARGUMENT;
+  if ((((uintptr_t)q) | ((uintptr_t)key_pages) | ((uintptr_t)value_pages)) & 15) return FE_BAD_ARGUMENT;
+  if (splits > 1 && (!part_o || !part_ml || !counters)) return FE_BAD_ARGUMENT;
+  dim3 grid(splits, kv_heads, num_seqs);
+  const float scale_log2 = scale * 1.4426950408889634f;
+  const Prepare none = {nullptr, nullptr, nullptr, 0.f};
+#define FE_GO(DD, PP)                                                                                      \
+  paged_decode_kernel<DD, PP><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+      (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, PP ? *prep : none)
+  if (prep) {
+    if (head_dim == 64) FE_GO(64, true);
+    else if (head_dim == 128) FE_GO(128, true);
+    else FE_GO(256, true);
+  } else {
+    if (head_dim == 64) FE_GO(64, false);
+    else if (head_dim == 128) FE_GO(128, false);
+    else FE_GO(256, false);
+  }
+#undef FE_GO
+  return fe_check_launch();
+}
+
 // Sequences with one query token only; others are left untouched.  Pages: keys
 // [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size];
 // block_size a power of two >= 16.  splits > 1 (at most 64) needs part_o [num_seqs * kv_heads * splits * groups * head_dim] and
@@ -284,23 +483,30 @@ extern "C" int fe_paged_attention_decode(const void* q, long long q_stride, cons
                                          int num_seqs, int kv_heads, int groups, int head_dim,
                                          int block_size, int num_blocks, int window, float scale,
                                          int splits, hipStream_t stream) {
-  if (num_seqs <= 0) return FE_OK;
-  if (head_dim != 64 && head_dim != 128 && head_dim != 256) return FE_BAD_ARGUMENT;
-  if (groups < 1 || groups > GMAX || kv_heads < 1 || kv_heads > 65535 || num_seqs > 65535) return FE_BAD_ARGUMENT;
-  if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1) return FE_BAD_ARGUMENT;
-  int block_shift = 0;
-  while ((1 << block_shift) < block_size) ++block_shift;
-  if (q_stride % 8 || splits < 1 || splits > 64) return FE_BAD_ARGUMENT;
-  if (splits > 1 && (!part_o || !part_ml || !counters)) return FE_BAD_ARGUMENT;
-  dim3 grid(splits, kv_heads, num_seqs);
-  const float scale_log2 = scale * 1.4426950408889634f;
-#define FE_GO(DD)                                                                                          \
-  paged_decode_kernel<DD><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages,    \
-      (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
-      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2)
-  if (head_dim == 64) FE_GO(64);
-  else if (head_dim == 128) FE_GO(128);
-  else FE_GO(256);
-#undef FE_GO
-  return fe_check_launch();
+  return launch_decode(q, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
+                       ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
+                       num_blocks, window, scale, splits, nullptr, stream);
+}
+
+// The same for a batch in which EVERY sequence brings one token, straight from the fused
+// projection's output qkv [num_seqs rows of (kv_heads * groups + 2 * kv_heads) * head_dim, row
+// stride q_stride]: q and k heads are normalised (weights [head_dim] float32, null: no norm)
+// and rotated whole by position ctx_len - 1 (inv_freq [head_dim / 2]), and each sequence's new
+// key and value are written to slot ctx_len - 1 of its pages.  qkv itself is not changed.
+extern "C" int fe_paged_attention_decode_prepare(const void* qkv, long long q_stride, const float* q_weight,
+                                                 const float* k_weight, const float* inv_freq, float eps,
+                                                 void* key_pages, void* value_pages, void* out,
+                                                 long long out_stride, float* part_o, float* part_ml,
+                                                 int* counters, const int* cu_q, const int* ctx_len,
+                                                 const int* block_table, int table_stride, int num_seqs,
+                                                 int kv_heads, int groups, int head_dim, int block_size,
+                                                 int num_blocks, int window, float scale, int splits,
+                                                 hipStream_t stream) {
+  if (!inv_freq || (!q_weight) != (!k_weight)) return FE_BAD_ARGUMENT;
+  if (q_weight && ((((uintptr_t)q_weight) | ((uintptr_t)k_weight)) & 15)) return FE_BAD_ARGUMENT;
+  if (q_stride < (long long)(kv_heads * groups + 2 * kv_heads) * head_dim) return FE_BAD_ARGUMENT;
+  const Prepare prep = {q_weight, k_weight, inv_freq, eps};
+  return launch_decode(qkv, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
+                       ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
+                       num_blocks, window, scale, splits, &prep, stream);
 }

@@ -15,6 +15,7 @@
 // token at position p of sequence s lives in block table[s][p / block_size],
 // slot p % block_size.
 #include "common.h"
+#include "rope_math.h"
 
 // One block serves `heads_per_block` heads of one token (4 waves, a head per wave at a time).
 // The cosines and sines of the token's angles are computed once per block into LDS: with many
@@ -192,22 +193,16 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
     float v[8];
     {
       const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        v[2 * e] = __uint_as_float(w4[e] << 16);
-        v[2 * e + 1] = __uint_as_float(w4[e] & 0xffff0000u);
-      }
+      unpack_bf16x8(w4, v);
     }
     const float* w = is_q ? q_weight : k_weight;
     if (w) {
-      float sumsq = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) sumsq += v[e] * v[e];
+      float sumsq = sum_squares8(v);
 #pragma unroll
       for (int offset = LPH / 2; offset > 0; offset >>= 1) sumsq += __shfl_xor(sumsq, offset, FE_WAVE);
-      const float inv = rsqrtf(sumsq / (float)D + eps);
+      const float inv = inverse_rms(sumsq, D, eps);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = v[e] * inv * w[first + e];
+      for (int e = 0; e < 8; ++e) v[e] = normalise(v[e], inv, w[first + e]);
     }
     uint32_t o4[4];
     float r[8];
@@ -215,10 +210,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
     for (int e = 0; e < 8; ++e) {
       const float other = __shfl_xor(v[e], LPH / 2, FE_WAVE);     // element first + e -/+ HALF
       const int j = (first + e) & (HALF - 1);
-      r[e] = low ? v[e] * cos_s[j] - other * sin_s[j] : v[e] * cos_s[j] + other * sin_s[j];
+      r[e] = low ? rotate_low(v[e], other, cos_s[j], sin_s[j]) : rotate_high(v[e], other, cos_s[j], sin_s[j]);
     }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) o4[e] = (uint32_t)float_to_bf16(r[2 * e]) | ((uint32_t)float_to_bf16(r[2 * e + 1]) << 16);
+    pack_bf16x8(r, o4);
     bf16_t* dst = is_q ? x : key_pages + page + (size_t)slot * D + first;
     *(uint4*)dst = make_uint4(o4[0], o4[1], o4[2], o4[3]);
   }

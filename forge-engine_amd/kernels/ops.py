@@ -464,6 +464,78 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
     return out
 
 
+def decode_prepare_supported(dtype, *, q_heads: int, kv_heads: int, head_dim: int, rotary_dim: int,
+                             block_size: int) -> bool:
+    """Whether ``decode_attention_prepare`` serves these sizes: a bfloat16 cache, heads of 64,
+    128 or 256 elements rotated whole, at most eight query heads per kv head."""
+    return (dtype == torch.bfloat16 and head_dim in (64, 128, 256) and rotary_dim == head_dim
+            and q_heads % kv_heads == 0 and q_heads // kv_heads <= 8
+            and block_size >= 16 and block_size & (block_size - 1) == 0)
+
+
+def decode_attention_prepare(qkv: Tensor, q_weight: Tensor | None, k_weight: Tensor | None, inv_freq: Tensor,
+                             key_pages: Tensor, value_pages: Tensor, out: Tensor, cu_q: Tensor, ctx_len: Tensor,
+                             block_table: Tensor, *, q_heads: int, kv_heads: int, head_dim: int, eps: float,
+                             scale: float, window: int | None = None, max_ctx: int | None = None,
+                             splits: int | None = None) -> Tensor:
+    """A step of single tokens only, from the fused projection's output to the attention's
+    output in one launch: what ``qk_norm_rope_write`` followed by ``paged_attention`` does for
+    such a batch (same bits in the cache; qkv is left as it is).
+
+    qkv [B, (Hq + 2 Hkv) D] bfloat16, one row per sequence; ctx_len counts the new token, whose
+    position is ctx_len - 1."""
+    _gpu(qkv, "qkv", torch.bfloat16)
+    num_seqs = qkv.shape[0]
+    width = (q_heads + 2 * kv_heads) * head_dim
+    if qkv.dim() != 2 or qkv.shape[1] != width:
+        raise KernelError(f"qkv must be [B, {width}], got {tuple(qkv.shape)}")
+    _gpu(key_pages, "key_pages", torch.bfloat16)
+    _gpu(value_pages, "value_pages", torch.bfloat16)
+    if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
+        raise KernelError(f"pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
+    num_blocks, _, block_size, _ = key_pages.shape
+    if value_pages.shape != (num_blocks, kv_heads, head_dim, block_size):
+        raise KernelError(f"value pages are transposed: [blocks, {kv_heads}, {head_dim}, block_size], got {tuple(value_pages.shape)}")
+    if not decode_prepare_supported(qkv.dtype, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+                                    rotary_dim=2 * inv_freq.numel() if inv_freq is not None else 0,
+                                    block_size=block_size):
+        raise KernelError("these sizes are not served by the fused decode kernel: heads of 64, 128 or 256 "
+                          "elements rotated whole, at most 8 query heads per kv head, pages of a power of two >= 16")
+    if (q_weight is None) != (k_weight is None):
+        raise KernelError("q and k are normalised both or neither")
+    for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+        if w is not None:
+            _gpu(w, name, torch.float32)
+            if w.shape != (head_dim,):
+                raise KernelError(f"{name} must be [{head_dim}]")
+    _gpu(inv_freq, "inv_freq", torch.float32)
+    _gpu(out, "out", torch.bfloat16)
+    if out.shape != (num_seqs, q_heads * head_dim):
+        raise KernelError(f"out must be [{num_seqs}, {q_heads * head_dim}], got {tuple(out.shape)}")
+    _gpu(cu_q, "cu_q", torch.int32)
+    _gpu(ctx_len, "ctx_len", torch.int32)
+    _gpu(block_table, "block_table", torch.int32)
+    if cu_q.numel() != num_seqs + 1 or ctx_len.numel() != num_seqs or block_table.shape[0] < num_seqs:
+        raise KernelError("cu_q, ctx_len and block_table do not match the number of sequences")
+    if block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
+    groups = q_heads // kv_heads
+    if splits is None:
+        splits = decode_splits(num_seqs, kv_heads, max_ctx if max_ctx is not None else 16 * 4 * 8)
+    part_o = part_ml = counters = None
+    if splits > 1:
+        part_o = torch.empty(num_seqs * kv_heads * splits * groups * head_dim, dtype=torch.float32, device=qkv.device)
+        part_ml = torch.empty(num_seqs * kv_heads * splits * groups * 2, dtype=torch.float32, device=qkv.device)
+        counters = _split_counters(qkv.device, num_seqs * kv_heads)
+    _call("attention_decode", "fe_paged_attention_decode_prepare", _ptr(qkv), c_longlong(width), _ptr(q_weight),
+          _ptr(k_weight), _ptr(inv_freq), c_float(eps), _ptr(key_pages), _ptr(value_pages), _ptr(out),
+          c_longlong(out.stride(0)), _ptr(part_o), _ptr(part_ml), _ptr(counters), _ptr(cu_q), _ptr(ctx_len),
+          _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs), c_int(kv_heads), c_int(groups),
+          c_int(head_dim), c_int(block_size), c_int(num_blocks), c_int(window or 0), c_float(scale),
+          c_int(splits), _stream())
+    return out
+
+
 # ------------------------------------------------------------------- sampling
 
 def argmax_rows(logits: Tensor, tokens: Tensor, status: Tensor) -> None:

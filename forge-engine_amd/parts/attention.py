@@ -117,6 +117,15 @@ class GroupedQueryAttention(Mixer):
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 1.0
         if writes_cache:
             qkv = ops.linear(x, self.qkv_weight, self.qkv_bias)
+            if self._single_tokens_only(batch, x, cache, rotary_dim):
+                # norms, rotation, cache write and attention in one launch
+                attn = torch.empty((x.shape[0], self.q_size), dtype=x.dtype, device=x.device)
+                ops.decode_attention_prepare(
+                    qkv, self.q_norm, self.k_norm, inv_freq, cache.key_pages, cache.value_pages, attn,
+                    batch.cu_q, batch.ctx_len, cache.block_table, q_heads=self.num_heads,
+                    kv_heads=self.num_kv_heads, head_dim=self.head_dim, eps=eps, scale=self.scale,
+                    window=self.window, max_ctx=batch.max_ctx)
+                return ops.linear_update(attn, self.o_weight, self.o_bias)
         else:  # another call wrote the keys and values this one reads: only q is needed
             bias = None if self.qkv_bias is None else self.qkv_bias[:self.q_size]
             qkv = ops.linear(x, self.qkv_weight[:self.q_size], bias)
@@ -132,6 +141,14 @@ class GroupedQueryAttention(Mixer):
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
             num_decode=batch.num_decode, max_ctx=batch.max_ctx)
         return ops.linear_update(attn, self.o_weight, self.o_bias)   # float32 update for the residual sum
+
+    def _single_tokens_only(self, batch, x: Tensor, cache: CacheView, rotary_dim: int) -> bool:
+        """Every sequence of the step brings one token, and the sizes are ones that the
+        decode kernel prepares queries and keys for itself."""
+        return (batch.num_decode is not None and batch.num_decode == batch.num_seqs == x.shape[0]
+                and ops.decode_prepare_supported(
+                    x.dtype, q_heads=self.num_heads, kv_heads=self.num_kv_heads, head_dim=self.head_dim,
+                    rotary_dim=rotary_dim, block_size=cache.key_pages.shape[2]))
 
     def kernel_libraries(self):
         return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny", "gemm_mid"}

@@ -573,6 +573,152 @@ def test_attention_kernels_on_random_mixed_batches(ops):
         torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2, msg=lambda m: f"case {case} {seqs} window {window}: {m}")
 
 
+def _prepare_case(g, q_heads, kv_heads, head_dim, block_size, contexts):
+    """A step of single tokens: raw projection output, norm weights, frequencies, filled pages."""
+    seqs = [(before, 1) for before in contexts]
+    qkv, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                  extra_width=2 * kv_heads * head_dim)
+    qw, kw = 1.0 + rand(g, head_dim, scale=0.1), 1.0 + rand(g, head_dim, scale=0.1)
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    positions = torch.tensor(contexts, dtype=torch.int32)
+    token_seq = torch.arange(len(contexts), dtype=torch.int32)
+    return qkv, kp, vp, cu, ctx, table, qw, kw, inv_freq, positions, token_seq
+
+
+@pytest.mark.parametrize("splits", [1, 3, 8])
+@pytest.mark.parametrize("with_norm", [True, False])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [
+    (32, 8, 128, 16), (5, 5, 64, 16), (10, 2, 128, 32), (8, 1, 256, 16), (6, 3, 64, 64), (7, 1, 128, 16),
+])
+def test_decode_attention_that_prepares_its_queries_and_keys(ops, q_heads, kv_heads, head_dim, block_size, splits, with_norm):
+    """One launch from the projection's output to the attention's output against the plain
+    reference of the two steps (norm + rotation + cache write, then attention), and against the
+    two kernels that do the same in two launches: the pages must hold the same bits."""
+    g = torch.Generator().manual_seed(33)
+    contexts = [0, 1, 14, 15, 16, 31, 32, 699, 255, 3]      # tokens each sequence holds before the step
+    qkv, kp, vp, cu, ctx, table, qw, kw, inv_freq, positions, token_seq = _prepare_case(
+        g, q_heads, kv_heads, head_dim, block_size, contexts)
+    if not with_norm:
+        qw = kw = None
+    n = len(contexts)
+    sizes = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim)
+    akw = dict(num_seqs=n, max_q_len=1, scale=head_dim ** -0.5, **sizes)
+    # plain reference
+    qkv_ref, kp_ref, vp_ref = qkv.clone(), kp.clone(), vp.clone()
+    refs.qk_norm_rope_write(qkv_ref, qw, kw, inv_freq, positions, token_seq, table, kp_ref, vp_ref,
+                            rotary_dim=head_dim, eps=1e-6, **sizes)
+    want = refs.paged_attention(qkv_ref, kp_ref, vp_ref, torch.empty(n, q_heads * head_dim, dtype=qkv.dtype),
+                                cu, ctx, table, **akw).float()
+    # two launches
+    dev = lambda t: None if t is None else t.to(DEV)
+    qkv_two, kp_two, vp_two = qkv.to(DEV), kp.to(DEV), vp.to(DEV)
+    ops.qk_norm_rope_write(qkv_two, dev(qw), dev(kw), dev(inv_freq), dev(positions), dev(token_seq), dev(table),
+                           kp_two, vp_two, rotary_dim=head_dim, eps=1e-6, **sizes)
+    two = ops.paged_attention(qkv_two, kp_two, vp_two, torch.empty(n, q_heads * head_dim, dtype=qkv.dtype, device=DEV),
+                              dev(cu), dev(ctx), dev(table), num_decode=n, max_ctx=700, splits=splits, **akw).cpu().float()
+    # one launch, twice (the second on the pages the first left: the arrival counters are zero again)
+    qkv_one, kp_one, vp_one = qkv.to(DEV), kp.to(DEV), vp.to(DEV)
+    for _ in range(2):
+        out = torch.full((n, q_heads * head_dim), float("nan"), dtype=qkv.dtype, device=DEV)
+        ops.decode_attention_prepare(qkv_one, dev(qw), dev(kw), dev(inv_freq), kp_one, vp_one, out, dev(cu), dev(ctx),
+                                     dev(table), eps=1e-6, scale=head_dim ** -0.5, max_ctx=700, splits=splits, **sizes)
+        got = out.cpu().float()
+        assert torch.equal(qkv_one.cpu(), qkv)               # the projection's output is left alone
+        assert torch.equal(kp_one.cpu(), kp_two.cpu())       # same bits as the stand-alone kernel writes
+        assert torch.equal(vp_one.cpu(), vp_two.cpu())
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(got, two, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(kp_one.cpu().float(), kp_ref.float(), **tol(torch.bfloat16))
+    assert torch.equal(vp_one.cpu(), vp_ref)
+
+
+@pytest.mark.parametrize("window", [1, 16, 37, 300])
+def test_decode_attention_that_prepares_with_a_window(ops, window):
+    g = torch.Generator().manual_seed(34)
+    contexts = [0, 36, 37, 500]
+    qkv, kp, vp, cu, ctx, table, qw, kw, inv_freq, positions, token_seq = _prepare_case(g, 8, 2, 128, 16, contexts)
+    sizes = dict(q_heads=8, kv_heads=2, head_dim=128)
+    qkv_ref, kp_ref, vp_ref = qkv.clone(), kp.clone(), vp.clone()
+    refs.qk_norm_rope_write(qkv_ref, qw, kw, inv_freq, positions, token_seq, table, kp_ref, vp_ref,
+                            rotary_dim=128, eps=1e-5, **sizes)
+    want = refs.paged_attention(qkv_ref, kp_ref, vp_ref, torch.empty(4, 1024, dtype=qkv.dtype), cu, ctx, table,
+                                num_seqs=4, max_q_len=1, scale=0.1, window=window, **sizes).float()
+    for splits in (1, 4):
+        kp_dev, vp_dev = kp.to(DEV), vp.to(DEV)
+        out = torch.full((4, 1024), float("nan"), dtype=qkv.dtype, device=DEV)
+        ops.decode_attention_prepare(qkv.to(DEV), qw.to(DEV), kw.to(DEV), inv_freq.to(DEV), kp_dev, vp_dev, out,
+                                     cu.to(DEV), ctx.to(DEV), table.to(DEV), eps=1e-5, scale=0.1, window=window,
+                                     max_ctx=501, splits=splits, **sizes)
+        torch.testing.assert_close(out.cpu().float(), want, atol=2e-2, rtol=2e-2)
+        assert torch.equal(vp_dev.cpu(), vp_ref)
+
+
+def test_decode_attention_that_prepares_sees_its_own_token_and_a_far_key(ops):
+    """The new token's own key never comes from memory, and keys far back do: each made to
+    stand out in turn (query and key are unit vectors scaled up, no norm, position 0 rotation
+    aside the rotation keeps lengths, so q.k of the chosen pair dominates)."""
+    g = torch.Generator().manual_seed(35)
+    head_dim, block_size, before = 128, 16, 999
+    qkv, kp, vp, cu, ctx, table, _, _, inv_freq, positions, token_seq = _prepare_case(g, 4, 1, head_dim, block_size, [before])
+    qkv = (qkv.float() * 0.01).to(torch.bfloat16)
+    sizes = dict(q_heads=4, kv_heads=1, head_dim=head_dim)
+    # its own token: the new key is the query's direction, scaled up; rotation by the same angle keeps q.k
+    own = qkv.clone()
+    own[0, :5 * head_dim] = 0.0
+    for h in range(5):                       # four query heads and the key head
+        own[0, h * head_dim + 5] = 30.0
+    for splits in (1, 5):
+        kp_dev, vp_dev = kp.to(DEV), vp.to(DEV)
+        out = torch.empty(1, 4 * head_dim, dtype=qkv.dtype, device=DEV)
+        ops.decode_attention_prepare(own.to(DEV), None, None, inv_freq.to(DEV), kp_dev, vp_dev, out, cu.to(DEV),
+                                     ctx.to(DEV), table.to(DEV), eps=1e-6, scale=head_dim ** -0.5, max_ctx=1000,
+                                     splits=splits, **sizes)
+        new_value = own[0, 5 * head_dim:6 * head_dim].float()
+        for h in range(4):
+            torch.testing.assert_close(out.cpu().float()[0, h * head_dim:(h + 1) * head_dim], new_value, atol=2e-2, rtol=2e-2)
+        page, slot = int(table[0, before // block_size]), before % block_size
+        assert torch.equal(vp_dev.cpu()[page, 0, :, slot], own[0, 5 * head_dim:6 * head_dim])
+    # a far key: stored as the query's rotated direction (the reference rotates the query for us)
+    rotated = own.clone()
+    refs.qk_norm_rope_write(rotated, None, None, inv_freq, positions, token_seq, table, kp.clone(), vp.clone(),
+                            rotary_dim=head_dim, eps=1e-6, **sizes)
+    quiet = own.clone()
+    quiet[0, 4 * head_dim:5 * head_dim] = 0.0            # the new key says nothing
+    for far in (0, 15, 16, 511, 512, 991, 998):
+        kq = kp.clone()
+        page, slot = int(table[0, far // block_size]), far % block_size
+        kq[page, 0, slot] = rotated[0, :head_dim]
+        for splits in (1, 5):
+            out = torch.empty(1, 4 * head_dim, dtype=qkv.dtype, device=DEV)
+            ops.decode_attention_prepare(quiet.to(DEV), None, None, inv_freq.to(DEV), kq.to(DEV), vp.to(DEV), out,
+                                         cu.to(DEV), ctx.to(DEV), table.to(DEV), eps=1e-6, scale=head_dim ** -0.5,
+                                         max_ctx=1000, splits=splits, **sizes)
+            for h in range(4):
+                torch.testing.assert_close(out.cpu().float()[0, h * head_dim:(h + 1) * head_dim],
+                                           vp[page, 0, :, slot].float(), atol=2e-2, rtol=2e-2)
+
+
+def test_decode_attention_that_prepares_refuses_what_it_does_not_serve(ops):
+    g = torch.Generator().manual_seed(36)
+    qkv, kp, vp, cu, ctx, table, qw, kw, inv_freq, _, _ = _prepare_case(g, 4, 2, 64, 16, [3, 9])
+    dev = lambda t: t.to(DEV)
+    out = torch.empty(2, 256, dtype=torch.bfloat16, device=DEV)
+    call = lambda **over: ops.decode_attention_prepare(
+        **{**dict(qkv=dev(qkv), q_weight=dev(qw), k_weight=dev(kw), inv_freq=dev(inv_freq), key_pages=dev(kp),
+                  value_pages=dev(vp), out=out, cu_q=dev(cu), ctx_len=dev(ctx), block_table=dev(table), q_heads=4,
+                  kv_heads=2, head_dim=64, eps=1e-6, scale=0.125), **over})
+    call()
+    with pytest.raises(ops.KernelError):
+        call(inv_freq=dev(inv_freq[:16]))                  # a head rotated in part
+    with pytest.raises(ops.KernelError):
+        call(k_weight=None)                                # one norm without the other
+    with pytest.raises(ops.KernelError):
+        call(qkv=dev(qkv[:, :-64].contiguous()))           # no room for the values
+    assert not ops.decode_prepare_supported(torch.float32, q_heads=4, kv_heads=2, head_dim=64, rotary_dim=64, block_size=16)
+    assert not ops.decode_prepare_supported(torch.bfloat16, q_heads=4, kv_heads=2, head_dim=48, rotary_dim=48, block_size=16)
+    assert not ops.decode_prepare_supported(torch.bfloat16, q_heads=18, kv_heads=2, head_dim=64, rotary_dim=64, block_size=16)
+
+
 @pytest.mark.parametrize("window", [1, 16, 37, 300])
 def test_decode_attention_kernel_window(ops, window):
     g = torch.Generator().manual_seed(31)
