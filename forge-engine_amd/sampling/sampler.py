@@ -68,15 +68,15 @@ class Sampler:
             return []
         if not (len(params) == len(seeds) == len(draw_index) == rows):
             raise ValueError("one parameter set, seed and draw index per logits row is needed")
-        tokens = torch.empty(rows, dtype=torch.int32, device=self.device)
-        status = torch.empty(rows, dtype=torch.int32, device=self.device)
+        both = torch.empty((2, rows), dtype=torch.int32, device=self.device)   # one transfer brings both back
+        tokens, status = both[0], both[1]
         greedy = [r for r in range(rows) if params[r].greedy]
         drawn = [r for r in range(rows) if not params[r].greedy]
         if not drawn:
             ops.argmax_rows(logits, tokens, status)
         else:
             self._mixed(logits, params, seeds, draw_index, greedy, drawn, tokens, status)
-        host = torch.stack((tokens, status)).cpu()
+        host = both.cpu()
         _raise_on_status(host[1].tolist())
         return host[0].tolist()
 
