@@ -147,15 +147,52 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
     const float* __restrict__ inv_freq, const int* __restrict__ positions,
     const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_stride,
     bf16_t* __restrict__ key_pages, bf16_t* __restrict__ value_pages, int q_heads, int kv_heads,
-    int block_size, int num_blocks, float eps, int write_kv, int heads_per_block, int groups_per_token) {
+    int block_size, int num_blocks, float eps, int write_kv, int heads_per_block, int groups_per_token,
+    int tokens, int values_apart) {
   constexpr int D = LPH * 8;
   constexpr int HALF = D / 2;
   constexpr int HEADS_AT_ONCE = 256 / LPH;
+  const int heads_all = q_heads + 2 * kv_heads;
+  if (values_apart && (int)blockIdx.x >= tokens * groups_per_token) {
+    // Values of 16 neighbouring tokens and one kv head, turned through LDS: a token's value is
+    // a row of the projection's output and a column of its page ([D][slot]), so written token
+    // by token every element is a 2-byte store of its own, 2 * block_size bytes from the next.
+    // Here 16 lanes write 16 neighbouring slots of one dim (tokens of one sequence follow one
+    // another in the batch), which the memory system takes as one piece.
+    constexpr int PITCH = D + 8;            // elements; rows stay 16-byte aligned, columns spread over the banks
+    __shared__ __attribute__((aligned(16))) bf16_t rows[16][PITCH];
+    __shared__ long long slot_at[16];       // element offset of [page][kv_head][0][slot], or -1
+    const int vb = blockIdx.x - tokens * groups_per_token;
+    const int kv_head = vb % kv_heads;
+    const int t0 = (vb / kv_heads) * 16;
+    if (threadIdx.x < 16) {
+      const int t = t0 + threadIdx.x;
+      long long at = -1;
+      if (t < tokens) {
+        const int pos = positions[t];
+        const int block = block_table[(size_t)token_seq[t] * table_stride + pos / block_size];
+        if (block >= 0 && block < num_blocks)       // host reserves pages before the launch
+          at = ((long long)block * kv_heads + kv_head) * block_size * D + pos % block_size;
+      }
+      slot_at[threadIdx.x] = at;
+    }
+    for (int piece = threadIdx.x; piece < 16 * LPH; piece += 256) {
+      const int row = piece / LPH, sub = piece % LPH;
+      const int t = min(t0 + row, tokens - 1);
+      *(uint4*)&rows[row][sub * 8] =
+          *(const uint4*)(qkv + ((size_t)t * heads_all + q_heads + kv_heads + kv_head) * D + sub * 8);
+    }
+    __syncthreads();
+    const int row = threadIdx.x & 15;
+    const long long at = slot_at[row];
+    if (at < 0) return;
+    for (int d = threadIdx.x >> 4; d < D; d += 16) value_pages[at + (long long)d * block_size] = rows[row][d];
+    return;
+  }
   __shared__ float cos_s[HALF], sin_s[HALF];
   const int t = blockIdx.x / groups_per_token;
   const int group = blockIdx.x - t * groups_per_token;
-  const int heads_all = q_heads + 2 * kv_heads;
-  const int head_end = min(heads_all, (group + 1) * heads_per_block);
+  const int head_end = min(values_apart ? q_heads + kv_heads : heads_all, (group + 1) * heads_per_block);
   const int pos = positions[t];
   for (int j = threadIdx.x; j < HALF; j += blockDim.x) {
     float sn, cs;
@@ -239,14 +276,18 @@ extern "C" int fe_qk_norm_rope_write(void* qkv, int dtype, const float* q_weight
   // the vector kernel works on 2048 / head_dim heads at once
   const int heads_per_block = tokens >= 256 ? heads_all : (vec ? 2048 / head_dim : 4);
   const int groups_per_token = (heads_all + heads_per_block - 1) / heads_per_block;
-  const long long blocks = (long long)tokens * groups_per_token;
+  long long blocks = (long long)tokens * groups_per_token;
   if (blocks > 0x7fffffffLL) return FE_BAD_ARGUMENT;
   if (vec) {
+    // with many tokens the values go to blocks of their own that write 16 slots of a page at a time
+    const int values_apart = write_kv && kv_heads > 0 && tokens >= 256;
+    if (values_apart) blocks += (long long)((tokens + 15) / 16) * kv_heads;
+    if (blocks > 0x7fffffffLL) return FE_BAD_ARGUMENT;
 #define FE_GO(LPH)                                                                                          \
   qk_norm_rope_write_vec_kernel<LPH><<<(unsigned)blocks, 256, 0, stream>>>(                                   \
       (bf16_t*)qkv, q_weight, k_weight, inv_freq, positions, token_seq, block_table, table_stride,            \
       (bf16_t*)key_pages, (bf16_t*)value_pages, q_heads, kv_heads, block_size, num_blocks, eps, write_kv,     \
-      heads_per_block, groups_per_token)
+      heads_per_block, groups_per_token, tokens, values_apart)
     if (head_dim == 64) FE_GO(8);
     else if (head_dim == 128) FE_GO(16);
     else FE_GO(32);
