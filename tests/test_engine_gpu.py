@@ -773,3 +773,50 @@ def test_batched_decode_through_graphs_matches_eager(dtype, folders):
     bound = 1e-4 * scale if dtype == "float32" else ru.BF16_FRACTION * scale
     assert float((rows[True] - rows[False]).abs().max()) <= bound * 0.5
     assert float((rows[True] - want).abs().max()) <= bound
+
+
+def test_steps_of_single_tokens_prepare_queries_and_keys_inside_attention(folders, monkeypatch):
+    """A step in which every request brings one token runs norm, rotation, cache write and
+    attention as one launch per layer; a mixed step runs them as two.  The same tokens fed
+    both ways (the others' single tokens beside a two-token portion of one request, then the
+    same single tokens alone) give the same cache and logits within rounding."""
+    from forge_engine_amd.kernels import ops
+    name = "C"          # head size 128, five query heads a kv head: sizes the fast kernels serve
+    config = TINY[name]
+    requests = ru.make_requests(config, 29, (40, 33, 21))
+    _, model = load_model(folders[name], dtype="bfloat16", device=DEV)
+    calls = {"one": 0, "two": 0}
+    one, two = ops.decode_attention_prepare, ops.qk_norm_rope_write
+
+    def count_one(*args, **kwargs):
+        calls["one"] += 1
+        return one(*args, **kwargs)
+
+    def count_two(*args, **kwargs):
+        calls["two"] += 1
+        return two(*args, **kwargs)
+
+    monkeypatch.setattr(ops, "decode_attention_prepare", count_one)
+    monkeypatch.setattr(ops, "qk_norm_rope_write", count_two)
+    layers = config["num_hidden_layers"]
+    got = {}
+    for mode in ("alone", "beside a portion"):
+        runner = ModelRunner(model, block_size=16, block_capacity=40, num_state_slots=6, use_graphs=False)
+        for k, tokens in requests.items():
+            runner.begin(k)
+            runner.step([StepEntry(k, tokens[:-6], [])])
+        runner.begin("other")
+        calls["one"] = calls["two"] = 0
+        rows = []
+        for step in range(6):
+            entries = [StepEntry(k, [tokens[len(tokens) - 6 + step]], [0]) for k, tokens in requests.items()]
+            if mode == "beside a portion":
+                entries.append(StepEntry("other", [3 + step, 5 + step], []))
+            rows.append(runner.step(entries).clone())
+        got[mode] = torch.stack(rows).cpu()
+        assert (calls["one"], calls["two"]) == ((6 * layers, 0) if mode == "alone" else (0, 6 * layers))
+    want = torch.stack([plain.forward(folder_weights(folders[name]), config, tokens)[-6:] for tokens in requests.values()], dim=1)
+    bound = ru.BF16_FRACTION * float(want.abs().max())
+    assert float((got["alone"] - want).abs().max()) <= bound
+    assert float((got["beside a portion"] - want).abs().max()) <= bound
+    assert float((got["alone"] - got["beside a portion"]).abs().max()) <= bound * 0.5
