@@ -820,3 +820,62 @@ def test_steps_of_single_tokens_prepare_queries_and_keys_inside_attention(folder
     assert float((got["alone"] - want).abs().max()) <= bound
     assert float((got["beside a portion"] - want).abs().max()) <= bound
     assert float((got["alone"] - got["beside a portion"]).abs().max()) <= bound * 0.5
+
+
+@pytest.fixture(scope="module")
+def wide_folder(tmp_path_factory):
+    """Two layers with the widths, head counts and vocabulary of Qwen3-4B."""
+    config = dict(TINY["C"], vocab_size=151936, hidden_size=2560, intermediate_size=9728, num_hidden_layers=2,
+                  num_attention_heads=32, num_key_value_heads=8, head_dim=128, max_position_embeddings=4096,
+                  rms_norm_eps=1e-6, rope_theta=5000000.0, tie_word_embeddings=True)
+    folder = tmp_path_factory.mktemp("engine_wide")
+    write_random_model(load_model_config(config), 37, folder)
+    weights = folder_weights(folder)
+    return folder, config, weights
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_of_the_large_model_against_the_plain_implementation(dtype, wide_folder):
+    """The kernels at the sizes they are tuned for (weight-streaming products with resident
+    blocks and K in parts, a vocabulary that is no power of two, four query heads a kv head):
+    a prompt whole, another with its last tokens one by one, and eight requests decoding
+    together through a captured graph, all against the plain implementation."""
+    folder, config, weights = wide_folder
+    _, model = load_model(folder, dtype=dtype, device=DEV)
+    requests = ru.make_requests(config, 41, (150, 97, 40, 43, 46, 49, 52, 55, 58, 61))
+    runner = ModelRunner(model, block_size=16, block_capacity=80, num_state_slots=12)
+    got, want = {}, {}
+
+    def keep(request_id, positions, logits):
+        for row, position in zip(logits.cpu(), positions):
+            got[(request_id, position)] = row.clone()
+
+    # whole: the last 8 places of one step
+    runner.begin("r0")
+    keep("r0", range(142, 150), runner.step([StepEntry("r0", requests["r0"], list(range(142, 150)))]))
+    runner.end("r0")
+    # most of it in one step, the last 12 one by one
+    runner.begin("r1")
+    tokens = requests["r1"]
+    keep("r1", [84], runner.step([StepEntry("r1", tokens[:85], [84])]))
+    for position in range(85, 97):
+        keep("r1", [position], runner.step([StepEntry("r1", [tokens[position]], [0])]))
+    runner.end("r1")
+    # eight together: prompts one after the other, then five steps of eight single tokens
+    group = [f"r{i}" for i in range(2, 10)]
+    for k in group:
+        runner.begin(k)
+        runner.step([StepEntry(k, requests[k][:-5], [])])
+    for step in range(5):
+        logits = runner.step([StepEntry(k, [requests[k][len(requests[k]) - 5 + step]], [0]) for k in group])
+        for row, k in zip(logits.cpu(), group):
+            got[(k, len(requests[k]) - 5 + step)] = row.clone()
+    assert runner.graph_replays >= 5 + 12
+    for k in group:
+        runner.end(k)
+    for request_id, tokens in requests.items():
+        logits = plain.forward(weights, config, tokens)
+        for (rid, position) in got:
+            if rid == request_id:
+                want[(rid, position)] = logits[position]
+    ru.compare(got, want, dtype)
