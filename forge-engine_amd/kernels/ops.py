@@ -243,13 +243,15 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
 
 
 # Measured on MI355X: a weight with few row tiles and a long K (the output and down projections: 160
-# tiles, K = 4096 and 9728) leaves CUs idle; parts of K of about four 128-steps each, summed by blocks
-# of four waves, take 7.0 instead of 9.5 us and 13.9 instead of 18.4 us at 8 rows.  The consumer
-# (add_rmsnorm, add_rows) adds the parts in order.
+# tiles, K = 4096 and 9728) leaves CUs idle; parts of K of at least four 128-steps each, of equal
+# length and few enough that all blocks are resident at once, summed by blocks of four waves, take
+# 7.0 instead of 9.5 us and 13.9 instead of 18.4 us at 8 rows.  The consumer (add_rmsnorm, add_rows)
+# adds the parts in order.
 UPDATE_SPLIT_MAX_TILES = 256
 UPDATE_SPLIT_MIN_STEPS = 32
 UPDATE_SPLIT_STEPS = 4
 UPDATE_SPLIT_MAX = 16
+UPDATE_SPLIT_BLOCKS = 1536     # blocks of four waves aimed at: all resident at once, parts of equal length
 
 
 # Between 17 and 64 rows the product is still bound by the weight's bytes; the matrix library needs
@@ -283,7 +285,9 @@ def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tens
     if (plain_bf16 and _skinny_fits(x, weight)
             and -(-weight.shape[0] // 16) <= UPDATE_SPLIT_MAX_TILES
             and -(-weight.shape[1] // 128) >= UPDATE_SPLIT_MIN_STEPS):
-        splits = min(UPDATE_SPLIT_MAX, -(-weight.shape[1] // 128) // UPDATE_SPLIT_STEPS)
+        steps, tiles = -(-weight.shape[1] // 128), -(-weight.shape[0] // 16)
+        splits = max(1, min(UPDATE_SPLIT_MAX, steps // UPDATE_SPLIT_STEPS, UPDATE_SPLIT_BLOCKS // tiles))
+        splits = -(-steps // -(-steps // splits))        # parts of equal length, none empty
         return gemm_skinny(x, weight, "f32", tiles=1, waves=4, splits=splits)
     if plain_bf16 and x.shape[0] > SKINNY_MAX_ROWS and _skinny_fits(x, weight, MID_ROWS):
         steps = -(-weight.shape[1] // 128)
