@@ -414,6 +414,33 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   __syncthreads();
   if (!is_last) return;
   const size_t first_part = ((size_t)seq * kv_heads + hk) * splits;
+  if (splits <= 8) {
+    // few splits: every thread reads the statistics of its row itself, together with its share
+    // of the partial outputs, so that all loads are in flight at once (same sums, same order)
+    for (int e = tid; e < groups * D; e += 256) {
+      const int g = e / D, d = e - g * D;
+      float m[8], l[8], o[8];
+#pragma unroll
+      for (int sp = 0; sp < 8; ++sp) {
+        const size_t row = (first_part + (sp < splits ? sp : 0)) * groups + g;
+        m[sp] = load_agent(&part_ml[row * 2]);
+        l[sp] = load_agent(&part_ml[row * 2 + 1]);
+        o[sp] = load_agent(&part_o[row * D + d]);
+      }
+      float m_tot = -INFINITY;
+#pragma unroll
+      for (int sp = 0; sp < 8; ++sp) m_tot = fmaxf(m_tot, sp < splits ? m[sp] : -INFINITY);
+      float l_tot = 0.f, ov = 0.f;
+#pragma unroll
+      for (int sp = 0; sp < 8; ++sp) {
+        const float f = (sp < splits && m_tot > -INFINITY) ? __builtin_amdgcn_exp2f(m[sp] - m_tot) : 0.f;
+        l_tot += f * l[sp];
+        ov += f * o[sp];
+      }
+      out[(size_t)q0 * out_stride + (size_t)(hk * groups + g) * D + d] = float_to_bf16(ov * (l_tot > 0.f ? 1.f / l_tot : 0.f));
+    }
+    return;
+  }
   if (tid < groups) {
     const int g = tid;
     float m_tot = -INFINITY;
