@@ -53,6 +53,31 @@ __device__ __forceinline__ float load_agent(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// One output element from up to N splits: all loads first, then the sums in split order.
+template <int N>
+__device__ __forceinline__ bf16_t merge_few(const float* part_o, const float* part_ml, size_t first_part,
+                                            int splits, int groups, int g, int dim, int d) {
+  float m[N], l[N], o[N];
+#pragma unroll
+  for (int sp = 0; sp < N; ++sp) {
+    const size_t row = (first_part + (sp < splits ? sp : 0)) * groups + g;
+    m[sp] = load_agent(&part_ml[row * 2]);
+    l[sp] = load_agent(&part_ml[row * 2 + 1]);
+    o[sp] = load_agent(&part_o[row * dim + d]);
+  }
+  float m_tot = -INFINITY;
+#pragma unroll
+  for (int sp = 0; sp < N; ++sp) m_tot = fmaxf(m_tot, sp < splits ? m[sp] : -INFINITY);
+  float l_tot = 0.f, ov = 0.f;
+#pragma unroll
+  for (int sp = 0; sp < N; ++sp) {
+    const float f = (sp < splits && m_tot > -INFINITY) ? __builtin_amdgcn_exp2f(m[sp] - m_tot) : 0.f;
+    l_tot += f * l[sp];
+    ov += f * o[sp];
+  }
+  return float_to_bf16(ov * (l_tot > 0.f ? 1.f / l_tot : 0.f));
+}
+
 // What the PREPARE variant needs beyond the plain one: the norms' weights (null: no norm), the
 // rotation's frequencies [D / 2], and the pages as writable memory.
 struct Prepare {
@@ -414,30 +439,15 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   __syncthreads();
   if (!is_last) return;
   const size_t first_part = ((size_t)seq * kv_heads + hk) * splits;
-  if (splits <= 8) {
+  if (splits <= 16) {
     // few splits: every thread reads the statistics of its row itself, together with its share
     // of the partial outputs, so that all loads are in flight at once (same sums, same order)
     for (int e = tid; e < groups * D; e += 256) {
       const int g = e / D, d = e - g * D;
-      float m[8], l[8], o[8];
-#pragma unroll
-      for (int sp = 0; sp < 8; ++sp) {
-        const size_t row = (first_part + (sp < splits ? sp : 0)) * groups + g;
-        m[sp] = load_agent(&part_ml[row * 2]);
-        l[sp] = load_agent(&part_ml[row * 2 + 1]);
-        o[sp] = load_agent(&part_o[row * D + d]);
-      }
-      float m_tot = -INFINITY;
-#pragma unroll
-      for (int sp = 0; sp < 8; ++sp) m_tot = fmaxf(m_tot, sp < splits ? m[sp] : -INFINITY);
-      float l_tot = 0.f, ov = 0.f;
-#pragma unroll
-      for (int sp = 0; sp < 8; ++sp) {
-        const float f = (sp < splits && m_tot > -INFINITY) ? __builtin_amdgcn_exp2f(m[sp] - m_tot) : 0.f;
-        l_tot += f * l[sp];
-        ov += f * o[sp];
-      }
-      out[(size_t)q0 * out_stride + (size_t)(hk * groups + g) * D + d] = float_to_bf16(ov * (l_tot > 0.f ? 1.f / l_tot : 0.f));
+      bf16_t* dst = out + (size_t)q0 * out_stride + (size_t)(hk * groups + g) * D + d;
+      if (splits <= 4) *dst = merge_few<4>(part_o, part_ml, first_part, splits, groups, g, D, d);
+      else if (splits <= 8) *dst = merge_few<8>(part_o, part_ml, first_part, splits, groups, g, D, d);
+      else *dst = merge_few<16>(part_o, part_ml, first_part, splits, groups, g, D, d);
     }
     return;
   }
