@@ -85,7 +85,13 @@ struct Prepare {
   const float* k_weight;
   const float* inv_freq;
   float eps;
+  // the projection's output as float32 partial sums [num_sums][rows][q_stride] instead of one
+  // bfloat16 matrix (a product whose K was split over blocks): added up in order and rounded here
+  const float* sums;
+  int num_sums;
+  long long sum_stride;
 };
+#define MAX_SUMS 8
 
 template <int D, bool PREPARE>
 __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
@@ -128,6 +134,30 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     sin_s[tid] = sn;
   }
 
+  // From partial sums: this block's query heads, key head and value head are added up once,
+  // rounded to bfloat16 and kept in LDS (all parts' loads in flight together).
+  __shared__ __attribute__((aligned(16))) bf16_t raw_s[PREPARE ? (GMAX + 2) * D : 8];
+  const bool from_sums = PREPARE && prep.num_sums > 0;
+  if (from_sums) {
+    for (int piece = tid; piece < (groups + 2) * (D / 4); piece += 256) {
+      const int head = piece / (D / 4), d = (piece - head * (D / 4)) * 4;
+      const int column_head = head < groups ? hk * groups + head
+                                            : kv_heads * groups + (head - groups) * kv_heads + hk;
+      const float* src = prep.sums + (size_t)q0 * q_stride + (size_t)column_head * D + d;
+      float4 part[MAX_SUMS];
+#pragma unroll
+      for (int i = 0; i < MAX_SUMS; ++i) part[i] = *(const float4*)(src + (size_t)min(i, prep.num_sums - 1) * prep.sum_stride);
+      float4 sum = part[0];
+#pragma unroll
+      for (int i = 1; i < MAX_SUMS; ++i)
+        if (i < prep.num_sums) { sum.x += part[i].x; sum.y += part[i].y; sum.z += part[i].z; sum.w += part[i].w; }
+      uint2 packed;
+      packed.x = (uint32_t)float_to_bf16(sum.x) | ((uint32_t)float_to_bf16(sum.y) << 16);
+      packed.y = (uint32_t)float_to_bf16(sum.z) | ((uint32_t)float_to_bf16(sum.w) << 16);
+      *(uint2*)&raw_s[head * D + d] = packed;
+    }
+  }
+
   // query rows as the B operand: lane (lr = row g, lq) holds q[g][32c + 8lq .. +8]
   bf16x8 qb[KC];
   {
@@ -135,7 +165,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
 #pragma unroll
     for (int c = 0; c < KC; ++c) {
       uintx4 v = uintx4{0u, 0u, 0u, 0u};
-      if (lr < groups) v = *(const uintx4*)(qrow + c * 32 + lq * 8);
+      if (lr < groups && !from_sums) v = *(const uintx4*)(qrow + c * 32 + lq * 8);
       qb[c] = __builtin_bit_cast(bf16x8, v);
     }
   }
@@ -247,7 +277,11 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
 
   bool extra = false;       // this block also brings the new token's own key and value
   if constexpr (PREPARE) {
-    __syncthreads();        // cos_s, sin_s
+    __syncthreads();        // cos_s, sin_s, raw_s
+    if (from_sums && lr < groups) {
+#pragma unroll
+      for (int c = 0; c < KC; ++c) qb[c] = *(const bf16x8*)&raw_s[lr * D + c * 32 + lq * 8];
+    }
     // Queries: chunk 4c + lq of head row lr sits in qb[c].  Norm, rotation and rounding as the
     // stand-alone kernel does them: the butterfly over chunks runs over c first, then over lq.
     float qv[KC][8];
@@ -310,7 +344,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
       const int pos = ctx - 1;
       const bf16_t* row = q + (size_t)q0 * q_stride;
       const size_t k_at = (size_t)(kv_heads * groups + hk) * D, v_at = k_at + (size_t)kv_heads * D;
-      const uint4 raw = *(const uint4*)(row + (role == 1 ? v_at : k_at) + sub * 8);
+      const uint4 raw = from_sums ? *(const uint4*)&raw_s[(groups + (role == 1 ? 1 : 0)) * D + sub * 8]
+                                  : *(const uint4*)(row + (role == 1 ? v_at : k_at) + sub * 8);
       const int block = table[min(pos >> block_shift, table_last)];
       const bool writable = block >= 0 && block < num_blocks;     // the host reserves pages before the launch
       const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -489,7 +524,7 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
   if (splits > 1 && (!part_o || !part_ml || !counters)) return FE_BAD_ARGUMENT;
   dim3 grid(splits, kv_heads, num_seqs);
   const float scale_log2 = scale * 1.4426950408889634f;
-  const Prepare none = {nullptr, nullptr, nullptr, 0.f};
+  const Prepare none = {nullptr, nullptr, nullptr, 0.f, nullptr, 0, 0};
 #define FE_GO(DD, PP)                                                                                      \
   paged_decode_kernel<DD, PP><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
@@ -530,7 +565,11 @@ extern "C" int fe_paged_attention_decode(const void* q, long long q_stride, cons
 // stride q_stride]: q and k heads are normalised (weights [head_dim] float32, null: no norm)
 // and rotated whole by position ctx_len - 1 (inv_freq [head_dim / 2]), and each sequence's new
 // key and value are written to slot ctx_len - 1 of its pages.  qkv itself is not changed.
-extern "C" int fe_paged_attention_decode_prepare(const void* qkv, long long q_stride, const float* q_weight,
+// qkv_sums > 0 (at most 8): qkv is float32 and holds that many partial sums of the projection,
+// sum_stride floats apart, each [num_seqs rows, row stride q_stride]; they are added up in order
+// and rounded to bfloat16 first.
+extern "C" int fe_paged_attention_decode_prepare(const void* qkv, int qkv_sums, long long sum_stride,
+                                                 long long q_stride, const float* q_weight,
                                                  const float* k_weight, const float* inv_freq, float eps,
                                                  void* key_pages, void* value_pages, void* out,
                                                  long long out_stride, float* part_o, float* part_ml,
@@ -542,7 +581,9 @@ extern "C" int fe_paged_attention_decode_prepare(const void* qkv, long long q_st
   if (!inv_freq || (!q_weight) != (!k_weight)) return FE_BAD_ARGUMENT;
   if (q_weight && ((((uintptr_t)q_weight) | ((uintptr_t)k_weight)) & 15)) return FE_BAD_ARGUMENT;
   if (q_stride < (long long)(kv_heads * groups + 2 * kv_heads) * head_dim) return FE_BAD_ARGUMENT;
-  const Prepare prep = {q_weight, k_weight, inv_freq, eps};
+  if (qkv_sums < 0 || qkv_sums > MAX_SUMS) return FE_BAD_ARGUMENT;
+  if (qkv_sums > 0 && (q_stride % 4 || sum_stride % 4 || sum_stride < (long long)num_seqs * q_stride)) return FE_BAD_ARGUMENT;
+  const Prepare prep = {q_weight, k_weight, inv_freq, eps, qkv_sums > 0 ? (const float*)qkv : nullptr, qkv_sums, sum_stride};
   return launch_decode(qkv, q_stride, key_pages, value_pages, out, out_stride, part_o, part_ml, counters, cu_q,
                        ctx_len, block_table, table_stride, num_seqs, kv_heads, groups, head_dim, block_size,
                        num_blocks, window, scale, splits, &prep, stream);

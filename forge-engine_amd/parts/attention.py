@@ -116,9 +116,12 @@ class GroupedQueryAttention(Mixer):
         inv_freq, rotary_dim = rotary if rotary is not None else (None, 0)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 1.0
         if writes_cache:
-            qkv = ops.linear(x, self.qkv_weight, self.qkv_bias)
             if self._single_tokens_only(batch, x, cache, rotary_dim):
-                # norms, rotation, cache write and attention in one launch
+                # norms, rotation, cache write and attention in one launch, which also adds up
+                # the projection's partial sums where the product is faster with K in parts
+                qkv = ops.linear_in_parts(x, self.qkv_weight) if self.qkv_bias is None else None
+                if qkv is None:
+                    qkv = ops.linear(x, self.qkv_weight, self.qkv_bias)
                 attn = torch.empty((x.shape[0], self.q_size), dtype=x.dtype, device=x.device)
                 ops.decode_attention_prepare(
                     qkv, self.q_norm, self.k_norm, inv_freq, cache.key_pages, cache.value_pages, attn,
@@ -126,6 +129,7 @@ class GroupedQueryAttention(Mixer):
                     kv_heads=self.num_kv_heads, head_dim=self.head_dim, eps=eps, scale=self.scale,
                     window=self.window, max_ctx=batch.max_ctx)
                 return ops.linear_update(attn, self.o_weight, self.o_bias)
+            qkv = ops.linear(x, self.qkv_weight, self.qkv_bias)
         else:  # another call wrote the keys and values this one reads: only q is needed
             bias = None if self.qkv_bias is None else self.qkv_bias[:self.q_size]
             qkv = ops.linear(x, self.qkv_weight[:self.q_size], bias)

@@ -210,7 +210,15 @@ def sample_rows(logits, temperatures, seeds, draw_index, tokens, status):
         tokens[r] = min(pick, logits.shape[1] - 1)
 
 
-NAMES = ("embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_update", "linear_swiglu", "gemm_skinny",
+def decode_prepare_supported(*args, **kwargs):
+    return False        # on the CPU a step of single tokens takes the two references below in turn
+
+
+def linear_in_parts(x, weight):
+    return None
+
+
+NAMES = ("decode_prepare_supported", "linear_in_parts", "embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_update", "linear_swiglu", "gemm_skinny",
          "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_rows")
 
 

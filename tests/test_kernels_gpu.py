@@ -632,6 +632,53 @@ def test_decode_attention_that_prepares_its_queries_and_keys(ops, q_heads, kv_he
     assert torch.equal(vp_one.cpu(), vp_ref)
 
 
+@pytest.mark.parametrize("parts", [1, 2, 5, 8])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [(32, 8, 128, 16), (5, 5, 64, 32), (8, 1, 256, 16)])
+def test_decode_attention_that_prepares_from_partial_sums(ops, q_heads, kv_heads, head_dim, block_size, parts):
+    """The projection's output as float32 partial sums: added up in order and rounded to bfloat16
+    inside the kernel, after which everything is as with the rounded matrix as input (same
+    output, same bits in the pages)."""
+    g = torch.Generator().manual_seed(37)
+    contexts = [0, 15, 16, 300, 77]
+    qkv, kp, vp, cu, ctx, table, qw, kw, inv_freq, _, _ = _prepare_case(g, q_heads, kv_heads, head_dim, block_size, contexts)
+    n = len(contexts)
+    sums = rand(g, parts, n, qkv.shape[1])
+    total = sums[0].clone()
+    for part in sums[1:]:
+        total += part
+    rounded = total.to(torch.bfloat16)
+    sizes = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim)
+    results = []
+    for source in (rounded, sums):
+        kp_dev, vp_dev, src = kp.to(DEV), vp.to(DEV), source.to(DEV)
+        out = torch.full((n, q_heads * head_dim), float("nan"), dtype=torch.bfloat16, device=DEV)
+        for splits in (1, 3):
+            ops.decode_attention_prepare(src, qw.to(DEV), kw.to(DEV), inv_freq.to(DEV), kp_dev, vp_dev, out, cu.to(DEV),
+                                         ctx.to(DEV), table.to(DEV), eps=1e-6, scale=head_dim ** -0.5, max_ctx=301,
+                                         splits=splits, **sizes)
+        assert torch.equal(src.cpu(), source)
+        results.append((out.cpu(), kp_dev.cpu(), vp_dev.cpu()))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    with pytest.raises(ops.KernelError):
+        ops.decode_attention_prepare(rand(g, 9, n, qkv.shape[1]).to(DEV), qw.to(DEV), kw.to(DEV), inv_freq.to(DEV), kp.to(DEV),
+                                     vp.to(DEV), torch.empty(n, q_heads * head_dim, dtype=torch.bfloat16, device=DEV), cu.to(DEV),
+                                     ctx.to(DEV), table.to(DEV), eps=1e-6, scale=1.0, **sizes)
+
+
+def test_linear_in_parts(ops):
+    g = torch.Generator().manual_seed(38)
+    w = rand(g, 6144, 2560, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    for rows in (1, 8, 16, 17, 64):
+        x = rand(g, rows, 2560, dtype=torch.bfloat16).to(DEV)
+        sums = ops.linear_in_parts(x, w)
+        assert sums.dtype == torch.float32 and sums.dim() == 3 and sums.shape[0] <= 8 and sums.shape[1:] == (rows, 6144)
+        torch.testing.assert_close(sums.sum(0).cpu(), x.cpu().float() @ w.cpu().float().T, atol=2e-3, rtol=2e-3)
+    assert ops.linear_in_parts(rand(g, 65, 2560, dtype=torch.bfloat16).to(DEV), w) is None       # many rows: the library
+    assert ops.linear_in_parts(rand(g, 4, 256, dtype=torch.bfloat16).to(DEV), w[:, :256]) is None  # a short K
+    assert ops.linear_in_parts(rand(g, 4, 2560).to(DEV), w.float()) is None                        # not bfloat16
+
+
 @pytest.mark.parametrize("window", [1, 16, 37, 300])
 def test_decode_attention_that_prepares_with_a_window(ops, window):
     g = torch.Generator().manual_seed(34)
