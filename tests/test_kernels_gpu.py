@@ -44,7 +44,7 @@ def test_embed_rows(ops, dtype, hidden):
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("delta_dtype", [None, torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hidden", [24, 200, 2560, 5000])
-@pytest.mark.parametrize("n", [7, 23])          # few rows of a wide stream take a kernel with more threads a row
+@pytest.mark.parametrize("n", [7, 23, 600])     # up to 512 rows of a wide stream take a kernel with more threads a row
 def test_add_rmsnorm(ops, out_dtype, delta_dtype, hidden, n):
     g = torch.Generator().manual_seed(1)
     h = rand(g, n, hidden, scale=3.0)
