@@ -8,8 +8,8 @@
 //
 // Block = 64 weight rows (four waves of 16) x one part of K.  The weight goes from
 // HBM straight into MFMA operand registers, each element used by one wave only;
-// x (shared by the four waves) is staged through LDS in 128-wide steps, two
-// stages, one barrier a step.  A wave needs no other wave's sums: its 16 weight
+// x (shared by the four waves) is staged through LDS in 128-wide steps, three
+// stages, one barrier a step, operands fetched two steps ahead.  A wave needs no other wave's sums: its 16 weight
 // rows are its own, so there is no reduction at the end.
 //
 // MFMA 16x16x32 bf16 with A = x (16 rows), B = W^T (16 weight rows):
@@ -27,11 +27,18 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 // MT row tiles of x (16 rows each).  LDS holds a step of x as [row][16 chunks of 16 bytes], chunk c
 // of row r at position c ^ (r % 16): the 16 lanes that read one chunk index of 16 rows then hit
 // 16 different bank groups.
+//
+// A step's operands are fetched two steps before they are used: a step's arithmetic (16 MFMAs
+// at 64 rows) is far shorter than a trip to memory, and a part of K is only a few steps long.
+// Three register sets rotate through a loop unrolled three times; the one or two steps that
+// remain run after it from the sets they were fetched into.  Every load is unconditional (past
+// the part's end the last step is read again and not used), so the loop body is straight-line
+// code and the loads stay where they are issued.
 template <int MT>
-__global__ __launch_bounds__(256) void gemm_mid_parts_kernel(
+__global__ __launch_bounds__(256, 2) void gemm_mid_parts_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ out, int M, int N,
     int K, long long ldw, long long ldo, int steps_per_part, long long part_stride) {
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][KSTEP];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[3][MT * 16][KSTEP];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -47,67 +54,71 @@ __global__ __launch_bounds__(256) void gemm_mid_parts_kernel(
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // x loader: piece p = tid + 256 i is chunk p % 16 of row p / 16 (MT pieces a thread)
-  uintx4 xr[MT];
-  auto load_x = [&](int step) {
+  if (first < last) {
+    uintx4 xr[3][MT], wr[3][4];
+    // x loader: piece p = tid + 256 i is chunk p % 16 of row p / 16 (MT pieces a thread)
+    // K is a multiple of the step, and rows of x beyond M read row 0 again: their sums are
+    // never stored.  Nothing is selected on a loaded value, so no load is waited for where it
+    // is issued.
+    auto load = [&](int step, uintx4* xdst, uintx4* wdst) {
+      step = min(step, last - 1);
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      const int p = tid + 256 * i;
-      const int row = p >> 4, k = step * KSTEP + (p & 15) * 8;
-      const bool ok = row < M && k < K;
-      const uintx4 v = *(const uintx4*)(x + (size_t)(ok ? row : 0) * K + (ok ? k : 0));
-      xr[i] = ok ? v : uintx4{0u, 0u, 0u, 0u};
-    }
-  };
-  auto store_x = [&](int stage) {
+      for (int i = 0; i < MT; ++i) {
+        const int p = tid + 256 * i;
+        const int row = p >> 4;
+        xdst[i] = *(const uintx4*)(x + (size_t)(row < M ? row : 0) * K + step * KSTEP + (p & 15) * 8);
+      }
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      const int p = tid + 256 * i;
-      const int row = p >> 4;
-      *(uintx4*)&xs[stage][row][(((p & 15) ^ (row & 15))) * 8] = xr[i];
-    }
-  };
-  uintx4 wa[4], wb[4];
-  auto load_w = [&](int step, uintx4* dst) {
-    const int k = step * KSTEP + lq * 8;
+      for (int c = 0; c < 4; ++c) wdst[c] = *(const uintx4*)(wrow + step * KSTEP + lq * 8 + c * 32);
+    };
+    auto store_x = [&](int stage, const uintx4* xsrc) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) dst[c] = *(const uintx4*)(wrow + (k + c * 32 < K ? k + c * 32 : 0));   // x is zero beyond K
-  };
-  auto multiply = [&](int stage, const uintx4* wreg) {
+      for (int i = 0; i < MT; ++i) {
+        const int p = tid + 256 * i;
+        const int row = p >> 4;
+        *(uintx4*)&xs[stage][row][(((p & 15) ^ (row & 15))) * 8] = xsrc[i];
+      }
+    };
+    auto multiply = [&](int stage, const uintx4* wreg) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const bf16x8 b = __builtin_bit_cast(bf16x8, wreg[c]);
+      for (int c = 0; c < 4; ++c) {
+        const bf16x8 b = __builtin_bit_cast(bf16x8, wreg[c]);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int row = mt * 16 + lr;
-        const bf16x8 a = *(const bf16x8*)&xs[stage][row][((c * 4 + lq) ^ lr) * 8];
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+        for (int mt = 0; mt < MT; ++mt) {
+          const int row = mt * 16 + lr;
+          const bf16x8 a = *(const bf16x8*)&xs[stage][row][((c * 4 + lq) ^ lr) * 8];
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+        }
+      }
+    };
+
+    // Step s (counted from the part's first) has its operands in register set s % 3 and its x in
+    // LDS stage s % 3.  The loop takes three steps a round so that both are compile-time constants.
+    load(first, xr[0], wr[0]);
+    load(first + 1, xr[1], wr[1]);
+    store_x(0, xr[0]);
+    __syncthreads();
+    int step = first;
+    for (; step + 3 <= last; step += 3) {
+#pragma unroll
+      for (int u = 0; u < 3; ++u) {
+        load(step + u + 2, xr[(u + 2) % 3], wr[(u + 2) % 3]);
+        multiply(u, wr[u]);
+        store_x((u + 1) % 3, xr[(u + 1) % 3]);
+        __syncthreads();
       }
     }
-  };
-
-  if (first < last) {
-    load_x(first);
-    load_w(first, wa);
-    store_x(0);
-    __syncthreads();
-    int stage = 0;
-    for (int step = first; step < last; step += 2) {
-      // even step of the pair: weights in wa; the next step's operands are fetched meanwhile
-      const bool more = step + 1 < last;
-      if (more) { load_x(step + 1); load_w(step + 1, wb); }
-      multiply(stage, wa);
-      if (!more) break;
-      store_x(stage ^ 1);
-      __syncthreads();
-      stage ^= 1;
-      const bool further = step + 2 < last;
-      if (further) { load_x(step + 2); load_w(step + 2, wa); }
-      multiply(stage, wb);
-      if (!further) break;
-      store_x(stage ^ 1);
-      __syncthreads();
-      stage ^= 1;
+    const int left = last - step;          // 0 .. 2 steps, the same for every thread
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      if (u < left) {
+        if (u + 2 < left) load(step + u + 2, xr[(u + 2) % 3], wr[(u + 2) % 3]);
+        multiply(u % 3, wr[u % 3]);
+        if (u + 1 < left) {
+          store_x((u + 1) % 3, xr[(u + 1) % 3]);
+          __syncthreads();
+        }
+      }
     }
   }
 
@@ -124,7 +135,7 @@ __global__ __launch_bounds__(256) void gemm_mid_parts_kernel(
   }
 }
 
-// x [M, K] bf16 contiguous, 16 < M <= 64 (fewer rows work too); w [N, K] bf16 with row stride ldw;
+// x [M, K] bf16 contiguous, 16 < M <= 64 (fewer rows work too), K a multiple of 128; w [N, K] bf16 with row stride ldw;
 // out: `parts` float32 matrices [M, N] (row stride ldo) part_stride floats apart, part s holding
 // the sum over the s-th run of whole 128-steps of K.  Every part is written in full (zeros where a
 // part has no steps), so the caller may add all of them up.
@@ -132,7 +143,7 @@ extern "C" int fe_gemm_mid_parts(const void* x, const void* w, float* out, int M
                                  long long ldw, long long ldo, int parts, long long part_stride,
                                  hipStream_t stream) {
   if (M < 1) return FE_OK;
-  if (M > 64 || N < 1 || K < 8 || K % 8 || ldw < K || ldw % 8 || ldo < N) return FE_BAD_ARGUMENT;
+  if (M > 64 || N < 1 || K < KSTEP || K % KSTEP || ldw < K || ldw % 8 || ldo < N) return FE_BAD_ARGUMENT;
   if ((((uintptr_t)x) & 15) || (((uintptr_t)w) & 15)) return FE_BAD_ARGUMENT;
   if (parts < 1 || parts > 64 || (parts > 1 && part_stride < (long long)M * ldo)) return FE_BAD_ARGUMENT;
   const int steps = (K + KSTEP - 1) / KSTEP;

@@ -256,9 +256,21 @@ UPDATE_SPLIT_BLOCKS = 1536     # blocks of four waves aimed at: all resident at 
 
 # Between 17 and 64 rows the product is still bound by the weight's bytes; the matrix library needs
 # 21 us for each of the two projections back to the hidden size at 64 rows (1 to 2.4 TB/s).  The
-# kernel below splits K over blocks of 64 weight rows, aiming at this many blocks.
+# kernel below splits K over blocks of 64 weight rows, aiming at this many blocks (measured at 64
+# rows: output 8.0, down 14.8, q/k/v 11.8 us; more parts make shorter pipelines and are slower).
 MID_ROWS = 64
-MID_TARGET_BLOCKS = 512
+MID_TARGET_BLOCKS = 240
+
+
+def _mid_parts(steps: int, blocks: int) -> int:
+    """Parts of K for the 17-64-row product: about MID_TARGET_BLOCKS blocks in all, at least four
+    128-steps a part (the kernel fetches two steps ahead), no part without steps."""
+    parts = max(1, min(16, MID_TARGET_BLOCKS // blocks, steps // 4))
+    return -(-steps // -(-steps // parts))
+
+
+def _mid_fits(x: Tensor, weight: Tensor) -> bool:
+    return _skinny_fits(x, weight, MID_ROWS) and weight.shape[1] % 128 == 0
 
 
 def gemm_mid_parts(x: Tensor, weight: Tensor, parts: int) -> Tensor:
@@ -266,8 +278,8 @@ def gemm_mid_parts(x: Tensor, weight: Tensor, parts: int) -> Tensor:
     of K, for up to 64 rows of bfloat16 x."""
     _gpu(x, "x", torch.bfloat16)
     _gpu(weight, "weight", torch.bfloat16, contiguous=False)
-    if not _skinny_fits(x, weight, MID_ROWS) or weight.shape[1] != x.shape[1] or not 1 <= parts <= 64:
-        raise KernelError("the product in parts takes at most 64 contiguous bfloat16 rows, K a multiple of 8, at most 64 parts")
+    if not _mid_fits(x, weight) or weight.shape[1] != x.shape[1] or not 1 <= parts <= 64:
+        raise KernelError("the product in parts takes at most 64 contiguous bfloat16 rows, K a multiple of 128, at most 64 parts")
     m, k = x.shape
     n = weight.shape[0]
     out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
@@ -289,20 +301,17 @@ def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tens
         splits = max(1, min(UPDATE_SPLIT_MAX, steps // UPDATE_SPLIT_STEPS, UPDATE_SPLIT_BLOCKS // tiles))
         splits = -(-steps // -(-steps // splits))        # parts of equal length, none empty
         return gemm_skinny(x, weight, "f32", tiles=1, waves=4, splits=splits)
-    if plain_bf16 and x.shape[0] > SKINNY_MAX_ROWS and _skinny_fits(x, weight, MID_ROWS):
+    if plain_bf16 and x.shape[0] > SKINNY_MAX_ROWS and _mid_fits(x, weight):
         steps = -(-weight.shape[1] // 128)
         blocks = -(-weight.shape[0] // 64)
-        parts = max(1, min(16, MID_TARGET_BLOCKS // blocks, steps // 2))
-        parts = -(-steps // -(-steps // parts))          # no part without steps
-        return gemm_mid_parts(x, weight, parts)
+        return gemm_mid_parts(x, weight, _mid_parts(steps, blocks))
     return linear(x, weight, bias, out_dtype=torch.float32)
 
 
 # Measured on MI355X for the q/k/v projection of Qwen3-4B (6144 x 2560): two parts of K at up to 16
-# rows take 10.1 instead of 12.0 us, five parts at 64 rows 11.9 instead of the library's 15.8.
+# rows take 10.1 instead of 12.0 us, two parts at 64 rows 11.8 instead of the library's 15.8.
 IN_PARTS_MIN_STEPS = 8
 IN_PARTS_FEW_ROWS = 2
-IN_PARTS_MORE_ROWS = 5
 
 
 def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
@@ -316,10 +325,8 @@ def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
         return None
     if _skinny_fits(x, weight):
         return gemm_skinny(x, weight, "f32", tiles=1, waves=4, splits=IN_PARTS_FEW_ROWS)
-    if _skinny_fits(x, weight, MID_ROWS):
-        parts = min(IN_PARTS_MORE_ROWS, steps // 2)
-        parts = -(-steps // -(-steps // parts))          # no part without steps
-        return gemm_mid_parts(x, weight, parts)
+    if _mid_fits(x, weight):
+        return gemm_mid_parts(x, weight, _mid_parts(steps, -(-weight.shape[0] // 64)))
     return None
 
 

@@ -458,7 +458,8 @@ def test_linear_update_routes(ops):
 
 
 @pytest.mark.parametrize("m", [17, 33, 48, 64, 5])
-@pytest.mark.parametrize("n,k,parts", [(2560, 4096, 8), (2560, 9728, 9), (200, 264, 2), (1003, 1000, 3), (64, 128, 1), (70, 8, 1)])
+@pytest.mark.parametrize("n,k,parts", [(2560, 4096, 8), (2560, 9728, 9), (200, 256, 2), (1003, 1024, 3), (64, 128, 1), (70, 640, 5),
+                                       (330, 1408, 2), (96, 2048, 16), (40, 896, 1)])
 def test_gemm_mid_parts(ops, m, n, k, parts):
     """17 to 64 rows: K in parts over blocks of 64 weight rows, x staged through LDS; the parts add
     up to the product, each row independent of the rows beside it, the same bits every time."""
@@ -483,6 +484,17 @@ def test_gemm_mid_parts(ops, m, n, k, parts):
     for part in got[1:]:
         summed += part
     assert torch.equal(ops.add_rows(h1, got), ops.add_rows(h2, summed))
+
+
+def test_gemm_mid_parts_refuses_a_k_that_is_no_multiple_of_its_step(ops):
+    g = torch.Generator().manual_seed(27)
+    x = rand(g, 20, 264, dtype=torch.bfloat16).to(DEV)
+    w = rand(g, 100, 264, dtype=torch.bfloat16).to(DEV)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_mid_parts(x, w, 2)
+    update = ops.linear_update(x, w)                      # the library takes it
+    assert update.shape == (20, 100)
+    torch.testing.assert_close(update.cpu(), x.float().cpu() @ w.float().cpu().T, atol=1e-3, rtol=1e-3)
 
 
 def test_linear_update_takes_the_mid_kernel(ops):
