@@ -82,31 +82,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 
   // One step = 128 k = four MFMAs; in MFMA c lane group lq holds k = 32*c + 8*lq .. +8 of
   // both operands, so one load instruction reads 64 contiguous bytes of each of 16 rows.
+  // Every load is unconditional: rows beyond M or N read row 0 again (their sums are never
+  // stored) and k beyond K reads the row's start (x is set to zero there where it is used, in
+  // the one step that can reach beyond K).  A load under a per-lane condition becomes a branch,
+  // and where branches meet the compiler waits for every load in flight.
   auto load = [&](StepRegs<MT, NW>& r, int step) {
     const int k = step * KSTEP + lq * 8;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      const bool k_ok = k + c * 32 < K;
+      const int at = k + c * 32 < K ? k + c * 32 : 0;
 #pragma unroll
-      for (int t = 0; t < NW; ++t) {
-        uintx4 v = uintx4{0u, 0u, 0u, 0u};
-        if (row_ok[t] && k_ok) v = *(const uintx4*)(wrow[t] + k + c * 32);
-        r.w[t][c] = v;
-      }
+      for (int t = 0; t < NW; ++t) r.w[t][c] = *(const uintx4*)(wrow[t] + at);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        uintx4 v = uintx4{0u, 0u, 0u, 0u};
-        if (x_ok[mt] && k_ok) v = *(const uintx4*)(xrow[mt] + k + c * 32);
-        r.x[mt][c] = v;
-      }
+      for (int mt = 0; mt < MT; ++mt) r.x[mt][c] = *(const uintx4*)(xrow[mt] + at);
     }
   };
-  auto multiply = [&](const StepRegs<MT, NW>& r) {
+  auto multiply = [&](const StepRegs<MT, NW>& r, int step) {
+    const bool reaches_beyond = (step + 1) * KSTEP > K;      // the same for the whole wave
 #pragma unroll
     for (int c = 0; c < 4; ++c)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8 a = __builtin_bit_cast(bf16x8, r.x[mt][c]);
+        uintx4 xv = r.x[mt][c];
+        if (reaches_beyond && step * KSTEP + lq * 8 + c * 32 >= K) xv = uintx4{0u, 0u, 0u, 0u};
+        const bf16x8 a = __builtin_bit_cast(bf16x8, xv);
 #pragma unroll
         for (int t = 0; t < NW; ++t)
           acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, r.w[t][c]), acc[mt][t], 0, 0, 0);
@@ -117,18 +116,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
   const int all_steps = (K + KSTEP - 1) / KSTEP;
   const int first_step = blockIdx.y * steps_per_split;
   const int steps = min(all_steps, first_step + steps_per_split);
+  // The product of a step is written out in both arms of each branch, so that the wait before it
+  // is the arm's own: behind a common join it would be a wait for every load in flight.
   StepRegs<MT, NW> ra, rb;
   int step = first_step + wave;
-  if (step < steps) load(ra, step);
-  while (step < steps) {
-    const int next = step + WAVES;
-    if (next < steps) load(rb, next);
-    multiply(ra);
-    if (next >= steps) break;
-    const int after = next + WAVES;
-    if (after < steps) load(ra, after);
-    multiply(rb);
-    step = after;
+  if (step < steps) {
+    load(ra, step);
+    while (true) {
+      const int next = step + WAVES;
+      if (next >= steps) { multiply(ra, step); break; }
+      load(rb, next);
+      multiply(ra, step);
+      const int after = next + WAVES;
+      if (after >= steps) { multiply(rb, next); break; }
+      load(ra, after);
+      multiply(rb, next);
+      step = after;
+    }
   }
 
   // the waves' partial sums meet in LDS, one (m tile, n tile) at a time, and are added in wave order
