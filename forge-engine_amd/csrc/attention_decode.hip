@@ -91,9 +91,11 @@ struct Prepare {
   int num_sums;
   long long sum_stride;
 };
-#define MAX_SUMS 8
+#define MAX_SUMS 4
 
-template <int D, bool PREPARE>
+// MODE 0: finished queries; 1: PREPARE from the projection's bfloat16 output; 2: PREPARE from its
+// float32 partial sums.
+template <int D, int MODE>
 __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* key_pages,
     const bf16_t* value_pages, bf16_t* __restrict__ out, long long out_stride,
@@ -101,6 +103,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     const int* __restrict__ ctx_len, const int* __restrict__ block_table, int table_stride,
     int kv_heads, int groups, int block_shift, int num_blocks, int window, float scale_log2,
     Prepare prep) {
+  constexpr bool PREPARE = MODE != 0, FROM_SUMS = MODE == 2;
   const int block_size = 1 << block_shift, block_mask = block_size - 1;
   constexpr int KC = D / 32;        // MFMA k-steps over the head dim (scores)
   constexpr int DT = D / 16;        // 16-dim tiles of the output
@@ -125,49 +128,40 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   const int lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 15, lq = lane >> 4;
 
-  // The rotation's cosines and sines of this token, once per block.
+  // Everything that depends on nothing but the sequence's length is requested before any of it
+  // is used, every load unconditional (out-of-range indices read a valid address and the value is
+  // dropped): the rotation's frequency of this thread, the projection's output (or its partial
+  // sums) for this block's heads, and the page ids of the wave's first two blocks of keys.  A
+  // load under a condition would become a branch, and where branches meet the compiler waits for
+  // every load in flight.
   __shared__ float cos_s[PREPARE ? D / 2 : 1], sin_s[PREPARE ? D / 2 : 1];
-  if (PREPARE && tid < D / 2) {
-    float sn, cs;
-    sincosf((float)(ctx - 1) * prep.inv_freq[tid], &sn, &cs);
-    cos_s[tid] = cs;
-    sin_s[tid] = sn;
-  }
+  __shared__ __attribute__((aligned(16))) bf16_t raw_s[FROM_SUMS ? (GMAX + 2) * D : 8];
+  float frequency = 0.f;
+  if constexpr (PREPARE) frequency = prep.inv_freq[min(tid, D / 2 - 1)];
 
-  // From partial sums: this block's query heads, key head and value head are added up once,
-  // rounded to bfloat16 and kept in LDS (all parts' loads in flight together).
-  __shared__ __attribute__((aligned(16))) bf16_t raw_s[PREPARE ? (GMAX + 2) * D : 8];
-  const bool from_sums = PREPARE && prep.num_sums > 0;
-  if (from_sums) {
-    for (int piece = tid; piece < (groups + 2) * (D / 4); piece += 256) {
+  // partial sums: pieces of four elements of this block's query heads, key head and value head
+  constexpr int PIECE_ROUNDS = FROM_SUMS ? ((GMAX + 2) * (D / 4) + 255) / 256 : 1;
+  float4 part[PIECE_ROUNDS][MAX_SUMS];
+  if constexpr (FROM_SUMS) {
+#pragma unroll
+    for (int round = 0; round < PIECE_ROUNDS; ++round) {
+      const int piece = min(tid + round * 256, (groups + 2) * (D / 4) - 1);
       const int head = piece / (D / 4), d = (piece - head * (D / 4)) * 4;
       const int column_head = head < groups ? hk * groups + head
                                             : kv_heads * groups + (head - groups) * kv_heads + hk;
       const float* src = prep.sums + (size_t)q0 * q_stride + (size_t)column_head * D + d;
-      float4 part[MAX_SUMS];
 #pragma unroll
-      for (int i = 0; i < MAX_SUMS; ++i) part[i] = *(const float4*)(src + (size_t)min(i, prep.num_sums - 1) * prep.sum_stride);
-      float4 sum = part[0];
-#pragma unroll
-      for (int i = 1; i < MAX_SUMS; ++i)
-        if (i < prep.num_sums) { sum.x += part[i].x; sum.y += part[i].y; sum.z += part[i].z; sum.w += part[i].w; }
-      uint2 packed;
-      packed.x = (uint32_t)float_to_bf16(sum.x) | ((uint32_t)float_to_bf16(sum.y) << 16);
-      packed.y = (uint32_t)float_to_bf16(sum.z) | ((uint32_t)float_to_bf16(sum.w) << 16);
-      *(uint2*)&raw_s[head * D + d] = packed;
+      for (int i = 0; i < MAX_SUMS; ++i) part[round][i] = *(const float4*)(src + (size_t)min(i, prep.num_sums - 1) * prep.sum_stride);
     }
   }
 
-  // query rows as the B operand: lane (lr = row g, lq) holds q[g][32c + 8lq .. +8]
+  // query rows as the B operand: lane (lr = row g, lq) holds q[g][32c + 8lq .. +8]; rows beyond
+  // the group read row 0 again, their scores and outputs are never stored
   bf16x8 qb[KC];
-  {
+  if constexpr (!FROM_SUMS) {
     const bf16_t* qrow = q + (size_t)q0 * q_stride + (size_t)(hk * groups + (lr < groups ? lr : 0)) * D;
 #pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      uintx4 v = uintx4{0u, 0u, 0u, 0u};
-      if (lr < groups && !from_sums) v = *(const uintx4*)(qrow + c * 32 + lq * 8);
-      qb[c] = __builtin_bit_cast(bf16x8, v);
-    }
+    for (int c = 0; c < KC; ++c) qb[c] = *(const bf16x8*)(qrow + c * 32 + lq * 8);
   }
 
   float m_run = -INFINITY, l_run = 0.f;   // of query row lr (the same in the four lanes that share it)
@@ -267,20 +261,45 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
 
   uintx4 k0[2][KC], k1[2][KC];
   const int b0 = my_first + wave;
-  int v0 = 0, v1 = 0, kr0 = 0, kr1 = 0;      // raw page ids: values of this / the next block, keys of the next two
-  if (b0 < my_last) {
-    v0 = raw_page(b0 * KEYS + 8 * lq);
-    fetch_keys(b0, checked(raw_page(b0 * KEYS + krow), b0 * KEYS + krow), k0);
-    kr1 = raw_page((b0 + WAVES) * KEYS + krow);
-    v1 = raw_page((b0 + WAVES) * KEYS + 8 * lq);
+  // raw page ids: values of this / the next block, keys of the next two (valid addresses whatever b0 is)
+  int v0 = raw_page(b0 * KEYS + 8 * lq);
+  const int kraw0 = raw_page(b0 * KEYS + krow);
+  int kr1 = raw_page((b0 + WAVES) * KEYS + krow);
+  int v1 = raw_page((b0 + WAVES) * KEYS + 8 * lq);
+  int kr0 = 0;
+  fetch_keys(b0, checked(kraw0, b0 * KEYS + krow), k0);
+
+  // What the requests above brought, while the keys are on their way: the rotation's cosines and
+  // sines of this token once per block, and the projection's output added up and rounded.
+  if constexpr (PREPARE) {
+    if (tid < D / 2) {
+      float sn, cs;
+      sincosf((float)(ctx - 1) * frequency, &sn, &cs);
+      cos_s[tid] = cs;
+      sin_s[tid] = sn;
+    }
+  }
+  if constexpr (FROM_SUMS) {
+#pragma unroll
+    for (int round = 0; round < PIECE_ROUNDS; ++round) {
+      const int piece = tid + round * 256;
+      float4 sum = part[round][0];
+#pragma unroll
+      for (int i = 1; i < MAX_SUMS; ++i)
+        if (i < prep.num_sums) { sum.x += part[round][i].x; sum.y += part[round][i].y; sum.z += part[round][i].z; sum.w += part[round][i].w; }
+      uint2 packed;
+      packed.x = (uint32_t)float_to_bf16(sum.x) | ((uint32_t)float_to_bf16(sum.y) << 16);
+      packed.y = (uint32_t)float_to_bf16(sum.z) | ((uint32_t)float_to_bf16(sum.w) << 16);
+      if (piece < (groups + 2) * (D / 4)) *(uint2*)&raw_s[piece * 4] = packed;
+    }
   }
 
   bool extra = false;       // this block also brings the new token's own key and value
   if constexpr (PREPARE) {
     __syncthreads();        // cos_s, sin_s, raw_s
-    if (from_sums && lr < groups) {
+    if constexpr (FROM_SUMS) {
 #pragma unroll
-      for (int c = 0; c < KC; ++c) qb[c] = *(const bf16x8*)&raw_s[lr * D + c * 32 + lq * 8];
+      for (int c = 0; c < KC; ++c) qb[c] = *(const bf16x8*)&raw_s[(lr < groups ? lr : 0) * D + c * 32 + lq * 8];
     }
     // Queries: chunk 4c + lq of head row lr sits in qb[c].  Norm, rotation and rounding as the
     // stand-alone kernel does them: the butterfly over chunks runs over c first, then over lq.
@@ -344,8 +363,9 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
       const int pos = ctx - 1;
       const bf16_t* row = q + (size_t)q0 * q_stride;
       const size_t k_at = (size_t)(kv_heads * groups + hk) * D, v_at = k_at + (size_t)kv_heads * D;
-      const uint4 raw = from_sums ? *(const uint4*)&raw_s[(groups + (role == 1 ? 1 : 0)) * D + sub * 8]
-                                  : *(const uint4*)(row + (role == 1 ? v_at : k_at) + sub * 8);
+      uint4 raw;
+      if constexpr (FROM_SUMS) raw = *(const uint4*)&raw_s[(groups + (role == 1 ? 1 : 0)) * D + sub * 8];
+      else raw = *(const uint4*)(row + (role == 1 ? v_at : k_at) + sub * 8);
       const int block = table[min(pos >> block_shift, table_last)];
       const bool writable = block >= 0 && block < num_blocks;     // the host reserves pages before the launch
       const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -525,18 +545,22 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
   dim3 grid(splits, kv_heads, num_seqs);
   const float scale_log2 = scale * 1.4426950408889634f;
   const Prepare none = {nullptr, nullptr, nullptr, 0.f, nullptr, 0, 0};
-#define FE_GO(DD, PP)                                                                                      \
-  paged_decode_kernel<DD, PP><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+#define FE_GO(DD, MODE)                                                                                    \
+  paged_decode_kernel<DD, MODE><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, part_o, part_ml, counters, cu_q, ctx_len, block_table,     \
-      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, PP ? *prep : none)
-  if (prep) {
-    if (head_dim == 64) FE_GO(64, true);
-    else if (head_dim == 128) FE_GO(128, true);
-    else FE_GO(256, true);
+      table_stride, kv_heads, groups, block_shift, num_blocks, window, scale_log2, MODE ? *prep : none)
+  if (prep && prep->num_sums > 0) {
+    if (head_dim == 64) FE_GO(64, 2);
+    else if (head_dim == 128) FE_GO(128, 2);
+    else FE_GO(256, 2);
+  } else if (prep) {
+    if (head_dim == 64) FE_GO(64, 1);
+    else if (head_dim == 128) FE_GO(128, 1);
+    else FE_GO(256, 1);
   } else {
-    if (head_dim == 64) FE_GO(64, false);
-    else if (head_dim == 128) FE_GO(128, false);
-    else FE_GO(256, false);
+    if (head_dim == 64) FE_GO(64, 0);
+    else if (head_dim == 128) FE_GO(128, 0);
+    else FE_GO(256, 0);
   }
 #undef FE_GO
   return fe_check_launch();
@@ -565,7 +589,7 @@ extern "C" int fe_paged_attention_decode(const void* q, long long q_stride, cons
 // stride q_stride]: q and k heads are normalised (weights [head_dim] float32, null: no norm)
 // and rotated whole by position ctx_len - 1 (inv_freq [head_dim / 2]), and each sequence's new
 // key and value are written to slot ctx_len - 1 of its pages.  qkv itself is not changed.
-// qkv_sums > 0 (at most 8): qkv is float32 and holds that many partial sums of the projection,
+// qkv_sums > 0 (at most 4): qkv is float32 and holds that many partial sums of the projection,
 // sum_stride floats apart, each [num_seqs rows, row stride q_stride]; they are added up in order
 // and rounded to bfloat16 first.
 extern "C" int fe_paged_attention_decode_prepare(const void* qkv, int qkv_sums, long long sum_stride,

@@ -262,10 +262,10 @@ MID_ROWS = 64
 MID_TARGET_BLOCKS = 240
 
 
-def _mid_parts(steps: int, blocks: int) -> int:
+def _mid_parts(steps: int, blocks: int, most: int = 16) -> int:
     """Parts of K for the 17-64-row product: about MID_TARGET_BLOCKS blocks in all, at least four
     128-steps a part (the kernel fetches two steps ahead), no part without steps."""
-    parts = max(1, min(16, MID_TARGET_BLOCKS // blocks, steps // 4))
+    parts = max(1, min(most, MID_TARGET_BLOCKS // blocks, steps // 4))
     return -(-steps // -(-steps // parts))
 
 
@@ -315,7 +315,7 @@ IN_PARTS_FEW_ROWS = 2
 
 
 def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
-    """x @ weight^T as float32 partial sums [parts <= 8, M, N] over parts of K, for a consumer that
+    """x @ weight^T as float32 partial sums [parts <= 4, M, N] over parts of K, for a consumer that
     adds them up itself (the decode attention kernel that prepares its own queries and keys);
     None where the plain product is the better choice or the sizes do not fit."""
     _gpu(x, "x")
@@ -326,7 +326,7 @@ def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
     if _skinny_fits(x, weight):
         return gemm_skinny(x, weight, "f32", tiles=1, waves=4, splits=IN_PARTS_FEW_ROWS)
     if _mid_fits(x, weight):
-        return gemm_mid_parts(x, weight, _mid_parts(steps, -(-weight.shape[0] // 64)))
+        return gemm_mid_parts(x, weight, _mid_parts(steps, -(-weight.shape[0] // 64), most=4))
     return None
 
 
@@ -518,14 +518,14 @@ def decode_attention_prepare(qkv: Tensor, q_weight: Tensor | None, k_weight: Ten
     output in one launch: what ``qk_norm_rope_write`` followed by ``paged_attention`` does for
     such a batch (same bits in the cache; qkv is left as it is).
 
-    qkv [B, (Hq + 2 Hkv) D] bfloat16, one row per sequence, or float32 [parts <= 8, B, ...]:
+    qkv [B, (Hq + 2 Hkv) D] bfloat16, one row per sequence, or float32 [parts <= 4, B, ...]:
     partial sums of the projection (``linear_in_parts``), added up in order and rounded to
     bfloat16 inside the kernel.  ctx_len counts the new token, whose position is ctx_len - 1."""
     width = (q_heads + 2 * kv_heads) * head_dim
     if isinstance(qkv, Tensor) and qkv.dtype == torch.float32:
         _gpu(qkv, "qkv", torch.float32)
-        if qkv.dim() != 3 or not 1 <= qkv.shape[0] <= 8 or qkv.shape[2] != width:
-            raise KernelError(f"qkv in parts must be [parts <= 8, B, {width}], got {tuple(qkv.shape)}")
+        if qkv.dim() != 3 or not 1 <= qkv.shape[0] <= 4 or qkv.shape[2] != width:
+            raise KernelError(f"qkv in parts must be [parts <= 4, B, {width}], got {tuple(qkv.shape)}")
         sums, num_seqs = qkv.shape[0], qkv.shape[1]
     else:
         _gpu(qkv, "qkv", torch.bfloat16)

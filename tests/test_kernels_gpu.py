@@ -644,7 +644,7 @@ def test_decode_attention_that_prepares_its_queries_and_keys(ops, q_heads, kv_he
     assert torch.equal(vp_one.cpu(), vp_ref)
 
 
-@pytest.mark.parametrize("parts", [1, 2, 5, 8])
+@pytest.mark.parametrize("parts", [1, 2, 3, 4])
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [(32, 8, 128, 16), (5, 5, 64, 32), (8, 1, 256, 16)])
 def test_decode_attention_that_prepares_from_partial_sums(ops, q_heads, kv_heads, head_dim, block_size, parts):
     """The projection's output as float32 partial sums: added up in order and rounded to bfloat16
@@ -673,7 +673,7 @@ def test_decode_attention_that_prepares_from_partial_sums(ops, q_heads, kv_heads
     for a, b in zip(*results):
         assert torch.equal(a, b)
     with pytest.raises(ops.KernelError):
-        ops.decode_attention_prepare(rand(g, 9, n, qkv.shape[1]).to(DEV), qw.to(DEV), kw.to(DEV), inv_freq.to(DEV), kp.to(DEV),
+        ops.decode_attention_prepare(rand(g, 5, n, qkv.shape[1]).to(DEV), qw.to(DEV), kw.to(DEV), inv_freq.to(DEV), kp.to(DEV),
                                      vp.to(DEV), torch.empty(n, q_heads * head_dim, dtype=torch.bfloat16, device=DEV), cu.to(DEV),
                                      ctx.to(DEV), table.to(DEV), eps=1e-6, scale=1.0, **sizes)
 
@@ -684,7 +684,7 @@ def test_linear_in_parts(ops):
     for rows in (1, 8, 16, 17, 64):
         x = rand(g, rows, 2560, dtype=torch.bfloat16).to(DEV)
         sums = ops.linear_in_parts(x, w)
-        assert sums.dtype == torch.float32 and sums.dim() == 3 and sums.shape[0] <= 8 and sums.shape[1:] == (rows, 6144)
+        assert sums.dtype == torch.float32 and sums.dim() == 3 and sums.shape[0] <= 4 and sums.shape[1:] == (rows, 6144)
         torch.testing.assert_close(sums.sum(0).cpu(), x.cpu().float() @ w.cpu().float().T, atol=2e-3, rtol=2e-3)
     assert ops.linear_in_parts(rand(g, 65, 2560, dtype=torch.bfloat16).to(DEV), w) is None       # many rows: the library
     assert ops.linear_in_parts(rand(g, 4, 256, dtype=torch.bfloat16).to(DEV), w[:, :256]) is None  # a short K
