@@ -104,14 +104,16 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_regs_kernel(
   const int s = rows ? rows[r] : r;
   float* hrow = h + (size_t)s * hidden;
   const TD* drow = delta ? delta + (size_t)s * hidden : nullptr;
-  float4 v[VEC];
+  float4 v[VEC], ww[VEC];      // the norm's weight is requested with the row, not after the sum
   float sumsq = 0.f;
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     const int i = (threadIdx.x + j * THREADS) * 4;
     v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    ww[j] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (i < hidden) {
       v[j] = load4_as_float(hrow + i);
+      ww[j] = *(const float4*)(w + i);
       if (drow) {
         float4 d = load4_as_float(drow + i);
         for (int k = 1; k < parts; k += 8) {     // eight parts' loads fly together; added in order
@@ -135,11 +137,9 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_regs_kernel(
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     const int i = (threadIdx.x + j * THREADS) * 4;
-    if (i < hidden) {
-      const float4 ww = *(const float4*)(w + i);
-      store4_from_float(orow + i, make_float4(v[j].x * inv * ww.x, v[j].y * inv * ww.y,
-                                              v[j].z * inv * ww.z, v[j].w * inv * ww.w));
-    }
+    if (i < hidden)
+      store4_from_float(orow + i, make_float4(v[j].x * inv * ww[j].x, v[j].y * inv * ww[j].y,
+                                              v[j].z * inv * ww[j].z, v[j].w * inv * ww[j].w));
   }
 }
 
