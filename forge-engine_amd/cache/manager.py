@@ -39,6 +39,8 @@ class RequestCache:
     length: int = 0                                   # tokens whose keys are in the cache
     tables: list[list[int]] = field(default_factory=list)   # per group: page id per logical block, NO_PAGE if given back
     first_block: list[int] = field(default_factory=list)    # per group: logical blocks below this were given back
+    lease: int = 0                                    # differs for every ``begin``: a request that ends and begins
+                                                      # again under its old name holds other pages
 
 
 def plan_groups(needs: list[CacheNeeds], schedule) -> tuple[list[CacheGroup], dict[int, tuple[int, int]]]:
@@ -82,6 +84,7 @@ class CacheManager:
         self.pools = [BlockAllocator(c) for c in capacities]
         self.slots = StateSlotPool(num_state_slots)
         self._requests: dict[str, RequestCache] = {}
+        self._leases = 0
 
     # ------------------------------------------------------------- queries
     def __contains__(self, request_id: str) -> bool:
@@ -123,8 +126,9 @@ class CacheManager:
     def begin(self, request_id: str) -> RequestCache:
         if request_id in self._requests:
             raise ValueError(f"request '{request_id}' already holds cache")
+        self._leases += 1
         entry = RequestCache(request_id, self.slots.lease(), 0,
-                             [[] for _ in self.groups], [0 for _ in self.groups])
+                             [[] for _ in self.groups], [0 for _ in self.groups], self._leases)
         self._requests[request_id] = entry
         return entry
 

@@ -28,7 +28,8 @@ class _DecodeGraph:
     """One captured decode step: fixed request count and block-table widths.
     The step's metadata lives in a static buffer (laid out as ``build_batch``
     lays out a batch of single tokens) that each replay refills; block-table
-    rows are rewritten only when a request's table changed."""
+    rows are rewritten only when a request's table changed (a request that ended and began again
+    under the same name holds another lease and other pages)."""
 
     def __init__(self, num_seqs: int, widths, device) -> None:
         n = num_seqs
@@ -66,7 +67,7 @@ class _DecodeGraph:
             keys, base = self.row_keys[g], self.table_at[g]
             for i, record in enumerate(records):
                 table = record.tables[g]
-                key = (record.request_id, len(table), record.first_block[g])
+                key = (record.lease, len(table), record.first_block[g])   # pages are only ever appended or given back from the front
                 if keys[i] != key:
                     row = buf[base + i * width:base + (i + 1) * width]
                     row[:len(table)] = table

@@ -879,3 +879,41 @@ def test_layers_of_the_large_model_against_the_plain_implementation(dtype, wide_
             if rid == request_id:
                 want[(rid, position)] = logits[position]
     ru.compare(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_name_used_again_decodes_from_its_new_pages(dtype, folders):
+    """A request ends and another begins under the same name with a table of the same length
+    but other pages (a third request took the old ones meanwhile): the captured decode step
+    must read the new table, not the row it kept for the name."""
+    name = "C"
+    config, weights = TINY[name], folder_weights(folders[name])
+    requests = ru.make_requests(config, 61, (20, 20, 21))
+    first, other, second = requests["r0"], requests["r1"], requests["r2"]
+    _, model = load_model(folders[name], dtype=dtype, device=DEV)
+    runner = ModelRunner(model, block_size=16, block_capacity=12, num_state_slots=4)
+
+    def decode(request_id, tokens, start):
+        rows = []
+        for position in range(start, len(tokens)):
+            rows.append(runner.step([StepEntry(request_id, [tokens[position]], [0])])[0].cpu().clone())
+        return torch.stack(rows)
+
+    runner.begin("a")
+    runner.step([StepEntry("a", first[:17], [])])
+    got_first = decode("a", first, 17)                  # captured here, with the table of the first lease
+    pages_before = [list(t) for t in runner.cache.request("a").tables]
+    runner.end("a")
+    runner.begin("other")
+    runner.step([StepEntry("other", other, [])])        # takes the pages that were given back
+    runner.begin("a")
+    runner.step([StepEntry("a", second[:17], [])])
+    assert [list(t) for t in runner.cache.request("a").tables] != pages_before
+    replays = runner.graph_replays
+    got_second = decode("a", second, 17)
+    assert runner.graph_replays == replays + len(second) - 17
+    for got, tokens in ((got_first, first), (got_second, second)):
+        want = plain.forward(weights, config, tokens)[17:]
+        scale = float(want.abs().max())
+        bound = 1e-4 * scale if dtype == "float32" else ru.BF16_FRACTION * scale
+        assert float((got - want).abs().max()) <= bound
