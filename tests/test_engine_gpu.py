@@ -843,7 +843,7 @@ def test_layers_of_the_large_model_against_the_plain_implementation(dtype, wide_
     folder, config, weights = wide_folder
     _, model = load_model(folder, dtype=dtype, device=DEV)
     requests = ru.make_requests(config, 41, (150, 97, 40, 43, 46, 49, 52, 55, 58, 61))
-    runner = ModelRunner(model, block_size=16, block_capacity=80, num_state_slots=12)
+    runner = ModelRunner(model, block_size=16, block_capacity=80, num_state_slots=20)
     got, want = {}, {}
 
     def keep(request_id, positions, logits):
@@ -872,6 +872,19 @@ def test_layers_of_the_large_model_against_the_plain_implementation(dtype, wide_
             got[(k, len(requests[k]) - 5 + step)] = row.clone()
     assert runner.graph_replays >= 5 + 12
     for k in group:
+        runner.end(k)
+    # eighteen together (more than 16 rows: the products for 17 to 64 rows), three steps
+    many = ru.make_requests(config, 43, tuple(range(8, 26)))
+    many = {f"m{i}": tokens for i, tokens in enumerate(many.values())}
+    requests = {**requests, **many}
+    for k, tokens in many.items():
+        runner.begin(k)
+        runner.step([StepEntry(k, tokens[:-3], [])])
+    for step in range(3):
+        logits = runner.step([StepEntry(k, [tokens[len(tokens) - 3 + step]], [0]) for k, tokens in many.items()])
+        for row, (k, tokens) in zip(logits.cpu(), many.items()):
+            got[(k, len(tokens) - 3 + step)] = row.clone()
+    for k in many:
         runner.end(k)
     for request_id, tokens in requests.items():
         logits = plain.forward(weights, config, tokens)
