@@ -243,13 +243,13 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
 
 
 # Measured on MI355X: a weight with few row tiles and a long K (the output and down projections: 160
-# tiles, K = 4096 and 9728) leaves CUs idle; parts of K of at least four 128-steps each, of equal
-# length and few enough that all blocks are resident at once, summed by blocks of four waves, take
-# 7.0 instead of 9.5 us and 13.9 instead of 18.4 us at 8 rows.  The consumer (add_rmsnorm, add_rows)
-# adds the parts in order.
+# tiles, K = 4096 and 9728) leaves CUs idle; parts of K of about twelve 128-steps each (three and
+# six parts), of equal length, summed by blocks of four waves, take 6.9 instead of 9.0 us and 13.1
+# instead of 18.4 us at 8 rows.  The consumer (add_rmsnorm, add_rows) adds the parts in order; more
+# parts make the product no faster and the norm slower (3.1 us behind three parts, 3.8 behind eight).
 UPDATE_SPLIT_MAX_TILES = 256
 UPDATE_SPLIT_MIN_STEPS = 32
-UPDATE_SPLIT_STEPS = 4
+UPDATE_SPLIT_STEPS = 12        # 128-steps a part: fewer, longer parts cost the product little and save the norm reads
 UPDATE_SPLIT_MAX = 16
 UPDATE_SPLIT_BLOCKS = 1536     # blocks of four waves aimed at: all resident at once, parts of equal length
 
@@ -298,7 +298,8 @@ def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tens
             and -(-weight.shape[0] // 16) <= UPDATE_SPLIT_MAX_TILES
             and -(-weight.shape[1] // 128) >= UPDATE_SPLIT_MIN_STEPS):
         steps, tiles = -(-weight.shape[1] // 128), -(-weight.shape[0] // 16)
-        splits = max(1, min(UPDATE_SPLIT_MAX, steps // UPDATE_SPLIT_STEPS, UPDATE_SPLIT_BLOCKS // tiles))
+        splits = max(1, min(UPDATE_SPLIT_MAX, (steps + UPDATE_SPLIT_STEPS // 2) // UPDATE_SPLIT_STEPS,
+                            UPDATE_SPLIT_BLOCKS // tiles))
         splits = -(-steps // -(-steps // splits))        # parts of equal length, none empty
         return gemm_skinny(x, weight, "f32", tiles=1, waves=4, splits=splits)
     if plain_bf16 and x.shape[0] > SKINNY_MAX_ROWS and _mid_fits(x, weight):
