@@ -137,7 +137,22 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   __shared__ float cos_s[PREPARE ? D / 2 : 1], sin_s[PREPARE ? D / 2 : 1];
   __shared__ __attribute__((aligned(16))) bf16_t raw_s[FROM_SUMS ? (GMAX + 2) * D : 8];
   float frequency = 0.f;
-  if constexpr (PREPARE) frequency = prep.inv_freq[min(tid, D / 2 - 1)];
+  // the norms' weights of this lane's elements too (without a norm: any valid address, not used):
+  // asked for after the keys they would be answered after the keys, and the queries' preparation
+  // would wait for both
+  float4 q_w[PREPARE ? KC : 1][2], k_w[2];
+  if constexpr (PREPARE) {
+    frequency = prep.inv_freq[min(tid, D / 2 - 1)];
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const float* at = prep.q_weight ? prep.q_weight + c * 32 + lq * 8 : prep.inv_freq;
+      q_w[c][0] = *(const float4*)at;
+      q_w[c][1] = *(const float4*)(at + 4);
+    }
+    const float* at = prep.k_weight ? prep.k_weight + (lane & (D / 8 - 1)) * 8 : prep.inv_freq;
+    k_w[0] = *(const float4*)at;
+    k_w[1] = *(const float4*)(at + 4);
+  }
 
   // partial sums: pieces of four elements of this block's query heads, key head and value head
   constexpr int PIECE_ROUNDS = FROM_SUMS ? ((GMAX + 2) * (D / 4) + 255) / 256 : 1;
@@ -296,7 +311,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
 
   bool extra = false;       // this block also brings the new token's own key and value
   if constexpr (PREPARE) {
-    __syncthreads();        // cos_s, sin_s, raw_s
+    __syncthreads();        // cos_s, sin_s, raw_s (the keys requested above stay in flight)
     if constexpr (FROM_SUMS) {
 #pragma unroll
       for (int c = 0; c < KC; ++c) qb[c] = *(const bf16x8*)&raw_s[(lr < groups ? lr : 0) * D + c * 32 + lq * 8];
@@ -328,8 +343,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
       const float inv = inverse_rms(sumsq, D, prep.eps);
 #pragma unroll
       for (int c = 0; c < KC; ++c) {
-        const float4 wa = *(const float4*)(prep.q_weight + c * 32 + lq * 8);
-        const float4 wb = *(const float4*)(prep.q_weight + c * 32 + lq * 8 + 4);
+        const float4 wa = q_w[c][0], wb = q_w[c][1];
         const float w8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
 #pragma unroll
         for (int e = 0; e < 8; ++e) qv[c][e] = normalise(qv[c][e], inv, w8[e]);
@@ -376,8 +390,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
 #pragma unroll
         for (int offset = LPH / 2; offset > 0; offset >>= 1) sumsq += __shfl_xor(sumsq, offset, FE_WAVE);
         const float inv = inverse_rms(sumsq, D, prep.eps);
-        const float4 wa = *(const float4*)(prep.k_weight + sub * 8);
-        const float4 wb = *(const float4*)(prep.k_weight + sub * 8 + 4);
+        const float4 wa = k_w[0], wb = k_w[1];
         const float w8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = normalise(v[e], inv, w8[e]);
