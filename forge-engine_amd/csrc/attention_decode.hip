@@ -53,29 +53,33 @@ __device__ __forceinline__ float load_agent(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// One output element from up to N splits: all loads first, then the sums in split order.
+// Two neighbouring output elements from up to N splits: all loads first (the pair of partial
+// outputs as one 8-byte load), then the sums in split order.
 template <int N>
-__device__ __forceinline__ bf16_t merge_few(const float* part_o, const float* part_ml, size_t first_part,
-                                            int splits, int groups, int g, int dim, int d) {
-  float m[N], l[N], o[N];
+__device__ __forceinline__ unsigned int merge_few(const float* part_o, const float* part_ml, size_t first_part,
+                                                  int splits, int groups, int g, int dim, int d) {
+  float m[N], l[N];
+  unsigned long long o[N];
 #pragma unroll
   for (int sp = 0; sp < N; ++sp) {
     const size_t row = (first_part + (sp < splits ? sp : 0)) * groups + g;
     m[sp] = load_agent(&part_ml[row * 2]);
     l[sp] = load_agent(&part_ml[row * 2 + 1]);
-    o[sp] = load_agent(&part_o[row * dim + d]);
+    o[sp] = __hip_atomic_load((const unsigned long long*)&part_o[row * dim + d], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   float m_tot = -INFINITY;
 #pragma unroll
   for (int sp = 0; sp < N; ++sp) m_tot = fmaxf(m_tot, sp < splits ? m[sp] : -INFINITY);
-  float l_tot = 0.f, ov = 0.f;
+  float l_tot = 0.f, ov0 = 0.f, ov1 = 0.f;
 #pragma unroll
   for (int sp = 0; sp < N; ++sp) {
     const float f = (sp < splits && m_tot > -INFINITY) ? __builtin_amdgcn_exp2f(m[sp] - m_tot) : 0.f;
     l_tot += f * l[sp];
-    ov += f * o[sp];
+    ov0 += f * __uint_as_float((unsigned int)o[sp]);
+    ov1 += f * __uint_as_float((unsigned int)(o[sp] >> 32));
   }
-  return float_to_bf16(ov * (l_tot > 0.f ? 1.f / l_tot : 0.f));
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  return (unsigned int)float_to_bf16(ov0 * inv) | ((unsigned int)float_to_bf16(ov1 * inv) << 16);
 }
 
 // What the PREPARE variant needs beyond the plain one: the norms' weights (null: no norm), the
@@ -510,9 +514,9 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
   if (splits <= 16) {
     // few splits: every thread reads the statistics of its row itself, together with its share
     // of the partial outputs, so that all loads are in flight at once (same sums, same order)
-    for (int e = tid; e < groups * D; e += 256) {
+    for (int e = 2 * tid; e < groups * D; e += 512) {
       const int g = e / D, d = e - g * D;
-      bf16_t* dst = out + (size_t)q0 * out_stride + (size_t)(hk * groups + g) * D + d;
+      unsigned int* dst = (unsigned int*)(out + (size_t)q0 * out_stride + (size_t)(hk * groups + g) * D + d);
       if (splits <= 4) *dst = merge_few<4>(part_o, part_ml, first_part, splits, groups, g, D, d);
       else if (splits <= 8) *dst = merge_few<8>(part_o, part_ml, first_part, splits, groups, g, D, d);
       else *dst = merge_few<16>(part_o, part_ml, first_part, splits, groups, g, D, d);
@@ -552,7 +556,8 @@ static int launch_decode(const void* q, long long q_stride, const void* key_page
   if (block_size < 16 || (block_size & (block_size - 1)) || num_blocks < 1 || table_stride < 1) return FE_BAD_ARGUMENT;
   int block_shift = 0;
   while ((1 << block_shift) < block_size) ++block_shift;
-  if (q_stride % 8 || splits < 1 || splits > 64) return FE_BAD_ARGUMENT;
+  if (q_stride % 8 || out_stride % 2 || splits < 1 || splits > 64) return FE_BAD_ARGUMENT;
+  if ((((uintptr_t)out) & 3) || (((uintptr_t)part_o) & 7)) return FE_BAD_ARGUMENT;   // pairs of outputs, pairs of partial sums
   if ((((uintptr_t)q) | ((uintptr_t)key_pages) | ((uintptr_t)value_pages)) & 15) return FE_BAD_ARGUMENT;
   if (splits > 1 && (!part_o || !part_ml || !counters)) return FE_BAD_ARGUMENT;
   dim3 grid(splits, kv_heads, num_seqs);
