@@ -1,0 +1,43 @@
+"""Host-side choices of the kernel wrappers that need no GPU: how a product's K is cut into parts
+and how many key splits the decode attention takes."""
+
+from __future__ import annotations
+
+import pytest
+
+from forge_engine_amd.kernels import ops
+
+
+@pytest.mark.parametrize("steps", [1, 3, 4, 7, 20, 32, 76, 500])
+@pytest.mark.parametrize("blocks", [1, 3, 40, 96, 160, 1000])
+@pytest.mark.parametrize("most", [1, 4, 16])
+def test_parts_of_k_are_never_empty_and_respect_their_bounds(steps, blocks, most):
+    parts = ops._mid_parts(steps, blocks, most)
+    assert 1 <= parts <= most
+    per_part = -(-steps // parts)
+    assert (parts - 1) * per_part < steps          # the last part still has a step
+    assert parts == 1 or per_part >= 4 or steps < 8   # a part is at least four steps long
+
+
+def test_parts_of_k_for_the_large_model():
+    # Qwen3-4B: q/k/v (20 steps, 96 blocks of 64 rows), output (32, 40), down (76, 40)
+    assert ops._mid_parts(20, 96, most=4) == 2
+    assert ops._mid_parts(32, 40) == 6
+    assert ops._mid_parts(76, 40) == 6
+
+
+@pytest.mark.parametrize("num_decode,kv_heads,max_ctx,expect", [
+    (8, 8, 1040, 4), (1, 8, 2048, 16), (64, 8, 1040, 1), (1, 8, 64, 1), (1, 1, 100000, 64),
+])
+def test_key_splits_of_the_decode_attention(num_decode, kv_heads, max_ctx, expect):
+    assert ops.decode_splits(num_decode, kv_heads, max_ctx) == expect
+
+
+def test_the_fused_decode_attention_serves_what_it_says():
+    import torch
+    ok = dict(q_heads=32, kv_heads=8, head_dim=128, rotary_dim=128, block_size=16)
+    assert ops.decode_prepare_supported(torch.bfloat16, **ok)
+    assert not ops.decode_prepare_supported(torch.float32, **ok)
+    for change in (dict(head_dim=96, rotary_dim=96), dict(rotary_dim=64), dict(q_heads=80), dict(block_size=8),
+                   dict(block_size=48), dict(q_heads=30)):
+        assert not ops.decode_prepare_supported(torch.bfloat16, **{**ok, **change}), change
