@@ -32,10 +32,10 @@ class RMSNorm(Norm):
         self.weight = tensor
 
     def forward(self, residual: Residual, rows: Tensor | None = None) -> Tensor:
-        if rows is not None:
-            h = residual.flush()
+        if rows is not None:    # the chosen rows of stream + pending update; both are left as they are
+            h = residual.h
             out = torch.empty((rows.numel(), self.size), dtype=self.ctx.dtype, device=h.device)
-            return ops.add_rmsnorm(h, None, self.weight, self.eps, out, rows=rows, store_sum=False)
+            return ops.add_rmsnorm(h, residual.pending, self.weight, self.eps, out, rows=rows, store_sum=False)
         update, residual.pending = residual.pending, None
         out = torch.empty((residual.h.shape[0], self.size), dtype=self.ctx.dtype, device=residual.h.device)
         return ops.add_rmsnorm(residual.h, update, self.weight, self.eps, out)

@@ -82,6 +82,18 @@ def test_add_rmsnorm_row_list(ops):
     got = ops.add_rmsnorm(h.to(DEV), None, w.to(DEV), 1e-6, torch.empty(4, 96, device=DEV),
                           rows=rows.to(DEV), store_sum=False)
     torch.testing.assert_close(got.cpu(), want, atol=1e-5, rtol=1e-5)
+    # with an update that has not been added yet (whole, or in parts): the rows of the sum, and the
+    # stream is left as it is
+    for hidden, parts in ((96, 1), (2560, 1), (2560, 3), (200, 9)):
+        h = rand(g, 9, hidden)
+        w = rand(g, hidden)
+        delta = rand(g, parts, 9, hidden) if parts > 1 else rand(g, 9, hidden)
+        want = refs.add_rmsnorm(h.clone(), delta, w, 1e-6, torch.empty(4, hidden), rows=rows, store_sum=False)
+        h_dev = h.to(DEV)
+        got = ops.add_rmsnorm(h_dev, delta.to(DEV), w.to(DEV), 1e-6, torch.empty(4, hidden, device=DEV),
+                              rows=rows.to(DEV), store_sum=False)
+        torch.testing.assert_close(got.cpu(), want, atol=1e-5, rtol=1e-5)
+        assert torch.equal(h_dev.cpu(), h)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
