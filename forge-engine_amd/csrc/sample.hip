@@ -47,17 +47,32 @@ __global__ __launch_bounds__(256) void argmax_parts_kernel(
   __shared__ int flags_s[4];
   const int part = blockIdx.x, row_id = blockIdx.y;
   const float* row = logits + (size_t)row_id * row_stride;
-  const int per = (vocab + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
-  const int begin = part * per, end = min(vocab, begin + per);
+  const int per = ((vocab + ARGMAX_PARTS - 1) / ARGMAX_PARTS + 3) & ~3;     // a multiple of four: parts start aligned
+  const int begin = min(vocab, part * per), end = min(vocab, begin + per);
   float bv = -INFINITY;
   int bi = 0x7fffffff, flags = 0;   // bit 0 NaN, bit 1 +inf, bit 3 a finite entry was seen
-  for (int i = begin + threadIdx.x; i < end; i += 256) {
-    const float v = row[i];
+  auto take = [&](float v, int i) {
     if (v != v) flags |= 1;
     else if (v == INFINITY) flags |= 2;
     else if (v != -INFINITY) flags |= 8;
     argmax_merge(bv, bi, v, i);
+  };
+  int i = begin + threadIdx.x;
+  if ((((uintptr_t)row) & 15) == 0) {          // four at a time, two loads in flight, in index order
+    const int whole = begin + ((end - begin) & ~3);
+    int at = begin + 4 * threadIdx.x;
+    for (; at + 1024 < whole; at += 2048) {
+      const float4 a = *(const float4*)(row + at), b = *(const float4*)(row + at + 1024);
+      take(a.x, at); take(a.y, at + 1); take(a.z, at + 2); take(a.w, at + 3);
+      take(b.x, at + 1024); take(b.y, at + 1025); take(b.z, at + 1026); take(b.w, at + 1027);
+    }
+    if (at < whole) {
+      const float4 a = *(const float4*)(row + at);
+      take(a.x, at); take(a.y, at + 1); take(a.z, at + 2); take(a.w, at + 3);
+    }
+    i = whole + threadIdx.x;                    // what is left: fewer than four entries
   }
+  for (; i < end; i += 256) take(row[i], i);
 #pragma unroll
   for (int offset = FE_WAVE / 2; offset > 0; offset >>= 1) {
     argmax_merge(bv, bi, __shfl_xor(bv, offset, FE_WAVE), __shfl_xor(bi, offset, FE_WAVE));
