@@ -96,6 +96,11 @@ class CacheManager:
         except KeyError:
             raise KeyError(f"unknown request '{request_id}'") from None
 
+    def holds(self, entries: list[RequestCache]) -> bool:
+        """Whether every record is still the live one of its request (none ended since)."""
+        requests = self._requests
+        return all(requests.get(entry.request_id) is entry for entry in entries)
+
     def live_requests(self) -> list[str]:
         return list(self._requests)
 

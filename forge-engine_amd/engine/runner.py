@@ -75,6 +75,15 @@ class _DecodeGraph:
                     keys[i] = key
 
 
+class _SteadyDecode:
+    """What the last decode step left for the next one, if that brings the same requests again:
+    their records, the graph they replay, and how many more tokens fit into every request's last
+    page (no page to reserve, no table row to rewrite until then)."""
+
+    def __init__(self, ids, records, slot, room: int) -> None:
+        self.ids, self.records, self.slot, self.room = ids, records, slot, room
+
+
 class _PortionGraph:
     """One captured step that holds prompt portions (beside single tokens or not): fixed token
     count, sequence count and wanted-row count rounded up, block-table widths rounded up.
@@ -142,6 +151,7 @@ class ModelRunner:
         self.model = model
         self.use_graphs = use_graphs and model.ctx.device.type == "cuda" and model.graph_safe
         self._graphs: dict[tuple, _DecodeGraph] = {}
+        self._steady: _SteadyDecode | None = None
         self._portion_graphs: dict[tuple, _PortionGraph] = {}
         self._portion_seen: dict[tuple, int] = {}
         self.graph_replays = 0
@@ -237,12 +247,34 @@ class ModelRunner:
         time than the step takes on the GPU."""
         cache = self.cache
         vocab = self.model.plan.vocab_size
-        records = [cache.request(e.request_id) for e in entries]
-        if len({e.request_id for e in entries}) != len(entries):
-            raise ValueError("a request appears twice in one step")
         tokens = [e.tokens[0] for e in entries]
         if min(tokens) < 0 or max(tokens) >= vocab:
             raise ValueError(f"a token id is outside the vocabulary of {vocab}")
+        steady = self._steady
+        if (steady is not None and steady.room > 0 and len(entries) == len(steady.ids)
+                and all(e.request_id == name for e, name in zip(entries, steady.ids))
+                and cache.holds(steady.records)):
+            # the same requests as the last step, none ended since, every one with room in its last
+            # page: only the tokens change and every position moves on by one
+            slot, n = steady.slot, len(entries)
+            slot.copied.synchronize()
+            buf = slot.np
+            buf[0:n] = tokens
+            buf[n:2 * n] += 1                                # positions
+            buf[4 * n + 1:6 * n + 1] += 1                    # ctx_len, ctx_before
+            slot.dev.copy_(slot.host, non_blocking=True)
+            slot.copied.record(torch.cuda.current_stream(self.device))
+            slot.graph.replay()
+            for record in steady.records:
+                record.length += 1
+            steady.room -= 1
+            self.graph_replays += 1
+            self.steps_run += 1
+            return slot.logits
+        self._steady = None
+        records = [cache.request(e.request_id) for e in entries]
+        if len({e.request_id for e in entries}) != len(entries):
+            raise ValueError("a request appears twice in one step")
         before = [r.length for r in records]
         need = {r.request_id: b + 1 for r, b in zip(records, before)
                 if any(len(t) * self.block_size <= b for t in r.tables)}
@@ -281,6 +313,9 @@ class ModelRunner:
         self.graph_replays += 1
         cache.commit_single_tokens(records)
         self.steps_run += 1
+        if not any(group.window is not None for group in cache.groups):   # a window gives pages back as it moves
+            room = min(len(table) * self.block_size - record.length for record in records for table in record.tables)
+            self._steady = _SteadyDecode(tuple(e.request_id for e in entries), records, slot, room)
         return slot.logits
 
     def _portion_key(self, entries: list[StepEntry]):
@@ -356,6 +391,7 @@ class ModelRunner:
         the next step of the same shape overwrites."""
         if self._graphable(entries):
             return self._graph_step(entries)
+        self._steady = None        # any other step may move the requests that the last decode step left
         shape = self._portion_key(entries) if entries else None
         if shape is not None:
             logits = self._portion_graph_step(entries, shape)
