@@ -152,6 +152,7 @@ class ModelRunner:
         self.use_graphs = use_graphs and model.ctx.device.type == "cuda" and model.graph_safe
         self._graphs: dict[tuple, _DecodeGraph] = {}
         self._steady: _SteadyDecode | None = None
+        self.steady_steps = 0
         self._portion_graphs: dict[tuple, _PortionGraph] = {}
         self._portion_seen: dict[tuple, int] = {}
         self.graph_replays = 0
@@ -268,6 +269,7 @@ class ModelRunner:
             for record in steady.records:
                 record.length += 1
             steady.room -= 1
+            self.steady_steps += 1
             self.graph_replays += 1
             self.steps_run += 1
             return slot.logits

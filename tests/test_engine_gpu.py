@@ -150,6 +150,9 @@ def test_long_decoding_through_graphs_matches_eager_and_plain(dtype, folders):
                 fed_other += 9
         runs[graphs] = torch.stack(rows).cpu()
         assert (runner.graph_replays > 250) == graphs
+        # most replays take the short way (same request, room in its last page); a new page every 16
+        # tokens and the other request's steps make the step look again
+        assert (runner.steady_steps > 200) == graphs and (not graphs or runner.steady_steps < runner.graph_replays - 15)
         runner.end("a")
         runner.end("b")
         assert runner.cache.allocated_pages == 0
