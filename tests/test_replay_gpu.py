@@ -88,3 +88,39 @@ def test_trace_run_program(folders, tmp_path):
     assert done.stdout.split() == [w for s in trace.steps for w in ("done", str(s["step"]))]
     got = ru.collect(trace, out, TINY["A"]["vocab_size"])
     ru.compare(got, ru.plain_logits(folders["A"], requests), "float32")
+
+
+def _drawn_configuration(seed: int):
+    """A small configuration whose every size is drawn: head sizes from 16 to 256, any group
+    size, widths and vocabularies that are no power of two, bias or not, tied or not."""
+    import random
+    rng = random.Random(1000 + seed)
+    kv = rng.choice([1, 2, 3, 4])
+    groups = rng.choice([1, 2, 3, 4, 5, 7, 8, 9])
+    config = {
+        "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "hidden_act": "silu",
+        "vocab_size": rng.choice([97, 256, 300, 1003, 2049]), "hidden_size": rng.choice([40, 64, 72, 136, 200, 264]),
+        "intermediate_size": rng.choice([48, 128, 136, 328, 520]), "num_hidden_layers": rng.choice([1, 2, 3]),
+        "num_attention_heads": kv * groups, "num_key_value_heads": kv,
+        "head_dim": rng.choice([16, 32, 48, 64, 64, 80, 96, 128, 128, 160, 256]),
+        "max_position_embeddings": 512, "rms_norm_eps": rng.choice([1e-6, 1e-5, 1e-3]),
+        "rope_theta": rng.choice([10000.0, 1e6, 5e6]), "tie_word_embeddings": rng.choice([True, False]),
+        "attention_bias": rng.choice([False, False, True]), "eos_token_id": None,
+    }
+    block_size = rng.choice([4, 8, 16, 16, 32, 64])
+    lengths = tuple(rng.choice([1, 2, 3, 17, 33, 40, 64, 65, 100, 150]) for _ in range(rng.randrange(3, 6)))
+    return config, block_size, lengths
+
+
+@pytest.mark.parametrize("seed", [1, 6, 12, 13, 24, 47, 74])
+def test_replay_of_drawn_configurations(seed, tmp_path):
+    """Configurations nobody chose by hand, every way of cutting, both dtypes."""
+    config, block_size, lengths = _drawn_configuration(seed)
+    folder = tmp_path / "model"
+    write_random_model(load_model_config(config), 50 + seed, folder)
+    requests = ru.make_requests(config, seed, lengths)
+    want = ru.plain_logits(folder, requests)
+    for dtype in ("float32", "bfloat16"):
+        for mode, make in TRACES.items():
+            got = ru.run_trace(folder, dtype, make(requests), tmp_path / f"{dtype}_{mode}", block_size=block_size)
+            ru.compare(got, want, dtype)
