@@ -196,3 +196,91 @@ def test_sampling_filter_vectors():
     assert kept(plain.filter_logits(torch.tensor([[0.0, 3.0, 2.0, 1.0]]), 1.0, top_k=2)) == [1, 2]
     assert kept(plain.filter_logits(torch.tensor([[5.0, 4.0, 0.0]]), 1.0, top_p=0.7)) == [0]
     assert kept(plain.filter_logits(torch.tensor([[0.0, -1.0, -3.0]]), 1.0, min_p=0.2)) == [0, 1]
+
+
+def test_key_scale_is_removed_by_the_per_head_norm():
+    # k_norm sits between the k projection and the rotation (qwen3.py:146-150): scaling W_k
+    # leaves the logits unchanged (up to eps, which is why the configuration with the smaller
+    # eps is used); without k_norm every score would scale.
+    config = TINY["A"]
+    w = plain.random_weights(config, 12)
+    ids = [3, 200, 17, 17, 64, 9]
+    a = plain.forward(w, config, ids)
+    w2 = dict(w)
+    for i in range(config["num_hidden_layers"]):
+        name = f"model.layers.{i}.self_attn.k_proj.weight"
+        w2[name] = w[name] * 8.0
+    torch.testing.assert_close(plain.forward(w2, config, ids), a, atol=1e-5, rtol=1e-4)
+    # the control: the same scaling of W_v does change them (nothing normalises v)
+    w3 = dict(w)
+    for i in range(config["num_hidden_layers"]):
+        name = f"model.layers.{i}.self_attn.v_proj.weight"
+        w3[name] = w[name] * 8.0
+    assert (plain.forward(w3, config, ids) - a).abs().max() > 1e-3
+
+
+def test_values_are_not_normalised():
+    # v goes from its projection straight into the weighted sum (qwen3.py:151-155): with the
+    # feed-forward silenced, scaling W_v by c scales the layer's update of the stream by c.
+    config = dict(TINY["A"], num_hidden_layers=1)
+    w = plain.random_weights(config, 13)
+    w["model.layers.0.mlp.down_proj.weight"].zero_()
+    ids = torch.tensor([9, 8, 100, 7])
+    e = w["model.embed_tokens.weight"][ids]
+    _, hidden = plain.forward(w, config, ids, return_hidden=True)
+    update = hidden[0] - e
+    w2 = dict(w)
+    w2["model.layers.0.self_attn.v_proj.weight"] = w["model.layers.0.self_attn.v_proj.weight"] * 3.0
+    _, hidden2 = plain.forward(w2, config, ids, return_hidden=True)
+    assert update.abs().max() > 1e-4
+    torch.testing.assert_close(hidden2[0] - e, 3.0 * update, atol=1e-6, rtol=1e-5)
+
+
+def _hand_attention_weights(a: float, b: float) -> dict:
+    eye = torch.eye(4)
+    return {"p.q_proj.weight": eye.clone(), "p.k_proj.weight": eye.clone(), "p.v_proj.weight": eye.clone(),
+            "p.o_proj.weight": eye.clone(), "p.q_norm.weight": torch.full((4,), a),
+            "p.k_norm.weight": torch.full((4,), b)}
+
+
+def test_attention_block_by_hand_scale_norms_and_values():
+    # One head of size 4, identity projections, theta so large that dims 1 and 3 do not turn
+    # (dims 0 and 2 hold zeros).  Rows (0,3,0,4) and (0,4,0,-3) have RMS 2.5, so after the
+    # per-head norms q = a x / 2.5 and k = b x / 2.5: for the second token q1.k0 = 0 and
+    # q1.k1 = 4ab, and its scores are (0, 4ab * D^-0.5) = (0, 2ab)  (qwen3.py:129,189-190).
+    # The values are the rows themselves.  Scale 1.0, a missing k_norm or a normalised v
+    # each give another result.
+    a, b = 1.5, 0.5
+    config = {"num_attention_heads": 1, "num_key_value_heads": 1, "head_dim": 4, "rms_norm_eps": 1e-12,
+              "rope_theta": 1e30}
+    x = torch.tensor([[0.0, 3.0, 0.0, 4.0], [0.0, 4.0, 0.0, -3.0]])
+    out = plain.attention_block(x, _hand_attention_weights(a, b), "p", config, torch.arange(2))
+    p1 = math.exp(2 * a * b) / (1.0 + math.exp(2 * a * b))
+    torch.testing.assert_close(out[0], x[0])
+    torch.testing.assert_close(out[1], (1 - p1) * x[0] + p1 * x[1], atol=1e-6, rtol=1e-6)
+
+
+def test_attention_block_is_library_attention_with_its_default_scale():
+    # norms and rotation by hand, then the library's attention, whose default scale is
+    # 1/sqrt(head size): pins the block's own choice of scale, that both q and k are
+    # normalised and that v is not.
+    config = dict(TINY["B"])
+    heads, kv_heads, d = config["num_attention_heads"], config["num_key_value_heads"], config["head_dim"]
+    w = plain.random_weights(config, 14)
+    prefix = "model.layers.1.self_attn"
+    g = torch.Generator().manual_seed(15)
+    x = torch.randn(7, config["hidden_size"], generator=g)
+    q = (x @ w[f"{prefix}.q_proj.weight"].T).view(7, heads, d)
+    k = (x @ w[f"{prefix}.k_proj.weight"].T).view(7, kv_heads, d)
+    v = (x @ w[f"{prefix}.v_proj.weight"].T).view(7, kv_heads, d)
+    q = F.rms_norm(q, (d,), w[f"{prefix}.q_norm.weight"], config["rms_norm_eps"]).transpose(0, 1)
+    k = F.rms_norm(k, (d,), w[f"{prefix}.k_norm.weight"], config["rms_norm_eps"]).transpose(0, 1)
+    cos, sin = plain.rotary_tables(torch.arange(7), d, config["rope_theta"])
+    q, k = plain.apply_rotary(q, cos, sin), plain.apply_rotary(k, cos, sin)
+    groups = heads // kv_heads
+    want = F.scaled_dot_product_attention(
+        q.unsqueeze(0), k.repeat_interleave(groups, 0).unsqueeze(0),
+        v.transpose(0, 1).repeat_interleave(groups, 0).unsqueeze(0), is_causal=True)[0]
+    want = want.transpose(0, 1).reshape(7, heads * d) @ w[f"{prefix}.o_proj.weight"].T
+    got = plain.attention_block(x, w, prefix, config, torch.arange(7))
+    torch.testing.assert_close(got, want, atol=1e-6, rtol=1e-5)
