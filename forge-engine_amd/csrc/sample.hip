@@ -4,6 +4,8 @@
 // (that is how filters remove tokens).  Each row also gets a status word:
 //   bit 0: a NaN was seen, bit 1: +inf was seen, bit 2: no finite entry.
 #include "common.h"
+#include "sample_api.h"
+#include <mutex>
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_WAVES (SAMPLE_THREADS / FE_WAVE)
@@ -221,6 +223,36 @@ extern "C" int fe_argmax_rows(const float* logits, long long row_stride, int row
   argmax_parts_kernel<<<grid, 256, 0, stream>>>(logits, row_stride, vocab, part_v, part_i, part_flags);
   argmax_merge_kernel<<<rows, 64, 0, stream>>>(part_v, part_i, part_flags, tokens, status);
   return fe_check_launch();
+}
+
+// The scratch of fe_argmax_rows_static.  In host code this name is only a handle for
+// hipGetSymbolAddress: each GPU holds its own copy at its own address, kept below per device.
+static __device__ __align__(256) int argmax_static_scratch[FE_ARGMAX_STATIC_MAX_ROWS * ARGMAX_PARTS * 3];
+
+#define FE_MAX_DEVICES 64
+static std::mutex static_scratch_lock;
+static void* static_scratch_of_device[FE_MAX_DEVICES];
+
+// The device address of the array on the current device (looked up at the first call there).
+static void* argmax_static_scratch_here() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= FE_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> hold(static_scratch_lock);
+  if (!static_scratch_of_device[device]) {
+    void* address = nullptr;
+    if (hipGetSymbolAddress(&address, HIP_SYMBOL(argmax_static_scratch)) != hipSuccess) return nullptr;
+    static_scratch_of_device[device] = address;
+  }
+  return static_scratch_of_device[device];
+}
+
+extern "C" int fe_argmax_rows_static(const float* logits, long long row_stride, int rows, int vocab,
+                                     int* tokens, int* status, hipStream_t stream) {
+  if (rows <= 0) return FE_OK;
+  if (rows > FE_ARGMAX_STATIC_MAX_ROWS) return FE_BAD_ARGUMENT;
+  void* scratch = argmax_static_scratch_here();
+  if (!scratch) return FE_LAUNCH_FAILED;
+  return fe_argmax_rows(logits, row_stride, rows, vocab, tokens, status, scratch, stream);
 }
 
 extern "C" int fe_sample_rows(const float* logits, long long row_stride, int rows, int vocab,

@@ -596,6 +596,25 @@ def argmax_rows(logits: Tensor, tokens: Tensor, status: Tensor) -> None:
           c_int(vocab), _ptr(tokens), _ptr(status), _ptr(scratch), _stream())
 
 
+ARGMAX_STATIC_MAX_ROWS = 1024   # FE_ARGMAX_STATIC_MAX_ROWS of csrc/sample_api.h
+
+
+def argmax_rows_static(logits: Tensor, tokens: Tensor, status: Tensor) -> None:
+    """``argmax_rows`` without any allocation: the partial maxima live in an array inside the
+    library's device image, shared by every call on the GPU (calls that overlap there race;
+    calls on one stream do not).  At most ``ARGMAX_STATIC_MAX_ROWS`` rows."""
+    _gpu(logits, "logits", torch.float32)
+    _gpu(tokens, "tokens", torch.int32)
+    _gpu(status, "status", torch.int32)
+    rows, vocab = logits.shape
+    if tokens.numel() != rows or status.numel() != rows:
+        raise KernelError("tokens and status need one entry per row")
+    if rows > ARGMAX_STATIC_MAX_ROWS:
+        raise KernelError(f"the arg-max without allocation takes at most {ARGMAX_STATIC_MAX_ROWS} rows, got {rows}")
+    _call("sample", "fe_argmax_rows_static", _ptr(logits), c_longlong(logits.stride(0)), c_int(rows),
+          c_int(vocab), _ptr(tokens), _ptr(status), _stream())
+
+
 def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index: Tensor,
                 tokens: Tensor, status: Tensor) -> None:
     """Draw tokens[r] from softmax(logits[r] / temperatures[r]) with the uniform
