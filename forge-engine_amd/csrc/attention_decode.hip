@@ -220,7 +220,15 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     // values (A operand of the second product): lane (lr = dim, lq) reads the 8 consecutive keys
     // 8lq .. 8lq+7 of dims 16t + lr from the transposed page
     const int vkey = b * KEYS + 8 * lq;
-    const bool v_ok = vkey < cached;
+    // Which of these eight keys lie inside [k_begin, cached): the values of the others are set
+    // to zero below.  Their probabilities are zero anyway, but a slot that no live key owns may
+    // hold anything (a NaN that an earlier request left there), and 0 * NaN is NaN.
+    const int v_hi = min(max(cached - vkey, 0), 8), v_lo = min(max(k_begin - vkey, 0), 8);
+    const unsigned int v_bits = ((1u << v_hi) - 1u) & ~((1u << v_lo) - 1u);
+    uintx4 v_mask;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      v_mask[i] = (((v_bits >> (2 * i)) & 1u) ? 0x0000ffffu : 0u) | (((v_bits >> (2 * i + 1)) & 1u) ? 0xffff0000u : 0u);
     const int vpage = checked(vraw, vkey);
     const bf16_t* vbase = value_pages + ((((size_t)vpage * kv_heads + hk) * D) << block_shift) + (vkey & block_mask);
     uintx4 va[DT];
@@ -273,7 +281,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
     for (int t = 0; t < DT; ++t) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[t][i] *= corr;
-      const uintx4 vt = v_ok ? va[t] : uintx4{0u, 0u, 0u, 0u};
+      const uintx4 vt = va[t] & v_mask;
       o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vt), pb, o[t], 0, 0, 0);
     }
   };

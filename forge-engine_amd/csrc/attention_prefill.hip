@@ -38,8 +38,10 @@
 // product.
 //
 // Keys at or beyond the context read the bytes of the last key instead (their
-// scores are masked; their probabilities are zero).  Pages must hold finite
-// values in every slot of a page in use (the engine's pages start as zeros).
+// scores are masked; their probabilities are zero).  In the tiles that hold keys
+// outside [first visible key, context) the values of those keys are set to zero
+// before the second product: a slot that no live key owns may hold anything (a
+// NaN that an earlier request left there), and 0 * NaN is NaN.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -250,13 +252,33 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
     FE_WAIT_VMEM(0);
     __syncthreads();             // the values (and the next keys) are in LDS
     if (mine) {
-#pragma unroll
-      for (int t = 0; t < DT; ++t)
+      if (key_base + BN > ctx || key_base < k_first) {     // a tile with keys that nobody owns (uniform over the block)
+        uintx4 v_mask[2];
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
-          const bf16x8 va = __builtin_bit_cast(bf16x8, Vs[(blk * 4 + lq) * D + t * 16 + lr]);
-          o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[blk], o[t], 0, 0, 0);
+          const int first_key = key_base + 32 * blk + 8 * lq;
+          const int hi = min(max(ctx - first_key, 0), 8), lo = min(max(k_first - first_key, 0), 8);
+          const unsigned int bits = ((1u << hi) - 1u) & ~((1u << lo) - 1u);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            v_mask[blk][i] = (((bits >> (2 * i)) & 1u) ? 0x0000ffffu : 0u) | (((bits >> (2 * i + 1)) & 1u) ? 0xffff0000u : 0u);
         }
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int blk = 0; blk < 2; ++blk) {
+            const bf16x8 va = __builtin_bit_cast(bf16x8, Vs[(blk * 4 + lq) * D + t * 16 + lr] & v_mask[blk]);
+            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[blk], o[t], 0, 0, 0);
+          }
+      } else {
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int blk = 0; blk < 2; ++blk) {
+            const bf16x8 va = __builtin_bit_cast(bf16x8, Vs[(blk * 4 + lq) * D + t * 16 + lr]);
+            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[blk], o[t], 0, 0, 0);
+          }
+      }
     }
   }
 

@@ -12,7 +12,7 @@ import torch
 from torch import Tensor
 
 from ..cache import CacheCapacityError, CacheManager, CacheView, plan_groups
-from ..kernels import library
+from ..kernels import library, ops
 from ..models.decoder import DecoderModel
 from .batch import StepBatch, StepEntry, build_batch, static_batch, static_batch_size
 
@@ -182,6 +182,7 @@ class ModelRunner:
                 self.states.append(torch.zeros((num_state_slots, *need.state.shape),
                                                dtype=need.state.dtype or torch.float32, device=self.device))
         self.steps_run = 0
+        self.workspace = ops.Workspace()    # scratch that this runner's launches (and its captured graphs) share
 
     # ------------------------------------------------------------ requests
     def begin(self, request_id: str) -> None:
@@ -391,6 +392,10 @@ class ModelRunner:
         ``CacheCapacityError`` (and changes nothing) if pages run out.  The
         result of a step that replays a captured graph lives in a buffer that
         the next step of the same shape overwrites."""
+        with ops.use_workspace(self.workspace):
+            return self._step(entries)
+
+    def _step(self, entries: list[StepEntry]) -> Tensor:
         if self._graphable(entries):
             return self._graph_step(entries)
         self._steady = None        # any other step may move the requests that the last decode step left

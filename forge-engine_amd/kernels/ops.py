@@ -9,6 +9,7 @@ implementation: without a GPU or without the compiled library a call raises.
 from __future__ import annotations
 
 import ctypes
+import threading
 from ctypes import c_float, c_int, c_longlong, c_void_p
 
 import torch
@@ -393,18 +394,58 @@ def qk_norm_rope_write(qkv: Tensor, q_weight: Tensor | None, k_weight: Tensor | 
 DECODE_TARGET_BLOCKS = 256     # blocks aimed at (measured: at 8 sequences x 8 kv heads four key splits beat eight)
 
 
-_SPLIT_COUNTERS: dict = {}
+class Workspace:
+    """Device memory that kernels share between launches and that must survive them: the arrival
+    counters of the decode kernel's key splits, one per (sequence, kv head), zero between launches
+    (the kernel leaves them so).  Launches that share counters must not overlap, so whoever runs
+    steps on a stream of its own (a ``ModelRunner``) owns a workspace of its own and makes it
+    current around its launches (``use_workspace``); calls outside any take the one of their
+    (device, stream).  A counter buffer is never given back while the workspace lives: a captured
+    graph keeps the address it was recorded with, so a larger buffer is added beside the old one,
+    never in its place."""
+
+    def __init__(self) -> None:
+        self._counters: dict = {}
+        self._retired: list[Tensor] = []
+
+    def split_counters(self, device: torch.device, count: int) -> Tensor:
+        key = (device.type, device.index)
+        have = self._counters.get(key)
+        if have is None or have.numel() < count:
+            if have is not None:
+                self._retired.append(have)      # launches already recorded keep using it
+            have = torch.zeros(max(count, 4096, 2 * (have.numel() if have is not None else 0)),
+                               dtype=torch.int32, device=device)
+            self._counters[key] = have
+        return have
+
+
+_WORKSPACES = threading.local()
+_STREAM_WORKSPACES: dict = {}
+
+
+class use_workspace:
+    """Make ``workspace`` the one that this thread's kernel calls draw from."""
+
+    def __init__(self, workspace: Workspace) -> None:
+        self.workspace = workspace
+
+    def __enter__(self) -> Workspace:
+        self.before = getattr(_WORKSPACES, "current", None)
+        _WORKSPACES.current = self.workspace
+        return self.workspace
+
+    def __exit__(self, *exc) -> None:
+        _WORKSPACES.current = self.before
 
 
 def _split_counters(device, count: int) -> Tensor:
-    """Arrival counters of the decode kernel's key splits, one per (sequence, kv head): zero
-    between launches (the kernel leaves them so), shared by all launches of a device's stream."""
-    key = (device.type, device.index)
-    have = _SPLIT_COUNTERS.get(key)
-    if have is None or have.numel() < count:
-        have = torch.zeros(max(count, 4096), dtype=torch.int32, device=device)
-        _SPLIT_COUNTERS[key] = have
-    return have
+    current = getattr(_WORKSPACES, "current", None)
+    if current is None:
+        stream = torch._C._cuda_getCurrentRawStream(device.index if device.index is not None else torch.cuda.current_device()) \
+            if device.type == "cuda" else 0
+        current = _STREAM_WORKSPACES.setdefault((device.type, device.index, stream), Workspace())
+    return current.split_counters(device, count)
 
 
 def decode_splits(num_decode: int, kv_heads: int, max_ctx: int) -> int:

@@ -41,3 +41,33 @@ def test_the_fused_decode_attention_serves_what_it_says():
     for change in (dict(head_dim=96, rotary_dim=96), dict(rotary_dim=64), dict(q_heads=80), dict(block_size=8),
                    dict(block_size=48), dict(q_heads=30)):
         assert not ops.decode_prepare_supported(torch.bfloat16, **{**ok, **change}), change
+
+
+def test_split_counters_outlive_their_growth():
+    """A captured graph keeps the address of the counters it was recorded with: when a step needs
+    more of them, the old buffer must stay alive (and zero) beside the new one."""
+    import torch
+
+    workspace = ops.Workspace()
+    cpu = torch.device("cpu")
+    first = workspace.split_counters(cpu, 64)
+    address = first.data_ptr()
+    assert workspace.split_counters(cpu, 4096) is first           # no growth: the same buffer
+    grown = workspace.split_counters(cpu, 100000)
+    assert grown.numel() >= 100000 and grown.data_ptr() != address
+    assert any(old is first for old in workspace._retired)        # still referenced, so never handed to another tensor
+    assert first.data_ptr() == address and int(first.abs().sum()) == 0
+    assert workspace.split_counters(cpu, 5000) is grown           # and later launches use the larger one
+
+
+def test_workspaces_are_per_owner():
+    import torch
+
+    a, b = ops.Workspace(), ops.Workspace()
+    cpu = torch.device("cpu")
+    with ops.use_workspace(a):
+        mine = ops._split_counters(cpu, 8)
+        with ops.use_workspace(b):
+            assert ops._split_counters(cpu, 8) is not mine
+        assert ops._split_counters(cpu, 8) is mine
+    assert ops._split_counters(cpu, 8) is not mine                # outside: the default of (device, stream)

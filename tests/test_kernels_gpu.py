@@ -824,6 +824,73 @@ def test_decode_attention_far_key_and_page_edges(ops):
                 torch.testing.assert_close(got[0, h * head_dim:(h + 1) * head_dim], vp[page, 0, :, slot].float(), atol=2e-2, rtol=2e-2)
 
 
+def _poison_unowned_slots(kp, vp, table, owned_from, owned_to, block_size):
+    """NaN into every slot of the pages that no live key owns: whole pages outside the tables,
+    slots at or beyond a sequence's context, slots below its window.  owned_from/to: per sequence."""
+    owned = torch.zeros(kp.shape[0], block_size, dtype=torch.bool)
+    for s in range(table.shape[0]):
+        for key in range(owned_from[s], owned_to[s]):
+            owned[int(table[s, key // block_size]), key % block_size] = True
+    kp[~owned[:, None, :, None].expand_as(kp)] = float("nan")
+    vp[~owned[:, None, None, :].expand_as(vp)] = float("nan")
+
+
+@pytest.mark.parametrize("window", [None, 40])
+def test_attention_kernels_ignore_what_unowned_slots_hold(ops, window):
+    """A page that is leased again still holds what the request before left there, which may be a
+    NaN (a batch that overflowed).  Every slot that no live key of the batch owns is set to NaN:
+    the fast kernels (single tokens with and without key splits, portions) must give what they
+    give for clean pages.  With a window, the slots below it count as unowned too and their table
+    entries are -1, as the cache manager leaves them once the window has passed."""
+    g = torch.Generator().manual_seed(43)
+    q_heads, kv_heads, head_dim, block_size = 8, 2, 128, 16
+    seqs = [(0, 70), (100, 1), (13, 9), (129, 1), (3, 1), (60, 66), (0, 2), (31, 1)]
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                extra_width=2 * kv_heads * head_dim)
+    kw = dict(num_seqs=len(seqs), max_q_len=70, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+              scale=head_dim ** -0.5, window=window)
+    want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype), cu, ctx, table, **kw).float()
+    first = [0 if window is None else max(0, before - window + 1) for before, _ in seqs]
+    kp_bad, vp_bad, table_bad = kp.clone(), vp.clone(), table.clone()
+    _poison_unowned_slots(kp_bad, vp_bad, table, first, [b + n for b, n in seqs], block_size)
+    for s, low in enumerate(first):
+        table_bad[s, :low // block_size] = -1               # pages wholly below the window were given back
+    assert torch.isnan(kp_bad).any() and torch.isnan(vp_bad).any()
+    for splits in (1, 3):
+        got = ops.paged_attention(q.to(DEV), kp_bad.to(DEV), vp_bad.to(DEV),
+                                  torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
+                                  cu.to(DEV), ctx.to(DEV), table_bad.to(DEV), num_decode=4, max_ctx=130, splits=splits, **kw).cpu().float()
+        assert torch.isfinite(got).all()
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("window", [None, 40])
+def test_decode_attention_that_prepares_ignores_what_unowned_slots_hold(ops, window):
+    g = torch.Generator().manual_seed(44)
+    contexts = [0, 15, 16, 100, 129, 31]
+    qkv, kp, vp, cu, ctx, table, qw, kw, inv_freq, positions, token_seq = _prepare_case(g, 8, 2, 128, 16, contexts)
+    sizes = dict(q_heads=8, kv_heads=2, head_dim=128)
+    qkv_ref, kp_ref, vp_ref = qkv.clone(), kp.clone(), vp.clone()
+    refs.qk_norm_rope_write(qkv_ref, qw, kw, inv_freq, positions, token_seq, table, kp_ref, vp_ref,
+                            rotary_dim=128, eps=1e-6, **sizes)
+    want = refs.paged_attention(qkv_ref, kp_ref, vp_ref, torch.empty(6, 1024, dtype=qkv.dtype), cu, ctx, table,
+                                num_seqs=6, max_q_len=1, scale=128 ** -0.5, window=window, **sizes).float()
+    first = [0 if window is None else max(0, before - window + 1) for before in contexts]
+    table_bad = table.clone()
+    for s, low in enumerate(first):
+        table_bad[s, :low // 16] = -1
+    for splits in (1, 3):
+        kp_bad, vp_bad = kp.clone(), vp.clone()
+        _poison_unowned_slots(kp_bad, vp_bad, table, first, contexts, 16)   # the new token's slot is unowned before the step
+        kp_dev, vp_dev = kp_bad.to(DEV), vp_bad.to(DEV)
+        out = torch.full((6, 1024), float("nan"), dtype=qkv.dtype, device=DEV)
+        ops.decode_attention_prepare(qkv.to(DEV), qw.to(DEV), kw.to(DEV), inv_freq.to(DEV), kp_dev, vp_dev, out,
+                                     cu.to(DEV), ctx.to(DEV), table_bad.to(DEV), eps=1e-6, scale=128 ** -0.5, window=window,
+                                     max_ctx=130, splits=splits, **sizes)
+        assert torch.isfinite(out).all()
+        torch.testing.assert_close(out.cpu().float(), want, atol=2e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [
     (8, 2, 128, 16), (5, 5, 64, 16), (12, 1, 128, 32), (3, 3, 64, 64),
 ])
