@@ -68,6 +68,12 @@ def plan_groups(needs: list[CacheNeeds], schedule) -> tuple[list[CacheGroup], di
             owner = needs[call.cache].paged
             if (owner.kv_heads, owner.head_dim) != (paged.kv_heads, paged.head_dim):
                 raise ValueError(f"schedule entry {index} reads a cache of another geometry")
+            # the owner's window decides which pages go back: a reader that looks further back
+            # would read pages that are no longer the request's
+            if owner.window is not None and (paged.window is None or paged.window > owner.window):
+                raise ValueError(
+                    f"schedule entry {index} looks back {paged.window or 'without limit'} but reads cache slot "
+                    f"{call.cache}, which keeps only the last {owner.window} keys")
     return groups, where
 
 
@@ -117,11 +123,20 @@ class CacheManager:
         want = self.blocks_for(new_length)
         return [max(0, want - len(table)) for table in entry.tables]
 
-    def worst_case_pages(self, total_tokens: int) -> list[int]:
-        """Upper bound, per group, of the pages a request of ``total_tokens``
-        ever holds at once (a windowed group holds at most the window plus one
-        step's tokens; the bound used here is the whole length)."""
-        return [self.blocks_for(total_tokens) for _ in self.groups]
+    def worst_case_pages(self, total_tokens: int, step_tokens: int | None = None) -> list[int]:
+        """Upper bound, per group, of the pages a request of ``total_tokens`` ever holds at
+        once.  A windowed group gives back the pages its window has passed after every step, so
+        with at most ``step_tokens`` tokens of the request in a step it holds the window's keys
+        and the step's, which touch one page more than their count fills; without
+        ``step_tokens`` the bound is the whole length."""
+        whole = self.blocks_for(total_tokens)
+        bounds = []
+        for group in self.groups:
+            if group.window is None or step_tokens is None:
+                bounds.append(whole)
+            else:
+                bounds.append(min(whole, self.blocks_for(group.window - 1 + step_tokens) + 1))
+        return bounds
 
     @property
     def allocated_pages(self) -> int:

@@ -189,7 +189,8 @@ class ConcurrentGenerationEngine:
         total = len(tokens) + params.max_new_tokens
         if config.max_context is not None and total > config.max_context:
             raise OverloadedError(f"request needs {total} positions but max_context is {config.max_context}")
-        needed = max(self._runner.cache.worst_case_pages(total), default=0)
+        portion = min(config.token_budget, config.prefill_chunk or config.token_budget)
+        needed = max(self._runner.cache.worst_case_pages(total, step_tokens=portion), default=0)
         if needed > config.block_capacity:
             raise OverloadedError(
                 f"request needs {needed} KV blocks but pool capacity is {config.block_capacity}")

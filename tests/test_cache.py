@@ -142,6 +142,38 @@ def test_plan_groups_by_geometry_and_shared_slots():
                     [LayerCall(0, 0), LayerCall(1, 0, writes_cache=False)])
 
 
+def test_a_reader_may_not_look_further_back_than_the_cache_it_reads_keeps():
+    # the owner's window decides which pages go back; a reader without a window, or with a wider one,
+    # would read pages that are no longer the request's
+    owner = CacheNeeds(PagedKV(2, 16, window=8))
+    for reader_window in (None, 9):
+        with pytest.raises(ValueError, match="keeps only the last 8 keys"):
+            plan_groups([owner, CacheNeeds(PagedKV(2, 16, window=reader_window))],
+                        [LayerCall(0, 0), LayerCall(1, 0, writes_cache=False)])
+    for reader_window in (8, 3):
+        plan_groups([owner, CacheNeeds(PagedKV(2, 16, window=reader_window))],
+                    [LayerCall(0, 0), LayerCall(1, 0, writes_cache=False)])
+    # an owner that keeps everything serves any reader
+    plan_groups([CacheNeeds(PagedKV(2, 16)), CacheNeeds(PagedKV(2, 16, window=5))],
+                [LayerCall(0, 0), LayerCall(1, 0, writes_cache=False)])
+
+
+def test_worst_case_of_a_windowed_group_is_its_window_and_a_step():
+    cache = manager(capacity=64, block_size=4, window=6, groups=2)      # group 0 windowed, group 1 keeps all
+    assert cache.worst_case_pages(100) == [25, 25]
+    assert cache.worst_case_pages(100, step_tokens=1) == [3, 25]        # 6 keys touch at most 3 pages of 4
+    assert cache.worst_case_pages(100, step_tokens=8) == [5, 25]
+    assert cache.worst_case_pages(5, step_tokens=8) == [2, 2]
+    # the bound holds: decode a long request one token at a time, and in steps of eight
+    for step in (1, 8):
+        entry = cache.begin(f"r{step}")
+        for length in range(step, 100, step):
+            cache.reserve({entry.request_id: length})
+            assert sum(page != NO_PAGE for page in entry.tables[0]) <= cache.worst_case_pages(100, step_tokens=step)[0]
+            cache.commit(entry.request_id, length)
+        cache.end(entry.request_id)
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_random_orders_keep_every_page_accounted(seed):
     rng = random.Random(seed)
