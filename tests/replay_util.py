@@ -159,11 +159,15 @@ def plain_logits(model_dir, requests) -> dict[tuple[str, int], torch.Tensor]:
 # Tolerances.  float32: the engine and the plain implementation differ only in
 # the order of float32 sums (1e-5, the reference's own bound for cached against
 # uncached logits, tests/test_generation_core.py:77-82).  bfloat16: activations
-# between kernels are rounded to 8 mantissa bits; the bound is a fraction of
-# the largest logit of the row's request, set once from the rounding model
-# (about sqrt(ops) * 2^-9) and not adjusted to make a case pass.
+# between kernels are rounded to 8 mantissa bits (2^-9 relative, half a dozen
+# roundings a layer, adding up like a random walk); the bound is a fraction of
+# the largest logit of the comparison.  The worst difference seen over every
+# test of the suite is 0.5 % of that; one page of one layer swapped between two
+# requests moves the logits by 3 % to 50 %
+# (test_swapped_pages_of_one_layer_are_seen_in_both_dtypes), so the bound sits
+# between the two, three times above the first.
 F32_ATOL, F32_RTOL = 1e-5, 1e-4
-BF16_FRACTION = 0.04
+BF16_FRACTION = 0.015
 
 
 def compare(got: dict, want: dict, dtype: str) -> float:

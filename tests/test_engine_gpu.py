@@ -123,8 +123,22 @@ def test_temperature_sampling_is_seeded_and_batch_independent(folders):
     alone = [engine.generate([p], params)[0] for p in prompts]
     assert together == alone
     assert engine.generate(prompts[:1], SamplingParams(temperature=0.8, seed=99, max_new_tokens=12))[0] != alone[0]
-    top = engine.generate(prompts[:2], SamplingParams(temperature=0.9, top_k=3, top_p=0.9, min_p=0.05, seed=5, max_new_tokens=6))
+    filtered = SamplingParams(temperature=0.9, top_k=3, top_p=0.9, min_p=0.05, seed=5, max_new_tokens=6)
+    top = engine.generate(prompts[:2], filtered)
     assert all(len(t) == 6 for t in top)
+    assert engine.generate(prompts[:2], filtered) == top
+    # every drawn token is one that the plain filters leave (sampling.py:83-140 of the reference)
+    weights = folder_weights(folders["B"])
+    kept_sizes = []
+    for prompt, tokens in zip(prompts[:2], top):
+        ids = list(prompt)
+        for token in tokens:
+            logits = plain.forward(weights, TINY["B"], ids)[-1]
+            left = plain.filter_logits(logits[None], 0.9, top_k=3, top_p=0.9, min_p=0.05)[0]
+            assert torch.isfinite(left[token]), f"token {token} after {len(ids)} ids was filtered out"
+            kept_sizes.append(int(torch.isfinite(left).sum()))
+            ids.append(token)
+    assert max(kept_sizes) <= 3
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

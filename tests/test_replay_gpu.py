@@ -74,6 +74,47 @@ def test_mixed_replay_reuses_pages(dtype, folders, plain_cache, tmp_path):
     ru.compare(got, expected("B", folders, plain_cache, requests), dtype)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_swapped_pages_of_one_layer_are_seen_in_both_dtypes(name, dtype, folders, plain_cache):
+    """The control of the comparisons above: two requests are fed all but their last eight tokens,
+    then one page of one layer changes places with a page of the other request (as a wrong entry
+    in that layer's block table would have it), and the last tokens are decoded.  The comparison
+    with the plain implementation must fail, in bfloat16 at its own bound too; without the swap
+    the same steps pass."""
+    import torch
+    from forge_engine_amd.engine import ModelRunner, StepEntry, load_model
+
+    requests = ru.make_requests(TINY[name], 3, (70, 90))
+    want = expected(name, folders, plain_cache, requests)
+    _, model = load_model(folders[name], dtype=dtype, device="cuda:0")
+    for layer in (None, 0, len(model.schedule) - 1):
+        runner = ModelRunner(model, block_size=BLOCK_SIZE[name], block_capacity=64, num_state_slots=4)
+        for request_id, tokens in requests.items():
+            runner.begin(request_id)
+            runner.step([StepEntry(request_id, tokens[:-8], [])])
+        if layer is not None:
+            mine = runner.cache.request("r0").tables[0][1]
+            theirs = runner.cache.request("r1").tables[0][2]
+            for pages in (runner.key_pages[0][layer], runner.value_pages[0][layer]):
+                kept = pages[mine].clone()
+                pages[mine].copy_(pages[theirs])
+                pages[theirs].copy_(kept)
+        got = {}
+        for i in range(8):
+            entries = [StepEntry(r, [t[len(t) - 8 + i]], [0]) for r, t in requests.items()]
+            logits = runner.step(entries).cpu()
+            for row, (request_id, tokens) in zip(logits, requests.items()):
+                got[(request_id, len(tokens) - 8 + i)] = row.clone()
+        torch.cuda.synchronize()
+        tail = {key: want[key] for key in got}
+        if layer is None:
+            ru.compare(got, tail, dtype)
+        else:
+            with pytest.raises(AssertionError, match="logits differ"):
+                ru.compare(got, tail, dtype)
+
+
 def test_trace_run_program(folders, tmp_path):
     """The program itself, as a child process: protocol, files, exit code."""
     requests = ru.make_requests(TINY["A"], 6, (9, 30))
