@@ -139,11 +139,13 @@ def lm_head(z: Tensor, weights: dict, config: dict) -> Tensor:
 
 
 def forward(weights: dict, config: dict, token_ids, first_position: int = 0,
-            return_hidden: bool = False):
+            return_hidden: bool = False, rows=None):
     """Logits [T, V] (float32) for one whole sequence (qwen3.py:297-342).
 
     ``first_position`` shifts every position by a constant; with rotary
-    positions only distances count, so the result must not change.
+    positions only distances count, so the result must not change.  ``rows``:
+    logits of these positions only (the head of a large vocabulary is most of
+    the work on a CPU); the reference computes all and its callers slice.
     """
     ids = torch.as_tensor(token_ids, dtype=torch.long)
     positions = torch.arange(first_position, first_position + ids.numel())
@@ -152,6 +154,8 @@ def forward(weights: dict, config: dict, token_ids, first_position: int = 0,
     for index in range(config["num_hidden_layers"]):
         h = decoder_layer(h, weights, index, config, positions)
         hidden.append(h)
+    if rows is not None:
+        h = h[torch.as_tensor(rows, dtype=torch.long)]
     z = rms_norm(h, weights["model.norm.weight"], config["rms_norm_eps"])
     logits = lm_head(z, weights, config)
     return (logits, hidden) if return_hidden else logits

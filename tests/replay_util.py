@@ -29,13 +29,15 @@ def round64(n: int) -> int:
 class TraceBuilder:
     """Collects steps; remembers which (request, position) each output row is."""
 
-    def __init__(self) -> None:
+    def __init__(self, want_all: bool = True) -> None:
+        self.want_all = want_all          # logits at every token of a step, or only at each entry's last
         self.steps: list[dict] = []
         self.rows: dict[int, list[tuple[str, int]]] = {}
         self.fed: dict[str, int] = {}
         self.peak_tokens = 0
 
-    def step(self, parts: list[tuple[str, list[int]]], end=(), want_all: bool = True) -> None:
+    def step(self, parts: list[tuple[str, list[int]]], end=(), want_all: bool | None = None) -> None:
+        want_all = self.want_all if want_all is None else want_all
         index = len(self.steps)
         entries, rows = [], []
         for request_id, tokens in parts:
@@ -70,9 +72,9 @@ def trace_tail(requests, tail: int = 32) -> TraceBuilder:
     return trace
 
 
-def trace_portions(requests, sizes=(16, 7, 5, 3, 2, 2, 9, 2, 4)) -> TraceBuilder:
+def trace_portions(requests, sizes=(16, 7, 5, 3, 2, 2, 9, 2, 4), want_all: bool = True) -> TraceBuilder:
     """Portions of changing size, down to two tokens."""
-    trace = TraceBuilder()
+    trace = TraceBuilder(want_all)
     for n, (request_id, tokens) in enumerate(requests.items()):
         at, k = 0, n  # each request starts elsewhere in the size cycle
         while at < len(tokens):
@@ -84,12 +86,13 @@ def trace_portions(requests, sizes=(16, 7, 5, 3, 2, 2, 9, 2, 4)) -> TraceBuilder
     return trace
 
 
-def trace_mixed(requests, seed: int, max_live: int = 4, prompt_fraction: float = 0.6) -> TraceBuilder:
+def trace_mixed(requests, seed: int, max_live: int = 4, prompt_fraction: float = 0.6,
+                want_all: bool = True, portion_sizes=(2, 3, 5, 8, 13)) -> TraceBuilder:
     """Up to ``max_live`` requests at a time: portions of the prompts of some
     beside single decoded tokens of others; a request may sit a step out; when
     one ends the next is admitted, so its pages are used again."""
     rng = random.Random(seed)
-    trace = TraceBuilder()
+    trace = TraceBuilder(want_all)
     waiting = list(requests.items())
     live: dict[str, dict] = {}
     while waiting or live:
@@ -103,7 +106,7 @@ def trace_mixed(requests, seed: int, max_live: int = 4, prompt_fraction: float =
             state = live[request_id]
             tokens, at = state["tokens"], state["at"]
             if at < state["prompt"]:
-                size = min(rng.choice((2, 3, 5, 8, 13)), state["prompt"] - at)
+                size = min(rng.choice(portion_sizes), state["prompt"] - at)
             else:
                 size = 1
             parts.append((request_id, tokens[at:at + size]))
@@ -144,15 +147,20 @@ def collect(trace: TraceBuilder, out_dir, vocab: int):
     return got
 
 
-def plain_logits(model_dir, requests) -> dict[tuple[str, int], torch.Tensor]:
-    """The plain implementation on the folder's own tensors (widened to float32)."""
+def plain_logits(model_dir, requests, only=None) -> dict[tuple[str, int], torch.Tensor]:
+    """The plain implementation on the folder's own tensors (widened to float32).  ``only``: the
+    (request, position) pairs that are wanted (default: every position)."""
     config = json.loads((Path(model_dir) / "config.json").read_text())
     weights = {k: v.float() for k, v in load_file(str(Path(model_dir) / "model.safetensors")).items()}
     want = {}
     for request_id, tokens in requests.items():
-        logits = plain.forward(weights, config, tokens)
-        for position in range(len(tokens)):
-            want[(request_id, position)] = logits[position]
+        if only is None:
+            positions = list(range(len(tokens)))
+        else:
+            positions = sorted(position for rid, position in only if rid == request_id)
+        logits = plain.forward(weights, config, tokens, rows=positions)
+        for row, position in zip(logits, positions):
+            want[(request_id, position)] = row
     return want
 
 

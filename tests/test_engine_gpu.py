@@ -912,6 +912,66 @@ def test_layers_of_the_large_model_against_the_plain_implementation(dtype, wide_
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["portions", "mixed"])
+def test_schedules_at_the_large_widths(mode, dtype, wide_folder, tmp_path):
+    """Replay at the widths of the large model, where the products that split K over blocks, keep
+    their activations resident and serve 17 to 64 rows engage (the tiny models never reach them):
+    portions of changing size, and up to four live requests with portions of some beside decoded
+    tokens of others in a pool so small that pages are used again.  Logits at the last token of
+    every entry of every step."""
+    folder, config, weights = wide_folder
+    requests = ru.make_requests(config, 71, (40, 70, 33, 90, 25, 50, 61))
+    if mode == "portions":
+        trace = ru.trace_portions(requests, sizes=(16, 7, 33, 3, 2, 64, 9, 2, 20), want_all=False)
+    else:
+        trace = ru.trace_mixed(requests, 11, max_live=4, want_all=False, portion_sizes=(2, 3, 5, 8, 13, 21))
+        assert sum(ru.round64(len(t)) for t in requests.values()) > trace.peak_tokens     # pages are used again
+    rows = {key for keys in trace.rows.values() for key in keys}
+    got = ru.run_trace(folder, dtype, trace, tmp_path, block_size=16)
+    want = {}
+    for request_id, tokens in requests.items():
+        positions = sorted(position for rid, position in rows if rid == request_id)
+        for row, position in zip(plain.forward(weights, config, tokens, rows=positions), positions):
+            want[(request_id, position)] = row
+    ru.compare(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_scheduler_with_sixty_four_rows_at_the_large_widths(dtype, wide_folder):
+    """Forty requests through the scheduler at its largest batch (64 requests a step, 256 tokens):
+    prompts are cut into portions beside decoded tokens, and decode steps of 17 to 40 rows replay
+    graphs of the products for that many rows.  Every generated token must be the plain
+    implementation's choice at its place (teacher-forced: one plain pass over prompt and output)."""
+    import random
+    folder, config, weights = wide_folder
+    rng = random.Random(91)
+    lengths = [rng.randrange(3, 60) for _ in range(40)]
+    prompts = list(ru.make_requests(config, 92, lengths).values())
+    new_tokens = [rng.randrange(3, 9) for _ in prompts]
+    scheduler = SchedulerConfig(block_size=16, block_capacity=40 * 5, token_budget=256, max_batch_size=64,
+                                max_requests=64)
+    engine = engine_from_folder(folder, scheduler_config=scheduler, dtype=dtype)
+    ids = [engine.submit(p, sampling_params=SamplingParams(max_new_tokens=n)) for p, n in zip(prompts, new_tokens)]
+    widest = 0
+    while not engine.idle:
+        engine.step()
+        widest = max(widest, len(engine.snapshot().last_batch))
+    assert widest > 32 and engine.cache_pool.allocated_pages == 0
+    for request_id, prompt, n in zip(ids, prompts, new_tokens):
+        got = list(engine.request(request_id).output_token_ids)
+        assert len(got) == n
+        places = list(range(len(prompt) - 1, len(prompt) - 1 + n))
+        logits = plain.forward(weights, config, prompt + got[:-1], rows=places)
+        for row, token in zip(logits, got):
+            if dtype == "float32":
+                # among 151,936 logits two can lie closer than float32 sums in another order resolve
+                # (seen: 4.53608 twice); anything further from the top than that is a wrong token
+                assert token == int(row.argmax()) or float(row.max() - row[token]) <= 2 * ru.F32_ATOL, request_id
+            else:
+                assert float(row.max() - row[token]) <= ru.BF16_FRACTION * float(row.abs().max()), request_id
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_name_used_again_decodes_from_its_new_pages(dtype, folders):
     """A request ends and another begins under the same name with a table of the same length
     but other pages (a third request took the old ones meanwhile): the captured decode step
