@@ -90,7 +90,8 @@ class _PortionGraph:
     Sequences beyond the step's own are empty (no tokens, so every kernel skips them), wanted
     rows beyond the step's own repeat row 0 and are cut off the result."""
 
-    def __init__(self, num_tokens: int, num_seqs: int, num_wanted: int, widths, device) -> None:
+    def __init__(self, num_tokens: int, num_seqs: int, num_wanted: int, widths, device, pad_state_slot: int = 0) -> None:
+        self.pad_state_slot = pad_state_slot
         size = static_batch_size(num_seqs, widths, num_tokens, num_wanted)
         self.host = torch.empty(size, dtype=torch.int32).pin_memory()
         self.dev = torch.zeros(size, dtype=torch.int32, device=device)
@@ -134,7 +135,7 @@ class _PortionGraph:
         start[n:] = 0
         slots = buf[3 * t + 3 * b + 1:3 * t + 4 * b + 1]
         slots[:n] = [r.state_slot for r in records]
-        slots[n:] = 0
+        slots[n:] = self.pad_state_slot
         for g, width in enumerate(self.widths):
             base = self.table_at[g]
             for i, record in enumerate(records):
@@ -179,14 +180,22 @@ class ModelRunner:
             if need.state is None:
                 self.states.append(None)
             else:
-                self.states.append(torch.zeros((num_state_slots, *need.state.shape),
+                # one row more than there are slots: the empty sequences that pad a captured step
+                # point there, so that a mixer that writes its state back never touches a live slot
+                self.states.append(torch.zeros((num_state_slots + 1, *need.state.shape),
                                                dtype=need.state.dtype or torch.float32, device=self.device))
+        self.pad_state_slot = num_state_slots
         self.steps_run = 0
         self.workspace = ops.Workspace()    # scratch that this runner's launches (and its captured graphs) share
 
     # ------------------------------------------------------------ requests
     def begin(self, request_id: str) -> None:
-        self.cache.begin(request_id)
+        """Lease a state slot and empty tables for the request.  The slot's fixed-size state starts
+        at zero: the runner clears it here, so a mixer never has to know a request's first step."""
+        record = self.cache.begin(request_id)
+        for state in self.states:
+            if state is not None:
+                state[record.state_slot].zero_()
 
     def end(self, request_id: str) -> None:
         self.cache.end(request_id)
@@ -224,10 +233,14 @@ class ModelRunner:
         tables = [[record.tables[g] for record in records] for g in range(len(self.cache.groups))]
         return build_batch(entries, before, [r.state_slot for r in records], tables, self.device)
 
-    def cache_views(self, batch: StepBatch) -> list[CacheView | None]:
+    def cache_views(self, batch: StepBatch, scratch_state: bool = False) -> list[CacheView | None]:
+        """What each schedule call sees of the cache in this step.  ``scratch_state``: fixed-size
+        state is handed out as a copy, for a run whose effects on it must not stay."""
         views: list[CacheView | None] = []
         for index, call in enumerate(self.model.schedule):
             state = self.states[index]
+            if scratch_state and state is not None:
+                state = state.clone()
             if call.cache in self._where:
                 g, j = self._where[call.cache]
                 group = self.cache.groups[g]
@@ -303,11 +316,7 @@ class ModelRunner:
             batch = build_batch(entries, before, [r.state_slot for r in records], tables, self.device,
                                 widths=widths, static=(slot.host, slot.dev), max_ctx=bound)
             views = self.cache_views(batch)
-            side = torch.cuda.Stream(device=self.device)
-            side.wait_stream(torch.cuda.current_stream(self.device))
-            with torch.cuda.stream(side):      # once eagerly: libraries load, scratch gets its size
-                self.model.forward(batch, views)
-            torch.cuda.current_stream(self.device).wait_stream(side)
+            self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 slot.logits = self.model.forward(batch, views)
@@ -320,6 +329,18 @@ class ModelRunner:
             room = min(len(table) * self.block_size - record.length for record in records for table in record.tables)
             self._steady = _SteadyDecode(tuple(e.request_id for e in entries), records, slot, room)
         return slot.logits
+
+    def _warm_up(self, batch: StepBatch) -> None:
+        """Run the step once eagerly before it is captured (libraries load, scratch gets its
+        size).  The step is then captured (which runs nothing) and replayed, so its effects would
+        happen twice: writes of keys and values into pages give the same pages both times, but a
+        mixer's update of its fixed-size state does not, so this run gets a copy of the state."""
+        views = self.cache_views(batch, scratch_state=True)
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):
+            self.model.forward(batch, views)
+        torch.cuda.current_stream(self.device).wait_stream(side)
 
     def _portion_key(self, entries: list[StepEntry]):
         """The shape under which a step with prompt portions may be captured, or None."""
@@ -357,7 +378,7 @@ class ModelRunner:
                 return None
             if len(self._portion_graphs) >= GRAPH_LIMIT:
                 self._portion_graphs.pop(next(iter(self._portion_graphs)))
-            slot = _PortionGraph(shape[0], shape[1], shape[2], widths, self.device)
+            slot = _PortionGraph(shape[0], shape[1], shape[2], widths, self.device, self.pad_state_slot)
         self._portion_graphs[key] = slot
         cache.reserve({e.request_id: n for e, n in zip(entries, after)})
         records = [cache.request(e.request_id) for e in entries]
@@ -369,11 +390,7 @@ class ModelRunner:
             batch = static_batch(slot.dev, num_tokens=shape[0], num_seqs=shape[1], num_wanted=shape[2],
                                  widths=widths, max_q_len=shape[0], max_ctx=widths[0] * self.block_size if widths else 0)
             views = self.cache_views(batch)
-            side = torch.cuda.Stream(device=self.device)
-            side.wait_stream(torch.cuda.current_stream(self.device))
-            with torch.cuda.stream(side):      # once eagerly: libraries load, scratch gets its size
-                self.model.forward(batch, views)
-            torch.cuda.current_stream(self.device).wait_stream(side)
+            self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 slot.logits = self.model.forward(batch, views)

@@ -395,6 +395,35 @@ class EmaMixer(Mixer):
         return out
 
 
+class DeviceEmaMixer(EmaMixer):
+    """The same mixer with nothing decided on the host: it reads the step's layout from the
+    device tensors of the batch (``cu_q``, ``token_seq``, ``state_slots``), so its steps may be
+    captured and replayed.  Within a step, token t of a sequence that starts at token a gets
+    s_t = decay^(t-a+1) * s_before + sum_{a <= u <= t} decay^(t-u) x_u; the state after the
+    sequence's last token goes back to its slot, and an empty sequence leaves its slot alone.
+    The slot starts at zero because the runner clears it when the request begins."""
+
+    graph_safe = True
+
+    def forward(self, x, batch, cache, writes_cache=True):
+        tokens = x.shape[0]
+        xf = x.float()
+        cu, seq, slots = batch.cu_q.long(), batch.token_seq.long(), batch.state_slots.long()
+        t = torch.arange(tokens, device=x.device)
+        start = cu.index_select(0, seq)
+        distance = t[:, None] - t[None, :]
+        visible = (seq[:, None] == seq[None, :]) & (distance >= 0)
+        mix = torch.where(visible, torch.pow(self.decay, distance.clamp(min=0).float()), torch.zeros((), device=x.device))
+        before = cache.state.index_select(0, slots)
+        carried = torch.pow(self.decay, (t - start + 1).float())[:, None] * before.index_select(0, seq)
+        states = mix @ xf + carried
+        lengths = cu[1:] - cu[:-1]
+        last = (cu[1:] - 1).clamp(min=0)
+        after = torch.where((lengths > 0)[:, None], states.index_select(0, last), before)
+        cache.state.index_copy_(0, slots, after)
+        return states @ self.weight.float().T
+
+
 @dataclass(frozen=True)
 class ToyConfig(ModelConfig):
     vocab_size: int
@@ -490,8 +519,12 @@ def toy_plain_forward(weights, config: ToyConfig, tokens):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_toy_architecture_registered_from_a_test(dtype):
-    register_part("mixer", "toy_ema", EmaMixer, replace=True)
+@pytest.mark.parametrize("ema", [EmaMixer, DeviceEmaMixer])
+def test_toy_architecture_registered_from_a_test(dtype, ema):
+    """``ema``: the stateful mixer decides on the host (its steps run eagerly), or reads only
+    device tensors (its steps are captured and replayed; a captured step must update the state
+    once, not once more for the run that precedes the capture)."""
+    register_part("mixer", "toy_ema", ema, replace=True)
     register_architecture("ToyMixedLM", ToyConfig, toy_plan, replace=True)
     raw = {"architectures": ["ToyMixedLM"], "vocab_size": 90, "hidden_size": 40, "intermediate_size": 72,
            "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16, "window": 6, "decay": 0.5,
@@ -555,6 +588,9 @@ def test_toy_architecture_registered_from_a_test(dtype):
             runner.end(k)
         assert runner.cache.allocated_pages == 0
         runner.cache.check_invariants()
+    # the mixer that reads only device tensors went through captured steps, single tokens and portions
+    assert (runner.graph_replays > 10) == (ema is DeviceEmaMixer)
+    assert (runner.portion_graph_replays > 0) == (ema is DeviceEmaMixer)
     for k in requests:
         rows = torch.cat(got[k])
         scale = float(want[k].abs().max())
