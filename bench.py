@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model qwen3-4b|qwen3-8b|qwen3-32b]
 
 The default run has the layer sizes of Qwen3-4B with random weights (bfloat16),
 eight requests decoding from 1,024-token random prompts in a cache pool sized
@@ -10,6 +10,18 @@ one 2,048-token prompt, and the decode step's memory roofline.  A "step" is one
 decode step: every request's last token through the model, and the next token
 sampled (greedy) and read back.  Everything goes through the engine's own step
 function, cache and kernels.
+
+Protocol (after tools/validate_l4.py:136-183 of the reference): W untimed steps,
+then K steps each bracketed by a pair of device events; the line reports their
+minimum, 10th percentile, median, 90th percentile and maximum, ``value`` is
+batch / median, and ``ms_per_step_wall`` is the host's clock over the same K
+steps (synchronised on both sides).  The roofline is given against the
+published peak and against a streaming read measured when the program starts.
+
+``--through scheduler`` decodes through ``ConcurrentGenerationEngine.step()``
+(admission, selection, sampling and finishing included) instead of calling the
+step function directly.  ``--workload mixed`` runs requests with prompts of
+random lengths to completion through the scheduler and reports the whole job.
 """
 
 from __future__ import annotations
@@ -27,12 +39,35 @@ sys.path.insert(0, str(ROOT))
 HBM_BYTES_PER_S = 8.0e12
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-QWEN3_4B = {
-    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "hidden_act": "silu",
-    "vocab_size": 151936, "hidden_size": 2560, "intermediate_size": 9728, "num_hidden_layers": 36,
-    "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
-    "max_position_embeddings": 262144, "rms_norm_eps": 1e-6, "rope_theta": 5000000.0,
-    "tie_word_embeddings": True, "attention_bias": False, "eos_token_id": 151645,
+
+def _qwen3(**sizes) -> dict:
+    base = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "hidden_act": "silu",
+            "vocab_size": 151936, "num_key_value_heads": 8, "head_dim": 128, "max_position_embeddings": 262144,
+            "rms_norm_eps": 1e-6, "attention_bias": False, "eos_token_id": 151645}
+    base.update(sizes)
+    return base
+
+
+# Sizes and workloads of the three models the benchmark names; the first is the default.
+MODELS = {
+    "qwen3-4b": {
+        "label": "Qwen3-4B",
+        "config": _qwen3(hidden_size=2560, intermediate_size=9728, num_hidden_layers=36, num_attention_heads=32,
+                         rope_theta=5000000.0, tie_word_embeddings=True),
+        "batch": 8, "points": "1,64", "prompt_len": 1024, "context": 8192,
+    },
+    "qwen3-8b": {
+        "label": "Qwen3-8B",
+        "config": _qwen3(hidden_size=4096, intermediate_size=12288, num_hidden_layers=36, num_attention_heads=32,
+                         rope_theta=1000000.0, tie_word_embeddings=False),
+        "batch": 8, "points": "1,64", "prompt_len": 1024, "context": 8192,
+    },
+    "qwen3-32b": {
+        "label": "Qwen3-32B",
+        "config": _qwen3(hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64,
+                         rope_theta=1000000.0, tie_word_embeddings=False),
+        "batch": 8, "points": "1,32", "prompt_len": 2048, "context": 16384,
+    },
 }
 
 
@@ -41,18 +76,32 @@ def parse_args():
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=50)
     parser.add_argument("--warmup", type=int, default=10)
-    parser.add_argument("--batch", type=int, default=8)
-    parser.add_argument("--prompt-len", type=int, default=1024)
-    parser.add_argument("--context", type=int, default=8192)
+    parser.add_argument("--model", choices=sorted(MODELS), default="qwen3-4b")
+    parser.add_argument("--batch", type=int, default=None)
+    parser.add_argument("--prompt-len", type=int, default=None)
+    parser.add_argument("--context", type=int, default=None)
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--block-size", type=int, default=16)
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
     parser.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
-    parser.add_argument("--points", default="1,64", help="other decode batch sizes to report")
+    parser.add_argument("--points", default=None, help="other decode batch sizes to report")
     parser.add_argument("--phase", choices=("all", "decode", "prefill"), default="all",
                         help="run one phase only (for profiles); the record then holds that phase alone")
+    parser.add_argument("--through", choices=("step", "scheduler"), default="step",
+                        help="decode by calling the step function, or through the scheduler's step()")
+    parser.add_argument("--workload", choices=("steady", "mixed"), default="steady",
+                        help="mixed: requests with prompts of random lengths run to completion through the scheduler")
+    parser.add_argument("--requests", type=int, default=64, help="mixed workload: number of requests")
+    parser.add_argument("--prompt-range", default="128,4096", help="mixed workload: prompt lengths, uniform")
+    parser.add_argument("--new-tokens", type=int, default=256, help="mixed workload: tokens generated per request")
+    parser.add_argument("--token-budget", type=int, default=2048, help="scheduler: tokens a step")
     parser.add_argument("--seed", type=int, default=0)
-    return parser.parse_args()
+    args = parser.parse_args()
+    chosen = MODELS[args.model]
+    for name in ("batch", "prompt_len", "context", "points"):
+        if getattr(args, name) is None:
+            setattr(args, name, chosen[name])
+    return args
 
 
 def weight_bytes(model) -> int:
@@ -69,6 +118,21 @@ def weight_bytes(model) -> int:
     return total
 
 
+def percentile(ordered: list[float], fraction: float) -> float:
+    """Linear interpolation between the two nearest of the sorted values."""
+    at = fraction * (len(ordered) - 1)
+    low = int(at)
+    high = min(low + 1, len(ordered) - 1)
+    return ordered[low] + (ordered[high] - ordered[low]) * (at - low)
+
+
+def spread(times_ms: list[float]) -> dict:
+    ordered = sorted(times_ms)
+    return {"min": round(ordered[0], 4), "p10": round(percentile(ordered, 0.1), 4),
+            "median": round(percentile(ordered, 0.5), 4), "p90": round(percentile(ordered, 0.9), 4),
+            "max": round(ordered[-1], 4)}
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -76,28 +140,46 @@ def main() -> int:
         return 2
     import torch
 
-    from forge_engine_amd.config import load_model_config
+    from forge_engine_amd.config import SchedulerConfig, load_model_config
     from forge_engine_amd.engine import ModelRunner, StepEntry, random_model
+    from forge_engine_amd.engine.scheduler import ConcurrentGenerationEngine
     from forge_engine_amd.sampling import SamplingParams
     from forge_engine_amd.sampling.sampler import Sampler
 
-    raw = dict(QWEN3_4B)
+    chosen = MODELS[args.model]
+    raw = dict(chosen["config"])
     full_layers = raw["num_hidden_layers"]
     if args.layers is not None:
         raw["num_hidden_layers"] = args.layers
     config = load_model_config(raw)
     device = torch.device("cuda:0")
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
+
+    def timed(fn, warmup, steps):
+        """Per-step device times (ms) of ``steps`` calls after ``warmup`` untimed ones, and the
+        host's mean over the same calls."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        start = time.perf_counter()
+        for begin, end in events:
+            begin.record()
+            fn()
+            end.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - start) / steps
+        return [begin.elapsed_time(end) for begin, end in events], wall * 1e3
+
+    def measured_read_bandwidth() -> float:
+        """Bytes a second of a plain streaming read (a sum over 1 GB that no cache holds)."""
+        data = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+        times, _ = timed(lambda: data.sum(), 3, 10)
+        del data
+        return (1 << 30) / (spread(times)["median"] * 1e-3)
+
+    read_peak = measured_read_bandwidth()
     model = random_model(config, args.seed, dtype=dtype, device=device)
-    batches = sorted({args.batch, *[int(b) for b in args.points.split(",") if b]})
-    if args.phase == "decode":
-        batches = [args.batch]
-    spare = args.steps + args.warmup + 8
-    per_request = -(-(args.prompt_len + spare) // args.block_size)
-    capacity = max(args.batch * -(-args.context // args.block_size), max(batches) * per_request,
-                   -(-(args.prefill_tokens + 1) // args.block_size))
-    runner = ModelRunner(model, block_size=args.block_size, block_capacity=capacity,
-                         num_state_slots=max(batches) + 1)
     sampler = Sampler(device)
     greedy = SamplingParams()
     generator = torch.Generator().manual_seed(args.seed)
@@ -105,15 +187,55 @@ def main() -> int:
     def random_tokens(n):
         return torch.randint(0, config.vocab_size, (n,), generator=generator).tolist()
 
-    def timed(fn, warmup, steps):
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
-        start = time.perf_counter()
-        for _ in range(steps):
-            fn()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - start) / steps
+    element = 2 if args.dtype == "bf16" else 4
+    layers = config.num_hidden_layers
+    kv_bytes_per_token = 2 * layers * config.kv_size * element
+
+    if args.workload == "mixed":
+        low, high = (int(v) for v in args.prompt_range.split(","))
+        lengths = torch.randint(low, high + 1, (args.requests,), generator=generator).tolist()
+        pages = sum(-(-(n + args.new_tokens) // args.block_size) for n in lengths)
+        runner = ModelRunner(model, block_size=args.block_size, block_capacity=pages, num_state_slots=args.requests)
+        scheduler = SchedulerConfig(max_requests=args.requests, max_batch_size=min(64, args.requests),
+                                    token_budget=args.token_budget, block_size=args.block_size, block_capacity=pages,
+                                    max_context=args.context)
+        engine = ConcurrentGenerationEngine(runner, sampler, greedy, scheduler, eos_token_ids=())
+        for round_index in range(2):        # the first round warms up (graphs are captured), the second is timed
+            ids = [engine.submit(random_tokens(n), sampling_params=SamplingParams(max_new_tokens=args.new_tokens))
+                   for n in lengths]
+            torch.cuda.synchronize()
+            start = time.perf_counter()
+            steps = 0
+            while not engine.idle:
+                engine.step()
+                steps += 1
+            torch.cuda.synchronize()
+            seconds = time.perf_counter() - start
+            for request_id in ids:
+                engine.forget(request_id)
+        generated = args.requests * args.new_tokens
+        print(json.dumps({
+            "workload": "mixed", "through": "scheduler", "model": chosen["label"], "dtype": args.dtype,
+            "requests": args.requests, "prompt_tokens": sum(lengths), "generated_tokens": generated,
+            "token_budget": args.token_budget, "steps": steps, "seconds": round(seconds, 3),
+            "generated_tokens_per_s": round(generated / seconds, 1),
+            "all_tokens_per_s": round((generated + sum(lengths)) / seconds, 1),
+            "layers_run": layers, "layers_model": full_layers,
+        }))
+        return 0
+
+    batches = sorted({args.batch, *[int(b) for b in args.points.split(",") if b]})
+    if args.phase == "decode" or args.through == "scheduler":
+        batches = [args.batch]
+    spare = args.steps + args.warmup + 8
+    # through the scheduler the first requests already decode while the last prompts are still fed
+    joining = max(batches) * args.prompt_len // max(args.token_budget, 1) + 2 if args.through == "scheduler" else 0
+    spare += joining
+    per_request = -(-(args.prompt_len + spare) // args.block_size)
+    capacity = max(args.batch * -(-args.context // args.block_size), max(batches) * per_request,
+                   -(-(args.prefill_tokens + 1) // args.block_size))
+    runner = ModelRunner(model, block_size=args.block_size, block_capacity=capacity,
+                         num_state_slots=max(batches) + 1)
 
     def decode_run(batch):
         names = [f"d{batch}_{i}" for i in range(batch)]
@@ -133,16 +255,30 @@ def main() -> int:
             for n, t in zip(names, tokens):
                 state[n] = t
 
-        seconds = timed(one_step, args.warmup, args.steps)
+        times, wall = timed(one_step, args.warmup, args.steps)
         contexts = [runner.length(n) for n in names]
         for name in names:
             runner.end(name)
-        return seconds, sum(contexts) / batch - args.steps / 2.0
+        return times, wall, sum(contexts) / batch - args.steps / 2.0
 
-    if args.phase == "prefill":
-        results = {}
-    else:
-        results = {b: decode_run(b) for b in batches}
+    def scheduler_run(batch):
+        """The same decode steps through the scheduler: requests are admitted with their prompts,
+        stepped until every one decodes, then K calls of step() are timed."""
+        scheduler = SchedulerConfig(max_requests=batch, max_batch_size=batch, token_budget=max(args.token_budget, batch),
+                                    block_size=args.block_size, block_capacity=capacity)
+        engine = ConcurrentGenerationEngine(runner, sampler, greedy, scheduler, eos_token_ids=())
+        budget = SamplingParams(max_new_tokens=args.steps + args.warmup + 4 + joining)
+        ids = [engine.submit(random_tokens(args.prompt_len), sampling_params=budget) for _ in range(batch)]
+        while any(n != 1 for n in engine.snapshot().last_batch_tokens) or len(engine.snapshot().last_batch) != batch:
+            engine.step()
+        times, wall = timed(engine.step, args.warmup, args.steps)
+        mean_ctx = sum(runner.length(request_id) for request_id in ids) / batch - args.steps / 2.0
+        for request_id in ids:
+            engine.cancel(request_id)
+        return times, wall, mean_ctx
+
+    run = scheduler_run if args.through == "scheduler" else decode_run
+    results = {} if args.phase == "prefill" else {b: run(b) for b in batches}
 
     # prefill: one whole prompt in one step, logits at its last token
     prompt = random_tokens(args.prefill_tokens)
@@ -156,44 +292,57 @@ def main() -> int:
         sampler.sample(logits, [greedy], [0], [0])
         runner.end(name)
 
-    if args.phase == "decode":
-        seconds = results[args.batch][0]
-        print(json.dumps({"phase": "decode", "batch": args.batch, "ms_per_step": round(seconds * 1e3, 4),
-                          "value": round(args.batch / seconds, 2), "unit": "tokens/s"}))
+    def roofline(batch, times, mean_ctx):
+        seconds = spread(times)["median"] * 1e-3
+        step_bytes = weight_bytes(model) + batch * mean_ctx * kv_bytes_per_token
+        achieved = step_bytes / seconds
+        return {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
+                "frac": round(achieved / HBM_BYTES_PER_S, 4), "measured_peak": round(read_peak / 1e9, 1),
+                "frac_measured": round(achieved / read_peak, 4)}
+
+    if args.phase == "decode" or args.through == "scheduler":
+        times, wall, mean_ctx = results[args.batch]
+        median = spread(times)["median"]
+        print(json.dumps({"phase": "decode", "through": args.through, "model": chosen["label"], "batch": args.batch,
+                          "ms_per_step": median, "ms_per_step_wall": round(wall, 4), "step_ms": spread(times),
+                          "value": round(args.batch / median * 1e3, 2), "unit": "tokens/s",
+                          "roofline": roofline(args.batch, times, mean_ctx),
+                          "layers_run": layers, "layers_model": full_layers}))
         return 0
-    prefill_seconds = timed(prefill_once, 2, max(3, min(10, args.steps)))
+    prefill_times, _ = timed(prefill_once, 2, max(3, min(10, args.steps)))
+    prefill_ms = spread(prefill_times)["median"]
     if args.phase == "prefill":
-        print(json.dumps({"phase": "prefill", "tokens": args.prefill_tokens, "ms": round(prefill_seconds * 1e3, 3),
-                          "value": round(args.prefill_tokens / prefill_seconds, 1), "unit": "tokens/s"}))
+        print(json.dumps({"phase": "prefill", "model": chosen["label"], "tokens": args.prefill_tokens, "ms": prefill_ms,
+                          "step_ms": spread(prefill_times),
+                          "value": round(args.prefill_tokens / prefill_ms * 1e3, 1), "unit": "tokens/s",
+                          "layers_run": layers, "layers_model": full_layers}))
         return 0
 
-    layers = config.num_hidden_layers
     matrix_params = layers * (config.hidden_size * (config.q_size + 2 * config.kv_size)
                               + config.q_size * config.hidden_size
                               + 3 * config.hidden_size * config.intermediate_size)
     t = args.prefill_tokens
     prefill_flops = 2.0 * t * matrix_params + 2.0 * t * t * config.q_size * layers \
         + 2.0 * config.vocab_size * config.hidden_size
-    element = 2 if args.dtype == "bf16" else 4
-    kv_bytes_per_token = 2 * layers * config.kv_size * element
-    seconds, mean_ctx = results[args.batch]
-    step_bytes = weight_bytes(model) + args.batch * mean_ctx * kv_bytes_per_token
-    achieved = step_bytes / seconds / 1e9
+    times, wall, mean_ctx = results[args.batch]
+    median = spread(times)["median"]
     record = {
-        "metric": f"decode tok/s at batch {args.batch} (Qwen3-4B sizes, {args.prompt_len}-token prompts)",
-        "value": round(args.batch / seconds, 2),
+        "metric": f"decode tok/s at batch {args.batch} ({chosen['label']} sizes, {args.prompt_len}-token prompts)",
+        "value": round(args.batch / median * 1e3, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(seconds * 1e3, 4),
+        "ms_per_step": median,
+        "ms_per_step_wall": round(wall, 4),
+        "step_ms": spread(times),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": args.dtype,
         "data": "synthetic: random weights drawn on the device, uniform-random token ids",
         "config": {
-            "model": "Qwen3-4B sizes (Qwen3ForCausalLM)", "global_batch": args.batch,
+            "model": f"{chosen['label']} sizes (Qwen3ForCausalLM)", "global_batch": args.batch,
             "seq_len": args.prompt_len, "parallelism": "single GPU", "context": args.context,
             "block_size": args.block_size, "layers_run": layers, "layers_model": full_layers,
             "hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size,
@@ -203,14 +352,11 @@ def main() -> int:
             "prefill_tokens": args.prefill_tokens, "sampling": "greedy",
         },
         "prefill": {
-            "value": round(t / prefill_seconds, 1), "tokens": t, "ms": round(prefill_seconds * 1e3, 3),
-            "frac": round(prefill_flops / prefill_seconds / PEAK_FLOPS[args.dtype], 4),
+            "value": round(t / prefill_ms * 1e3, 1), "tokens": t, "ms": prefill_ms,
+            "frac": round(prefill_flops / (prefill_ms * 1e-3) / PEAK_FLOPS[args.dtype], 4),
         },
-        "roofline": {
-            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
-            "frac": round(achieved / (HBM_BYTES_PER_S / 1e9), 4),
-        },
-        "points": {f"decode_b{b}": round(b / results[b][0], 2) for b in batches if b != args.batch},
+        "roofline": roofline(args.batch, times, mean_ctx),
+        "points": {f"decode_b{b}": round(b / spread(results[b][0])["median"] * 1e3, 2) for b in batches if b != args.batch},
     }
     print(json.dumps(record))
     return 0

@@ -38,10 +38,12 @@
 // product.
 //
 // Keys at or beyond the context read the bytes of the last key instead (their
-// scores are masked; their probabilities are zero).  In the tiles that hold keys
-// outside [first visible key, context) the values of those keys are set to zero
-// before the second product: a slot that no live key owns may hold anything (a
-// NaN that an earlier request left there), and 0 * NaN is NaN.
+// scores are masked; their probabilities are zero).  A slot that no live key owns
+// may hold anything (a NaN that an earlier request left there), and 0 * NaN is NaN:
+// in the tiles that cross the context or the window's lower edge the values of such
+// slots are set to zero in LDS before the second product (and below a window the
+// values' loads are moved up to the first visible key's chunk, so that no page is
+// read that was given back).
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -135,8 +137,12 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
   const int last_key = ctx - 1;
 
   // the page of this wave's 16 keys of a tile (uniform over the wave)
+  // Keys below the first visible one (a window) may lie in pages that were given back: the loads
+  // of values are moved up to the 16-key group and 8-key chunk of the first visible key, which
+  // hold this request's own keys; the keys' loads may read anything, their scores are replaced.
+  const int low_group = k_first & ~15, low_chunk = k_first & ~7;
   auto page_of = [&](int tile) -> int {
-    const int key = min(tile * BN + 16 * wave, last_key);
+    const int key = max(min(tile * BN + 16 * wave, last_key), low_group);
     const int id = table[key >> block_shift];
     return (id >= 0 && id < num_blocks) ? id : 0;
   };
@@ -166,7 +172,7 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
     const size_t base = ((size_t)page * kv_heads + hk) * D;
 #pragma unroll
     for (int i = 0; i < VI; ++i) {
-      const int key = min(tile * BN + v_first[i], last_key & ~7);
+      const int key = max(min(tile * BN + v_first[i], last_key & ~7), low_chunk);
       load_to_lds(value_pages + ((base + v_dim[i]) << block_shift) + (key & block_mask), &Vs[(wave * VI + i) * 64]);
     }
   };
@@ -250,35 +256,37 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
       }
     }
     FE_WAIT_VMEM(0);
+    if (__builtin_expect(key_base + BN > ctx || key_base < k_first, 0)) {
+      // The tile holds slots at or beyond the context (the 8-key chunk of the last key has them
+      // behind it; later chunks are copies of that chunk) or below the first visible key.  Their
+      // probabilities are zero, but a slot that no live key owns may hold anything (a NaN that
+      // an earlier request left there), and 0 * NaN is NaN: every wave sets them to zero in the
+      // part of the tile that it loaded itself, before the barrier hands the tile to the others.
+      // At most twice per block (its first and its last tile); one 4-byte word (two keys) at a
+      // time, so that the rare path needs no registers of the common one.
+      const int above = ctx - key_base, below = k_first - key_base;   // keys of the tile inside [below, above) count
+      unsigned int* words = (unsigned int*)Vs;
+      for (int i = 0; i < VI; ++i) {
+        const int u = (wave * VI + i) * 64 + lane;
+        const int first_key = (u / D) * 8;
+#pragma unroll 1
+        for (int j = 0; j < 4; ++j) {
+          const int k0 = first_key + 2 * j;
+          const unsigned int keep = ((k0 >= below && k0 < above) ? 0x0000ffffu : 0u) |
+                                    ((k0 + 1 >= below && k0 + 1 < above) ? 0xffff0000u : 0u);
+          if (keep != 0xffffffffu) words[u * 4 + j] &= keep;
+        }
+      }
+    }
     __syncthreads();             // the values (and the next keys) are in LDS
     if (mine) {
-      if (key_base + BN > ctx || key_base < k_first) {     // a tile with keys that nobody owns (uniform over the block)
-        uintx4 v_mask[2];
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
-          const int first_key = key_base + 32 * blk + 8 * lq;
-          const int hi = min(max(ctx - first_key, 0), 8), lo = min(max(k_first - first_key, 0), 8);
-          const unsigned int bits = ((1u << hi) - 1u) & ~((1u << lo) - 1u);
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            v_mask[blk][i] = (((bits >> (2 * i)) & 1u) ? 0x0000ffffu : 0u) | (((bits >> (2 * i + 1)) & 1u) ? 0xffff0000u : 0u);
+          const bf16x8 va = __builtin_bit_cast(bf16x8, Vs[(blk * 4 + lq) * D + t * 16 + lr]);
+          o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[blk], o[t], 0, 0, 0);
         }
-#pragma unroll
-        for (int t = 0; t < DT; ++t)
-#pragma unroll
-          for (int blk = 0; blk < 2; ++blk) {
-            const bf16x8 va = __builtin_bit_cast(bf16x8, Vs[(blk * 4 + lq) * D + t * 16 + lr] & v_mask[blk]);
-            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[blk], o[t], 0, 0, 0);
-          }
-      } else {
-#pragma unroll
-        for (int t = 0; t < DT; ++t)
-#pragma unroll
-          for (int blk = 0; blk < 2; ++blk) {
-            const bf16x8 va = __builtin_bit_cast(bf16x8, Vs[(blk * 4 + lq) * D + t * 16 + lr]);
-            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[blk], o[t], 0, 0, 0);
-          }
-      }
     }
   }
 

@@ -110,6 +110,16 @@ class _Request:
     def feed(self) -> list[int]:
         return self.prompt + self.outputs
 
+    def next_tokens(self, count: int) -> list[int]:
+        """The next ``count`` tokens that go into the model: what follows ``fed`` in prompt +
+        outputs, without building that list (a decoding request asks for one token a step)."""
+        start, prompt = self.fed, self.prompt
+        if start >= len(prompt):
+            return self.outputs[start - len(prompt):start - len(prompt) + count]
+        if start + count <= len(prompt):
+            return prompt[start:start + count]
+        return prompt[start:] + self.outputs[:start + count - len(prompt)]
+
     def remaining(self) -> int:
         return len(self.prompt) + len(self.outputs) - self.fed
 
@@ -274,9 +284,8 @@ class ConcurrentGenerationEngine:
                 return events
             entries, wanted = [], []
             for request, count in selected:
-                feed = request.feed()
-                tokens = feed[request.fed:request.fed + count]
-                complete = request.fed + count == len(feed)
+                tokens = request.next_tokens(count)
+                complete = count == request.remaining()
                 entries.append(StepEntry(request.request_id, tokens, [count - 1] if complete else []))
                 if complete:
                     wanted.append(request)

@@ -31,7 +31,9 @@ def _hash_of(library: ctypes.CDLL) -> str | None:
 
 
 def _try_open(path: Path, expected: str) -> ctypes.CDLL | None:
-    if not path.exists():
+    # A stale library must not be opened at all: the loader keeps a handle per path name, so a
+    # library rebuilt at the same path afterwards would still resolve to the stale code.
+    if not path.exists() or expected.encode() not in path.read_bytes():
         return None
     try:
         library = ctypes.CDLL(str(path))
