@@ -172,11 +172,20 @@ def main() -> int:
         return [begin.elapsed_time(end) for begin, end in events], wall * 1e3
 
     def measured_read_bandwidth() -> float:
-        """Bytes a second of a plain streaming read (a sum over 1 GB that no cache holds)."""
-        data = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
-        times, _ = timed(lambda: data.sum(), 3, 10)
+        """Bytes a second of a plain streaming read: twenty sums over 800 MB that no cache holds,
+        between one pair of device events."""
+        data = torch.empty(200_000_000, dtype=torch.float32, device=device).normal_()
+        for _ in range(3):
+            data.sum()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        for _ in range(20):
+            data.sum()
+        end.record()
+        torch.cuda.synchronize()
+        seconds = begin.elapsed_time(end) * 1e-3 / 20
         del data
-        return (1 << 30) / (spread(times)["median"] * 1e-3)
+        return 800_000_000 / seconds
 
     read_peak = measured_read_bandwidth()
     model = random_model(config, args.seed, dtype=dtype, device=device)
