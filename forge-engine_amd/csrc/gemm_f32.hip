@@ -3,7 +3,8 @@
 // Plain FMA on the vector ALU, float32 accumulation in a fixed K order that
 // does not depend on M: no matrix-core instruction, so no reduced-precision
 // mode can slip in.  64x64 output tile per block of 256 threads, K in steps
-// of 16 through LDS; any M, N, K.
+// of 16 through LDS; any M, N, K.  Up to 16 rows of A with K a multiple of four take a
+// weight-streaming variant (below) instead.
 #include "common.h"
 
 #define TILE_M 64
@@ -90,11 +91,90 @@ __global__ __launch_bounds__(256) void gemm_nt_f32_kernel(
   }
 }
 
+// The same product for up to 16 rows of A (a decode step), where the work is reading B once:
+// a block takes R rows of B and MR rows of A; its four waves split K in interleaved steps of
+// 256 (a lane reads 16 contiguous bytes of every row, a wave 1 KB), each lane keeps R x MR
+// sums over its own k, the sums meet by a butterfly over the lanes and then over the waves in
+// LDS, in a fixed order.  The order of a row's sum depends on K alone: not on M, not on the
+// rows beside it, not on R or MR.  Needs K % 4 == 0 and 16-byte aligned rows.
+template <int MR, int R>
+__global__ __launch_bounds__(256) void gemm_rows_f32_kernel(
+    const float* __restrict__ A, const float* __restrict__ B, const float* __restrict__ bias,
+    float* __restrict__ C, int M, int N, int K, long long lda, long long ldb, long long ldc) {
+  __shared__ float red[4][R * MR];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * R, m0 = blockIdx.y * MR;
+  const float* arow[MR];
+  const float* brow[R];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) arow[m] = A + (size_t)min(m0 + m, M - 1) * lda;     // rows beyond M: the last again, never stored
+#pragma unroll
+  for (int r = 0; r < R; ++r) brow[r] = B + (size_t)min(n0 + r, N - 1) * ldb;
+  float acc[R][MR];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
+
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  int k = (wave * 64 + lane) * 4;
+  float4 bnext[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) bnext[r] = k < K ? *(const float4*)(brow[r] + k) : zero;
+  for (; k < K; k += 1024) {
+    float4 bv[R], av[MR];
+#pragma unroll
+    for (int r = 0; r < R; ++r) bv[r] = bnext[r];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) av[m] = *(const float4*)(arow[m] + k);
+    const int kn = k + 1024;                       // the next step's rows of B fly during this step's sums
+#pragma unroll
+    for (int r = 0; r < R; ++r) bnext[r] = kn < K ? *(const float4*)(brow[r] + kn) : zero;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MR; ++m) {
+        float s = acc[r][m];
+        s = fmaf(av[m].x, bv[r].x, s);
+        s = fmaf(av[m].y, bv[r].y, s);
+        s = fmaf(av[m].z, bv[r].z, s);
+        s = fmaf(av[m].w, bv[r].w, s);
+        acc[r][m] = s;
+      }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const float total = wave_sum(acc[r][m]);
+      if (lane == 0) red[wave][r * MR + m] = total;
+    }
+  __syncthreads();
+  if (tid < R * MR) {
+    const int r = tid / MR, m = tid - r * MR;
+    const int n = n0 + r, row = m0 + m;
+    if (n < N && row < M) {
+      const float total = ((red[0][tid] + red[1][tid]) + red[2][tid]) + red[3][tid];
+      C[(size_t)row * ldc + n] = total + (bias ? bias[n] : 0.f);
+    }
+  }
+}
+
+#define FE_ROWS_F32_MAX 16     // most rows of A that the weight-streaming variant takes
+
 extern "C" int fe_gemm_nt_f32(const float* A, const float* B, const float* bias, float* C,
                               int M, int N, int K, long long lda, long long ldb, long long ldc,
                               hipStream_t stream) {
   if (M <= 0 || N <= 0) return FE_OK;
   if (K <= 0 || lda < K || ldb < K || ldc < N) return FE_BAD_ARGUMENT;
+  const bool rows_ok = M <= FE_ROWS_F32_MAX && K % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 &&
+                       ((((uintptr_t)A) | ((uintptr_t)B)) & 15) == 0;
+  if (rows_ok) {
+    if (M <= 4) gemm_rows_f32_kernel<4, 8><<<dim3((N + 7) / 8, 1), 256, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
+    else if (M <= 8) gemm_rows_f32_kernel<8, 8><<<dim3((N + 7) / 8, 1), 256, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
+    else gemm_rows_f32_kernel<16, 4><<<dim3((N + 3) / 4, 1), 256, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
+    return fe_check_launch();
+  }
   const long long grid_y = (M + TILE_M - 1) / TILE_M;
   if (grid_y > 65535) return FE_BAD_ARGUMENT;
   dim3 grid((N + TILE_N - 1) / TILE_N, (unsigned)grid_y);
