@@ -456,6 +456,20 @@ def decode_splits(num_decode: int, kv_heads: int, max_ctx: int) -> int:
     return max(1, min(want, most, 64))
 
 
+GENERIC_TARGET_BLOCKS = 512    # blocks the general attention kernel aims at before it stops cutting the keys into runs
+
+
+def generic_splits(num_seqs: int, kv_heads: int, groups: int, max_q_len: int, head_dim: int, max_ctx: int | None) -> int:
+    """Runs that the general attention kernel cuts every row's keys into: 1 when the step already
+    fills the chip or the context is not known, else enough for about GENERIC_TARGET_BLOCKS
+    blocks, each with at least four of the kernel's key tiles."""
+    if max_ctx is None:
+        return 1
+    blocks = -(-max(1, max_q_len) * groups // 16) * kv_heads * num_seqs
+    key_tile = 64 if head_dim <= 64 else (32 if head_dim <= 128 else 16)
+    return max(1, min(-(-GENERIC_TARGET_BLOCKS // blocks), max_ctx // (4 * key_tile), 64))
+
+
 def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tensor, cu_q: Tensor,
                     ctx_len: Tensor, block_table: Tensor, *, num_seqs: int, max_q_len: int,
                     q_heads: int, kv_heads: int, head_dim: int, scale: float,
@@ -484,8 +498,8 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
         raise KernelError(f"out must be [{tokens}, {q_heads * head_dim}], got {tuple(out.shape)}")
     if q_heads % kv_heads:
         raise KernelError("query heads must be a multiple of kv heads")
-    if head_dim % 16 or not 16 <= head_dim <= 256:
-        raise KernelError(f"head size {head_dim} is not a multiple of 16 in [16, 256]")
+    if head_dim % 2 or not 2 <= head_dim <= 256:
+        raise KernelError(f"head size {head_dim} is not an even number in [2, 256]")
     if key_pages.dim() != 4 or key_pages.shape[1] != kv_heads or key_pages.shape[3] != head_dim:
         raise KernelError(f"pages must be [blocks, {kv_heads}, block_size, {head_dim}], got {tuple(key_pages.shape)}")
     if value_pages.shape != (key_pages.shape[0], kv_heads, head_dim, key_pages.shape[2]):
@@ -494,8 +508,6 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
         raise KernelError("cu_q, ctx_len and block_table do not match the number of sequences")
     if block_table.dim() != 2 or block_table.stride(1) != 1:
         raise KernelError("block_table must be [sequences, max_blocks] with unit inner stride")
-    if q.data_ptr() % 16 or (q.stride(0) if tokens > 1 else 0) % 8:
-        raise KernelError("q rows must be 16-byte aligned")
     num_blocks, _, block_size, _ = key_pages.shape
     groups = q_heads // kv_heads
     q_stride = q.stride(0) if tokens > 1 else q.shape[1]
@@ -503,17 +515,24 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
         any_single, any_longer, num_decode = True, max_q_len > 1, num_seqs
     else:
         any_single, any_longer = num_decode > 0, num_decode < num_seqs
-    bf16_pages = q.dtype == torch.bfloat16 and block_size >= 16 and block_size & (block_size - 1) == 0
+    bf16_pages = (q.dtype == torch.bfloat16 and block_size >= 16 and block_size & (block_size - 1) == 0
+                  and q.data_ptr() % 16 == 0 and q_stride % 8 == 0)      # the fast kernels read 16 bytes at a time
     fast_decode = bf16_pages and head_dim in (64, 128, 256) and groups <= 8
     fast_prefill = bf16_pages and head_dim in (64, 128)
 
     def general(min_q: int, max_q: int) -> None:
+        runs = generic_splits(num_seqs, kv_heads, groups, min(max_q, max_q_len), head_dim, max_ctx)
+        part_acc = part_ml = None
+        if runs > 1:
+            part_acc = torch.empty((runs, tokens, q_heads * head_dim), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((runs, tokens, q_heads, 2), dtype=torch.float32, device=q.device)
         _call("attention_generic", "fe_paged_attention_generic", _ptr(q), c_longlong(q_stride),
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)),
               c_int(_code(q.dtype)), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table),
               c_int(block_table.stride(0)), c_int(num_seqs), c_int(max_q_len), c_int(kv_heads),
               c_int(groups), c_int(head_dim), c_int(block_size), c_int(num_blocks),
-              c_int(window or 0), c_float(scale), c_int(min_q), c_int(max_q), _stream())
+              c_int(window or 0), c_float(scale), c_int(min_q), c_int(max_q), c_int(runs), _ptr(part_acc),
+              _ptr(part_ml), c_int(tokens), _stream())
 
     if any_single and fast_decode:
         if splits is None:

@@ -28,8 +28,8 @@ class GroupedQueryAttention(Mixer):
         super().__init__(ctx, prefix)
         if num_heads % num_kv_heads:
             raise ValueError("query heads must be a multiple of kv heads")
-        if head_dim % 16 or not 16 <= head_dim <= 256:
-            raise ValueError(f"head size {head_dim} is not supported: multiples of 16 from 16 to 256")
+        if head_dim % 2 or not 2 <= head_dim <= 256:
+            raise ValueError(f"head size {head_dim} is not supported: even sizes from 2 to 256")
         self.hidden_size = hidden_size
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads

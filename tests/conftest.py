@@ -52,6 +52,13 @@ TINY_C = _qwen3(
     max_position_embeddings=512, rms_norm_eps=1e-6, rope_theta=5000000.0,
     tie_word_embeddings=True,
 )
+# the tiny configuration of the reference's own model tests (tests/test_qwen3.py:12-28): heads of 4
+TINY_R = _qwen3(
+    vocab_size=32, hidden_size=8, intermediate_size=16, num_hidden_layers=2,
+    num_attention_heads=2, num_key_value_heads=1, head_dim=4,
+    max_position_embeddings=64, rms_norm_eps=1e-6, rope_theta=10000.0,
+    tie_word_embeddings=True, eos_token_id=2,
+)
 TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 BLOCK_SIZE = {"A": 4, "B": 8, "C": 16}
 

@@ -252,6 +252,49 @@ def test_paged_attention_mixed_batch(ops, dtype, q_heads, kv_heads, head_dim, bl
     torch.testing.assert_close(got, want, **tol(dtype))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [
+    (2, 1, 4, 2), (3, 3, 6, 4), (4, 2, 10, 16), (6, 2, 24, 8), (5, 1, 72, 16), (2, 2, 200, 16), (9, 3, 2, 5),
+])
+def test_paged_attention_any_even_head_size(ops, dtype, q_heads, kv_heads, head_dim, block_size):
+    """Head sizes that are no multiple of 16 (the reference's own tiny test model has heads of 4)
+    and rows that are not 16-byte aligned: the general kernel takes them one element at a time."""
+    g = torch.Generator().manual_seed(11)
+    seqs = [(0, 19), (33, 1), (7, 5), (0, 1), (64, 2)]
+    case = _attention_case(g, dtype, seqs, q_heads, kv_heads, head_dim, block_size, extra_width=2 * kv_heads * head_dim)
+    got, want = _run_attention(ops, *case, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim)
+    torch.testing.assert_close(got, want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [(32, 8, 128, 16), (4, 2, 16, 4), (6, 2, 48, 8), (3, 1, 256, 32)])
+def test_paged_attention_general_kernel_cuts_long_contexts_into_runs(ops, dtype, q_heads, kv_heads, head_dim, block_size, monkeypatch):
+    """Few sequences with long contexts: the general kernel cuts every row's keys into runs walked
+    by blocks of their own and merges them; any number of runs gives the plain result (runs that
+    hold no tile included), with a window too."""
+    g = torch.Generator().manual_seed(12)
+    seqs = [(700, 1), (0, 1), (1023, 1), (130, 3)]
+    q, kp, vp, cu, ctx, table = _attention_case(g, dtype, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                extra_width=2 * kv_heads * head_dim)
+    if dtype == torch.bfloat16:
+        q = q[:, :q_heads * head_dim + 1][:, :q_heads * head_dim]      # rows 2 bytes off 16-byte alignment: not a case for the fast kernels
+    for window in (None, 100):
+        kw = dict(num_seqs=len(seqs), max_q_len=3, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+                  scale=head_dim ** -0.5, window=window)
+        want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype), cu, ctx, table, **kw).float()
+        seen = []
+        for runs in (1, 2, 5, 64):
+            monkeypatch.setattr(ops, "generic_splits", lambda *a, runs=runs: seen.append(runs) or runs)
+            got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV),
+                                      torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
+                                      cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=None, max_ctx=1024, **kw).cpu().float()
+            torch.testing.assert_close(got, want, **tol(dtype))
+        assert seen == [1, 2, 5, 64] or dtype == torch.bfloat16
+    monkeypatch.undo()
+    assert ops.generic_splits(8, 8, 4, 1, 128, 1040) == 8 and ops.generic_splits(64, 8, 4, 1, 128, 1040) == 1
+    assert ops.generic_splits(1, 1, 1, 1, 16, 100) == 1 and ops.generic_splits(1, 8, 4, 1, 128, None) == 1
+
+
 @pytest.mark.parametrize("window", [1, 5, 16, 40])
 def test_paged_attention_window(ops, window):
     g = torch.Generator().manual_seed(7)
@@ -355,14 +398,15 @@ def test_kernels_refuse_what_they_cannot_do(ops):
     from forge_engine_amd.kernels.ops import KernelError
     with pytest.raises(KernelError, match="GPU"):
         ops.swiglu(torch.zeros(2, 8), torch.zeros(2, 4))
-    q = torch.zeros(1, 40, device=DEV)
-    pages = torch.zeros(2, 1, 4, 40, device=DEV)
-    with pytest.raises(KernelError, match="head size"):
-        ops.paged_attention(q, pages, pages, torch.zeros(1, 40, device=DEV),
-                            torch.tensor([0, 1], dtype=torch.int32, device=DEV),
-                            torch.tensor([1], dtype=torch.int32, device=DEV),
-                            torch.zeros(1, 1, dtype=torch.int32, device=DEV), num_seqs=1, max_q_len=1,
-                            q_heads=1, kv_heads=1, head_dim=40, scale=1.0)
+    for head_dim in (5, 258):       # odd, or beyond the largest head
+        q = torch.zeros(1, head_dim, device=DEV)
+        pages = torch.zeros(2, 1, 4, head_dim, device=DEV)
+        with pytest.raises(KernelError, match="head size"):
+            ops.paged_attention(q, pages, pages.transpose(2, 3).contiguous(), torch.zeros(1, head_dim, device=DEV),
+                                torch.tensor([0, 1], dtype=torch.int32, device=DEV),
+                                torch.tensor([1], dtype=torch.int32, device=DEV),
+                                torch.zeros(1, 1, dtype=torch.int32, device=DEV), num_seqs=1, max_q_len=1,
+                                q_heads=1, kv_heads=1, head_dim=head_dim, scale=1.0)
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 17, 33, 64])

@@ -66,6 +66,19 @@ def test_replay_matches_plain(name, mode, dtype, folders, plain_cache, tmp_path)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", list(TRACES))
+def test_replay_of_the_reference_tiny_configuration(mode, dtype, tmp_path):
+    """The configuration of the reference's own model tests: two query heads of four elements over
+    one kv head, a width of eight (every product and head size below the kernels' vector widths)."""
+    from conftest import TINY_R
+    folder = tmp_path / "model"
+    write_random_model(load_model_config(TINY_R), 77, folder)
+    requests = ru.make_requests(TINY_R, 5, (3, 7, 30, 61, 12))
+    got = ru.run_trace(folder, dtype, TRACES[mode](requests), tmp_path / "out", block_size=2)
+    ru.compare(got, ru.plain_logits(folder, requests), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_mixed_replay_reuses_pages(dtype, folders, plain_cache, tmp_path):
     requests = ru.make_requests(TINY["B"], 4, (30, 50, 20, 64, 33, 12, 41, 90, 5))
     trace = ru.trace_mixed(requests, 9, max_live=4)
@@ -143,7 +156,7 @@ def _drawn_configuration(seed: int):
         "vocab_size": rng.choice([97, 256, 300, 1003, 2049]), "hidden_size": rng.choice([40, 64, 72, 136, 200, 264]),
         "intermediate_size": rng.choice([48, 128, 136, 328, 520]), "num_hidden_layers": rng.choice([1, 2, 3]),
         "num_attention_heads": kv * groups, "num_key_value_heads": kv,
-        "head_dim": rng.choice([16, 32, 48, 64, 64, 80, 96, 128, 128, 160, 256]),
+        "head_dim": rng.choice([16, 32, 48, 64, 64, 80, 96, 128, 128, 160, 256]) if seed < 100 else rng.choice([2, 4, 6, 10, 12, 20, 36, 100]),
         "max_position_embeddings": 512, "rms_norm_eps": rng.choice([1e-6, 1e-5, 1e-3]),
         "rope_theta": rng.choice([10000.0, 1e6, 5e6]), "tie_word_embeddings": rng.choice([True, False]),
         "attention_bias": rng.choice([False, False, True]), "eos_token_id": None,
@@ -153,7 +166,7 @@ def _drawn_configuration(seed: int):
     return config, block_size, lengths
 
 
-@pytest.mark.parametrize("seed", [1, 6, 12, 13, 24, 47, 74])
+@pytest.mark.parametrize("seed", [1, 6, 12, 13, 24, 47, 74, 101, 102, 103])      # from 100 on: head sizes that are no multiple of 16
 def test_replay_of_drawn_configurations(seed, tmp_path):
     """Configurations nobody chose by hand, every way of cutting, both dtypes."""
     config, block_size, lengths = _drawn_configuration(seed)
