@@ -124,34 +124,39 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
   const int tiles_per_split = (tile_last - tile_first + splits - 1) / splits;
   const int my_first = tile_first + split * tiles_per_split;
   const int my_last = min(tile_last, my_first + tiles_per_split);
+  __shared__ int page_s[TK], slot_s[TK];   // where each key of the tile lives: page (-1: not read) and slot in it
   for (int kt = my_first * TK; kt < my_last * TK; kt += TK) {
     __syncthreads();  // previous tile consumed (and Q visible on the first pass)
+    if (tid < TK) {   // one division and one look at the table per key, not per element
+      const int kp = kt + tid;
+      int block = -1;
+      if (kp >= k_begin && kp < k_end) {
+        block = table[kp / block_size];
+        if (block >= num_blocks) block = -1;
+      }
+      page_s[tid] = block;
+      slot_s[tid] = kp % block_size;
+    }
+    __syncthreads();
     for (int e = tid; e < TK * chunks; e += 256) {
       const int kk = e / chunks;
       const int d4 = (e - kk * chunks) * 4;
-      const int kp = kt + kk;
-      float kv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (kp >= k_begin && kp < k_end) {
-        const int block = table[kp / block_size];
-        if (block >= 0 && block < num_blocks)
-          load4(key_pages + (((size_t)block * kv_heads + hk) * block_size + (kp % block_size)) * D + d4, vec, D - d4, kv);
-      }
+      // every load is unconditional (a key that is not read takes page 0 and its value is dropped):
+      // a load under a per-thread condition is a branch, and a thread's loads would wait for one another
+      const int block = page_s[kk];
+      float kv[4];
+      load4(key_pages + (((size_t)max(block, 0) * kv_heads + hk) * block_size + slot_s[kk]) * D + d4, vec, D - d4, kv);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (d4 + i < D) Ks[kk * kstride + d4 + i] = kv[i];
+        if (d4 + i < D) Ks[kk * kstride + d4 + i] = block >= 0 ? kv[i] : 0.f;
     }
     // values live transposed in their pages ([D][slot]): consecutive threads take consecutive keys
     for (int e = tid; e < TK * D; e += 256) {
       const int d = e / TK;
       const int kk = e - d * TK;
-      const int kp = kt + kk;
-      float v = 0.f;
-      if (kp >= k_begin && kp < k_end) {
-        const int block = table[kp / block_size];
-        if (block >= 0 && block < num_blocks)
-          v = load_as_float(value_pages + (((size_t)block * kv_heads + hk) * D + d) * block_size + (kp % block_size));
-      }
-      Vs[kk * kstride + d] = v;
+      const int block = page_s[kk];
+      const float v = load_as_float(value_pages + (((size_t)max(block, 0) * kv_heads + hk) * D + d) * block_size + slot_s[kk]);
+      Vs[kk * kstride + d] = block >= 0 ? v : 0.f;
     }
     __syncthreads();
 
@@ -159,6 +164,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
 #pragma unroll
     for (int i = 0; i < KPT; ++i) s[i] = 0.f;
     const float* qrow = Qs + r * kstride;
+#pragma unroll 8
     for (int d = 0; d < D; ++d) {
       const float qv = qrow[d];
 #pragma unroll
@@ -199,6 +205,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
 #pragma unroll
     for (int i = 0; i < DPT; ++i) acc[i] *= corr;
     const float* prow = Ps + r * TK;
+#pragma unroll 4
     for (int kk = 0; kk < TK; ++kk) {
       const float p = prow[kk];
       const float* vrow = Vs + kk * kstride;

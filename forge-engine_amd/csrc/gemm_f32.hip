@@ -116,20 +116,22 @@ __global__ __launch_bounds__(256) void gemm_rows_f32_kernel(
 #pragma unroll
     for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
 
-  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  // Loads are unconditional (a load under a per-lane condition becomes a branch, and where
+  // branches meet every load in flight is waited for): a step beyond K reads the row's last
+  // four elements again and is never used, because the loop ends first.
   int k = (wave * 64 + lane) * 4;
   float4 bnext[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) bnext[r] = k < K ? *(const float4*)(brow[r] + k) : zero;
+  for (int r = 0; r < R; ++r) bnext[r] = *(const float4*)(brow[r] + min(k, K - 4));
   for (; k < K; k += 1024) {
     float4 bv[R], av[MR];
 #pragma unroll
     for (int r = 0; r < R; ++r) bv[r] = bnext[r];
 #pragma unroll
     for (int m = 0; m < MR; ++m) av[m] = *(const float4*)(arow[m] + k);
-    const int kn = k + 1024;                       // the next step's rows of B fly during this step's sums
+    const int kn = min(k + 1024, K - 4);           // the next step's rows of B fly during this step's sums
 #pragma unroll
-    for (int r = 0; r < R; ++r) bnext[r] = kn < K ? *(const float4*)(brow[r] + kn) : zero;
+    for (int r = 0; r < R; ++r) bnext[r] = *(const float4*)(brow[r] + kn);
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -171,7 +173,7 @@ extern "C" int fe_gemm_nt_f32(const float* A, const float* B, const float* bias,
                        ((((uintptr_t)A) | ((uintptr_t)B)) & 15) == 0;
   if (rows_ok) {
     if (M <= 4) gemm_rows_f32_kernel<4, 8><<<dim3((N + 7) / 8, 1), 256, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
-    else if (M <= 8) gemm_rows_f32_kernel<8, 8><<<dim3((N + 7) / 8, 1), 256, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
+    else if (M <= 8) gemm_rows_f32_kernel<8, 4><<<dim3((N + 3) / 4, 1), 256, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);   // measured: four rows of B a block beat eight (more waves in flight)
     else gemm_rows_f32_kernel<16, 4><<<dim3((N + 3) / 4, 1), 256, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
     return fe_check_launch();
   }
