@@ -193,20 +193,23 @@ static int launch_skinny(const SkinnyCall& c) {
   return fe_check_launch();
 }
 
-// Resident variant for weights with many row tiles and K up to 4096: a launch has at most
+// Resident variant for weights with many row tiles and K up to 6144: a launch has at most
 // RESIDENT_BLOCKS blocks, each takes tiles blockIdx.x, blockIdx.x + gridDim.x, ... and reads its
 // slices of x ONCE into registers for all of them.  Reading x again for every 16 weight rows
 // costs a third of the speed at 8 rows of x although it comes from the L2 cache (measured on
 // MI355X: 4.4 against 6.2 TB/s for the 778 MB of a 151936 x 2560 head).  The sums are formed in
 // the same order as in the kernel above, so both give the same bits.
+// K beyond 4096 (up to 6144) takes blocks of 16 waves instead of 8, so that a wave holds at most
+// three steps of x: 256 such blocks, one a CU.
 #define RESIDENT_BLOCKS 512
 #define RESIDENT_WAVES 8
+#define RESIDENT_WAVES_WIDE 16
+#define RESIDENT_MAX_STEPS (3 * RESIDENT_WAVES_WIDE)    // three steps a wave: four would spill at 16 waves a block
 
-template <int EPI, int XS>
-__global__ __launch_bounds__(RESIDENT_WAVES * 64) void gemm_skinny_resident_kernel(
+template <int EPI, int XS, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
     int K, long long ldw, long long ldo, int second_offset, int tiles) {
-  constexpr int WAVES = RESIDENT_WAVES;
   constexpr int HALVES = EPI == EPI_SWIGLU ? 2 : 1;
   __shared__ __attribute__((aligned(16))) float red[HALVES][WAVES][64][4];
 
@@ -285,22 +288,27 @@ __global__ __launch_bounds__(RESIDENT_WAVES * 64) void gemm_skinny_resident_kern
 
 static bool resident_fits(int M, int N, int K) {
   const int steps = (K + KSTEP - 1) / KSTEP;
-  return M <= 16 && steps <= 4 * RESIDENT_WAVES && (N + ROWS - 1) / ROWS > RESIDENT_BLOCKS;
+  return M <= 16 && steps <= RESIDENT_MAX_STEPS && (N + ROWS - 1) / ROWS > RESIDENT_BLOCKS;
 }
 
 template <int EPI>
 static int launch_resident(const void* x, const void* w, void* out, int M, int N, int K, long long ldw,
                            long long ldo, int second_offset, hipStream_t stream) {
   const int tiles = (N + ROWS - 1) / ROWS;
-  const int blocks = tiles < RESIDENT_BLOCKS ? tiles : RESIDENT_BLOCKS;
-  const int xs = ((K + KSTEP - 1) / KSTEP + RESIDENT_WAVES - 1) / RESIDENT_WAVES;
-#define FE_GO(XS)                                                                                   \
-  gemm_skinny_resident_kernel<EPI, XS><<<blocks, RESIDENT_WAVES * 64, 0, stream>>>(                   \
+  const int steps = (K + KSTEP - 1) / KSTEP;
+  const bool wide = steps > 4 * RESIDENT_WAVES;
+  const int waves = wide ? RESIDENT_WAVES_WIDE : RESIDENT_WAVES;
+  const int most = wide ? RESIDENT_BLOCKS / 2 : RESIDENT_BLOCKS;
+  const int blocks = tiles < most ? tiles : most;
+  const int xs = (steps + waves - 1) / waves;
+#define FE_GO(XS, WV)                                                                               \
+  gemm_skinny_resident_kernel<EPI, XS, WV><<<blocks, WV * 64, 0, stream>>>(                          \
       (const bf16_t*)x, (const bf16_t*)w, out, M, N, K, ldw, ldo, second_offset, tiles)
-  if (xs <= 1) FE_GO(1);
-  else if (xs == 2) FE_GO(2);
-  else if (xs == 3) FE_GO(3);
-  else FE_GO(4);
+  if (wide) FE_GO(3, RESIDENT_WAVES_WIDE);
+  else if (xs <= 1) FE_GO(1, RESIDENT_WAVES);
+  else if (xs == 2) FE_GO(2, RESIDENT_WAVES);
+  else if (xs == 3) FE_GO(3, RESIDENT_WAVES);
+  else FE_GO(4, RESIDENT_WAVES);
 #undef FE_GO
   return fe_check_launch();
 }
@@ -369,7 +377,7 @@ extern "C" int fe_gemm_skinny(const void* x, const void* w, void* out, int M, in
   const int steps = (K + KSTEP - 1) / KSTEP;
   const int weight_rows = epilogue == EPI_SWIGLU ? 2 * N : N;
   if (tiles == -1 || (tiles == 0 && waves == 0 && splits == 1 && resident_fits(M, N, K))) {
-    if (M > 16 || steps > 4 * RESIDENT_WAVES || splits != 1) return FE_BAD_ARGUMENT;
+    if (M > 16 || steps > RESIDENT_MAX_STEPS || splits != 1) return FE_BAD_ARGUMENT;
     if (epilogue == EPI_SWIGLU) return launch_resident<EPI_SWIGLU>(x, w, out, M, N, K, ldw, ldo, N, stream);
     if (epilogue == EPI_F32) return launch_resident<EPI_F32>(x, w, out, M, N, K, ldw, ldo, 0, stream);
     return launch_resident<EPI_BF16>(x, w, out, M, N, K, ldw, ldo, 0, stream);

@@ -150,6 +150,8 @@ static void launch_add_rmsnorm_typed(float* h, const TD* delta, const float* w, 
   const bool aligned = hidden % 4 == 0 && part_stride % 4 == 0 && (((uintptr_t)h | (uintptr_t)delta | (uintptr_t)w | (uintptr_t)out) & 15) == 0;
   if (aligned && n_rows <= 512 && hidden > 1024 && hidden <= 4096)   // up to a few hundred rows: a whole row in flight at once
     add_rmsnorm_regs_kernel<TD, TO, 1, 1024><<<n_rows, 1024, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
+  else if (aligned && n_rows <= 512 && hidden > 4096 && hidden <= 8192)
+    add_rmsnorm_regs_kernel<TD, TO, 2, 1024><<<n_rows, 1024, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
   else if (aligned && hidden <= 1024)
     add_rmsnorm_regs_kernel<TD, TO, 1, 256><<<n_rows, 256, 0, stream>>>(h, delta, w, out, rows, hidden, eps, store_sum, parts, part_stride);
   else if (aligned && hidden <= 4096)

@@ -248,7 +248,7 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
 # six parts), of equal length, summed by blocks of four waves, take 6.9 instead of 9.0 us and 13.1
 # instead of 18.4 us at 8 rows.  The consumer (add_rmsnorm, add_rows) adds the parts in order; more
 # parts make the product no faster and the norm slower (3.1 us behind three parts, 3.8 behind eight).
-UPDATE_SPLIT_MAX_TILES = 256
+UPDATE_SPLIT_MAX_TILES = 384       # hidden sizes up to 6144 (160 tiles at 2560, 320 at 5120: both measured)
 UPDATE_SPLIT_MIN_STEPS = 32
 UPDATE_SPLIT_STEPS = 12        # 128-steps a part: fewer, longer parts cost the product little and save the norm reads
 UPDATE_SPLIT_MAX = 16

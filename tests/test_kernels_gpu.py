@@ -43,7 +43,7 @@ def test_embed_rows(ops, dtype, hidden):
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("delta_dtype", [None, torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("hidden", [24, 200, 2560, 5000])
+@pytest.mark.parametrize("hidden", [24, 200, 2560, 5000, 5120, 8192])
 @pytest.mark.parametrize("n", [7, 23, 600])     # up to 512 rows of a wide stream take a kernel with more threads a row
 def test_add_rmsnorm(ops, out_dtype, delta_dtype, hidden, n):
     g = torch.Generator().manual_seed(1)
@@ -445,24 +445,26 @@ def test_gemm_skinny_swiglu(ops, m, inter, k):
 
 
 @pytest.mark.parametrize("m", [1, 5, 16])
-@pytest.mark.parametrize("n,k", [(8200, 264), (9003, 1000), (8209, 2560), (8195, 4096)])
+@pytest.mark.parametrize("n,k", [(8200, 264), (9003, 1000), (8209, 2560), (8195, 4096), (8200, 5120), (8209, 6144), (8195, 4104)])
 def test_gemm_skinny_resident(ops, m, n, k):
     """Weights with more than 512 row tiles take the variant whose blocks stay and keep x in
-    registers: same bits as the one-tile-per-block kernel, also for the gated product."""
+    registers: same bits as the one-tile-per-block kernel with as many waves a block (8 up to
+    K = 4096, 16 beyond), also for the gated product."""
     g = torch.Generator().manual_seed(23)
     x = rand(g, m, k, dtype=torch.bfloat16).to(DEV)
     w = rand(g, n, k, dtype=torch.bfloat16, scale=0.05).to(DEV)
     want = x.float().cpu() @ w.float().cpu().T
-    plain = ops.gemm_skinny(x, w, "f32", tiles=1, waves=8).cpu()
+    waves = 8 if k <= 4096 else 16
+    plain = ops.gemm_skinny(x, w, "f32", tiles=1, waves=waves).cpu()
     bound = 2e-6 * float(want.abs().max()) * math.sqrt(k) + 1e-6
     assert float((plain - want).abs().max()) <= bound
     assert torch.equal(ops.gemm_skinny(x, w, "f32", tiles=-1).cpu(), plain)
     assert torch.equal(ops.gemm_skinny(x, w, "f32").cpu(), plain)
-    assert torch.equal(ops.gemm_skinny(x, w, "bf16").cpu(), ops.gemm_skinny(x, w, "bf16", tiles=1, waves=8).cpu())
+    assert torch.equal(ops.gemm_skinny(x, w, "bf16").cpu(), ops.gemm_skinny(x, w, "bf16", tiles=1, waves=waves).cpu())
     if n % 2:
         w = w[:n - 1]
     gated = ops.gemm_skinny(x, w, "swiglu", tiles=-1).cpu()
-    assert torch.equal(gated, ops.gemm_skinny(x, w, "swiglu", tiles=1, waves=8).cpu())
+    assert torch.equal(gated, ops.gemm_skinny(x, w, "swiglu", tiles=1, waves=waves).cpu())
     want = refs.linear_swiglu(x.cpu(), w.cpu()).float()
     torch.testing.assert_close(gated.float(), want, atol=1e-2 * float(want.abs().max()) + 1e-6, rtol=1e-2)
 
@@ -473,8 +475,8 @@ def test_gemm_skinny_resident_refuses(ops):
     w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(KernelError):
         ops.gemm_skinny(x, w, "f32", tiles=-1)          # more than 16 rows
-    x = torch.zeros(4, 4104, dtype=torch.bfloat16, device=DEV)
-    w = torch.zeros(64, 4104, dtype=torch.bfloat16, device=DEV)
+    x = torch.zeros(4, 6152, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 6152, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(KernelError):
         ops.gemm_skinny(x, w, "f32", tiles=-1)          # K beyond what the registers hold
 
