@@ -172,20 +172,23 @@ def main() -> int:
         return [begin.elapsed_time(end) for begin, end in events], wall * 1e3
 
     def measured_read_bandwidth() -> float:
-        """Bytes a second of a plain streaming read: twenty sums over 800 MB that no cache holds,
-        between one pair of device events."""
-        data = torch.empty(200_000_000, dtype=torch.float32, device=device).normal_()
-        for _ in range(3):
-            data.sum()
+        """Bytes a second of a plain streaming read: a kernel that only reads, over four 400 MB
+        buffers in turn so that no cache holds what it reads, twenty times between one pair of
+        device events."""
+        from forge_engine_amd.kernels import ops
+
+        buffers = [torch.zeros(100_000_000, dtype=torch.float32, device=device) for _ in range(4)]
+        sink = torch.zeros(1, dtype=torch.float32, device=device)
+        for data in buffers:
+            ops.stream_read(data, sink)
         begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         begin.record()
-        for _ in range(20):
-            data.sum()
+        for index in range(20):
+            ops.stream_read(buffers[index % 4], sink)
         end.record()
         torch.cuda.synchronize()
         seconds = begin.elapsed_time(end) * 1e-3 / 20
-        del data
-        return 800_000_000 / seconds
+        return 400_000_000 / seconds
 
     read_peak = measured_read_bandwidth()
     model = random_model(config, args.seed, dtype=dtype, device=device)

@@ -277,3 +277,23 @@ extern "C" int fe_swiglu(const void* gate_up, void* out, int dtype, int tokens, 
     return FE_BAD_ARGUMENT;
   return fe_check_launch();
 }
+
+// A plain streaming read of `bytes` bytes (a multiple of 16), for measuring what the memory
+// delivers to a kernel that does nothing else: every block walks the buffer in 16-byte pieces,
+// 2048 blocks of 256 threads.  sink[0] is written only if the data add up to a value they never
+// have, so the loads cannot be dropped.
+__global__ __launch_bounds__(256) void stream_read_kernel(const float4* __restrict__ data, size_t pieces, float* sink) {
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < pieces; i += (size_t)gridDim.x * 256) {
+    const float4 v = data[i];
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  if (s.x + s.y + s.z + s.w == 123456.789f) sink[0] = s.x;
+}
+
+extern "C" int fe_stream_read(const void* data, long long bytes, float* sink, hipStream_t stream) {
+  if (bytes <= 0) return FE_OK;
+  if (bytes % 16 || (((uintptr_t)data) & 15) || !sink) return FE_BAD_ARGUMENT;
+  stream_read_kernel<<<2048, 256, 0, stream>>>((const float4*)data, (size_t)(bytes / 16), sink);
+  return fe_check_launch();
+}

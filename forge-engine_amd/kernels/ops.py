@@ -142,6 +142,17 @@ def swiglu(gate_up: Tensor, out: Tensor) -> Tensor:
     return out
 
 
+def stream_read(data: Tensor, sink: Tensor) -> None:
+    """Read every byte of ``data`` once and do nothing else (a measurement of what the memory
+    delivers); ``sink`` is one float32 that is never really written."""
+    _gpu(data, "data")
+    _gpu(sink, "sink", torch.float32)
+    size = data.numel() * data.element_size()
+    if size % 16:
+        raise KernelError("the buffer's size must be a multiple of 16 bytes")
+    _call("rowwise", "fe_stream_read", _ptr(data), c_longlong(size), _ptr(sink), _stream())
+
+
 # ------------------------------------------------------------ matrix products
 
 def gemm_nt_f32(a: Tensor, b: Tensor, bias: Tensor | None = None, out: Tensor | None = None) -> Tensor:

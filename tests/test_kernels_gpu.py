@@ -96,6 +96,16 @@ def test_add_rmsnorm_row_list(ops):
         assert torch.equal(h_dev.cpu(), h)
 
 
+def test_stream_read_touches_nothing(ops):
+    data = torch.arange(4096, dtype=torch.float32, device=DEV)
+    sink = torch.full((1,), 7.0, device=DEV)
+    ops.stream_read(data, sink)
+    torch.cuda.synchronize()
+    assert sink.item() == 7.0 and torch.equal(data.cpu(), torch.arange(4096, dtype=torch.float32))
+    with pytest.raises(ops.KernelError):
+        ops.stream_read(data[:3], sink)              # not a multiple of 16 bytes
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_add_rows_and_swiglu(ops, dtype):
     g = torch.Generator().manual_seed(3)
