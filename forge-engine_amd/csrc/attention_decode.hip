@@ -258,8 +258,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
       s[j] = (key >= k_begin && key < cached) ? v : -INFINITY;
       mx = fmaxf(mx, s[j]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, FE_WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, FE_WAVE));
+    mx = max_xor16(mx);
+    mx = max_xor32(mx);
     const float m_new = fmaxf(m_run, mx);
     const float m_use = m_new > -INFINITY ? m_new : 0.f;
     const float corr = __builtin_amdgcn_exp2f(m_run - m_use);
@@ -269,8 +269,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
       s[j] = __builtin_amdgcn_exp2f(s[j] - m_use);
       sum += s[j];
     }
-    sum += __shfl_xor(sum, 16, FE_WAVE);
-    sum += __shfl_xor(sum, 32, FE_WAVE);
+    sum = sum_xor16(sum);
+    sum = sum_xor32(sum);
     l_run = l_run * corr + sum;
     m_run = m_new;
     uintx4 pw;
@@ -350,8 +350,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
         for (int c = 0; c < KC; ++c) total[c] = next[c];
       }
       float sumsq = total[0];
-      sumsq += __shfl_xor(sumsq, 32, FE_WAVE);
-      sumsq += __shfl_xor(sumsq, 16, FE_WAVE);
+      sumsq = sum_xor32(sumsq);
+      sumsq = sum_xor16(sumsq);
       const float inv = inverse_rms(sumsq, D, prep.eps);
 #pragma unroll
       for (int c = 0; c < KC; ++c) {
@@ -446,8 +446,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void paged_decode_kernel(
 #pragma unroll
         for (int e = 0; e < 8; ++e) dot = __fmaf_rn(qf[e], kf[e], dot);
       }
-      dot += __shfl_xor(dot, 16, FE_WAVE);
-      dot += __shfl_xor(dot, 32, FE_WAVE);
+      dot = sum_xor16(dot);
+      dot = sum_xor32(dot);
       if (lq == 0 && lr < groups) { Ms[WAVES][lr] = dot * scale_log2; Ls[WAVES][lr] = 1.f; }
     }
   }

@@ -3,6 +3,11 @@
 //
 // Block = 64 query tokens of one query head of one sequence, four waves of 16
 // rows; keys and values are walked in tiles of 64, shared by the waves in LDS.
+// Long walks take blocks of eight waves (KG = 2): two groups of four waves with
+// LDS buffers of their own walk every other tile each and merge their results
+// at the end, which halves the chain of dependent tiles that the longest block
+// of a launch is (one prompt of 2,048 tokens: all blocks are resident at once
+// and the one with 32 tiles sets the time).
 //   S^T = K Q^T    MFMA 16x16x32, A = 16 keys from LDS, B = 16 query rows held
 //                  in registers for the whole kernel.  The 32 keys of a block
 //                  feed two MFMA tiles whose rows interleave in groups of four,
@@ -70,8 +75,8 @@ __device__ __forceinline__ void load_to_lds(const void* global, void* lds) {
                                    (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
 }
 
-template <int D>
-__global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
+template <int D, int KG>
+__global__ __launch_bounds__(256 * KG, 4) void paged_prefill_kernel(   // four waves a SIMD: at most 128 registers
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
@@ -84,8 +89,7 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
   constexpr int CH = D / 8;             // 16-byte chunks per key row
   constexpr int KI = BN * CH / 256;     // key load instructions per wave and tile
   constexpr int VI = 8 * D / 256;       // value load instructions per wave and tile
-  __shared__ __attribute__((aligned(16))) uintx4 Ks[BN * CH];
-  __shared__ __attribute__((aligned(16))) uintx4 Vs[8 * D];
+  __shared__ __attribute__((aligned(16))) uintx4 lds[KG * (BN * CH + 8 * D)];   // per key group: a tile of keys, a tile of values
 
   // Block id b runs on XCD b % 8.  An XCD, with its own L2, takes a run of neighbouring (sequence,
   // head) pairs, which share keys and values; within the XCD the blocks are ordered by row tile,
@@ -108,7 +112,10 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
   const int* table = block_table + (size_t)seq * table_stride;
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kg = __builtin_amdgcn_readfirstlane(tid >> 8);          // key group: walks tiles tile_first + kg, + KG, ...
+  const int wave = __builtin_amdgcn_readfirstlane((tid >> 6) & 3);  // within the group: 16 rows, a quarter of the loads
+  uintx4* Ks = lds + kg * (BN * CH + 8 * D);
+  uintx4* Vs = Ks + BN * CH;
   const int lr = lane & 15, lq = lane >> 4;
   const int krow = 8 * (lr >> 2) + (lr & 3);   // MFMA row r of key tile h is key 8*(r/4) + 4h + r%4 of its 32-key block
 
@@ -160,8 +167,25 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
     v_dim[i] = u % D;
     v_first[i] = (u / D) * 8;         // first key of the chunk within the tile
   }
+  // A tile that lies wholly inside [first visible key's group, context) needs no clamping: the
+  // address of a load is then a part that is uniform over the wave (page, kv head, where the wave's
+  // 16 keys start in the page; scalar arithmetic) plus a part that never changes (the lane's place
+  // among those 16 keys), so the tiles of the steady state cost no vector instructions for their
+  // addresses.  The tiles at the edges take the general path.
+  unsigned int k_lane[KI], v_lane[VI];
+#pragma unroll
+  for (int i = 0; i < KI; ++i) k_lane[i] = (unsigned int)((k_row[i] & 15) * D + k_chunk[i] * 8);
+#pragma unroll
+  for (int i = 0; i < VI; ++i) v_lane[i] = (unsigned int)((v_dim[i] << block_shift) + (v_first[i] & 15));
+  auto inner = [&](int tile) -> bool { return tile * BN + BN <= ctx && tile * BN >= low_group; };
   auto load_keys = [&](int tile, int page) {
     const size_t base = ((size_t)page * kv_heads + hk) << block_shift;
+    if (inner(tile)) {
+      const bf16_t* from = key_pages + (base + ((tile * BN + 16 * wave) & block_mask)) * D;
+#pragma unroll
+      for (int i = 0; i < KI; ++i) load_to_lds(from + k_lane[i], &Ks[(wave * KI + i) * 64]);
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < KI; ++i) {
       const int key = min(tile * BN + k_row[i], last_key);
@@ -170,6 +194,12 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
   };
   auto load_values = [&](int tile, int page) {
     const size_t base = ((size_t)page * kv_heads + hk) * D;
+    if (inner(tile)) {
+      const bf16_t* from = value_pages + (base << block_shift) + ((tile * BN + 16 * wave) & block_mask);
+#pragma unroll
+      for (int i = 0; i < VI; ++i) load_to_lds(from + v_lane[i], &Vs[(wave * VI + i) * 64]);
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < VI; ++i) {
       const int key = max(min(tile * BN + v_first[i], last_key & ~7), low_chunk);
@@ -177,15 +207,20 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
     }
   };
 
-  int page = page_of(tile_first);
-  load_keys(tile_first, page);
-  int page_next = tile_first < tile_last ? page_of(tile_first + 1) : 0;
+  // every group makes the same number of rounds (the barriers are the block's); a group without a
+  // tile in a round only waits
+  const int rounds = (tile_last - tile_first + KG) / KG;
+  int tile = tile_first + kg;
+  int page = page_of(min(tile, tile_last));
+  if (tile <= tile_last) load_keys(tile, page);
+  int page_next = tile + KG <= tile_last ? page_of(tile + KG) : 0;
   FE_WAIT_VMEM(0);
   __syncthreads();               // the first tile's keys are in LDS
-  for (int tile = tile_first; tile <= tile_last; ++tile) {
-    const bool more = tile < tile_last;
+  for (int round = 0; round < rounds; ++round, tile += KG) {
+    const bool active = tile <= tile_last;
+    const bool more = tile + KG <= tile_last;
     const int key_base = tile * BN;
-    const bool mine = key_base <= wave_lo + 15;     // some key of the tile is visible to this wave's rows
+    const bool mine = active && key_base <= wave_lo + 15;     // some key of the tile is visible to this wave's rows
     floatx4 st[2][2];
     if (mine) {
 #pragma unroll
@@ -203,11 +238,11 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
     // Every wave has its scores, and multiplied the tile before: both buffers are free.  This
     // tile's values and the next tile's keys are requested now and fly during the softmax.
     __syncthreads();
-    load_values(tile, page);
+    if (active) load_values(tile, page);
     if (more) {
-      load_keys(tile + 1, page_next);
+      load_keys(tile + KG, page_next);
       page = page_next;
-      if (tile + 2 <= tile_last) page_next = page_of(tile + 2);
+      if (tile + 2 * KG <= tile_last) page_next = page_of(tile + 2 * KG);
     }
     bf16x8 pb[2];
     if (mine) {
@@ -226,8 +261,8 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
         s[j] = v;
         mx = fmaxf(mx, v);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, FE_WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, FE_WAVE));
+      mx = max_xor16(mx);
+      mx = max_xor32(mx);
       const float m_new = fmaxf(m_run, mx * scale_log2);   // the scale is positive
       const float m_use = m_new > -INFINITY ? m_new : 0.f; // a row with nothing visible yet
       const float corr = __builtin_amdgcn_exp2f(m_run - m_use);
@@ -237,8 +272,8 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
         s[j] = __builtin_amdgcn_exp2f(fmaf(s[j], scale_log2, -m_use));
         sum += s[j];
       }
-      sum += __shfl_xor(sum, 16, FE_WAVE);
-      sum += __shfl_xor(sum, 32, FE_WAVE);
+      sum = sum_xor16(sum);
+      sum = sum_xor32(sum);
       l_run = l_run * corr + sum;
       m_run = m_new;
 #pragma unroll
@@ -256,7 +291,7 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
       }
     }
     FE_WAIT_VMEM(0);
-    if (__builtin_expect(key_base + BN > ctx || key_base < k_first, 0)) {
+    if (__builtin_expect(active && (key_base + BN > ctx || key_base < k_first), 0)) {
       // The tile holds slots at or beyond the context (the 8-key chunk of the last key has them
       // behind it; later chunks are copies of that chunk) or below the first visible key.  Their
       // probabilities are zero, but a slot that no live key owns may hold anything (a NaN that
@@ -290,6 +325,33 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
     }
   }
 
+  if constexpr (KG == 2) {
+    // the second group hands its running maximum, sum and output to the first through LDS (the
+    // tiles' buffers are free now), value by value with the lanes side by side
+    __syncthreads();
+    float* hand = (float*)lds;
+    const int slot = wave * 64 + lane;
+    if (kg == 1) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) hand[(t * 4 + i) * 256 + slot] = o[t][i];
+      hand[(DT * 4) * 256 + slot] = m_run;
+      hand[(DT * 4 + 1) * 256 + slot] = l_run;
+    }
+    __syncthreads();
+    if (kg == 1) return;
+    const float m_other = hand[(DT * 4) * 256 + slot], l_other = hand[(DT * 4 + 1) * 256 + slot];
+    const float m_all = fmaxf(m_run, m_other);
+    const float f_mine = m_run > -INFINITY ? __builtin_amdgcn_exp2f(m_run - m_all) : 0.f;
+    const float f_other = m_other > -INFINITY ? __builtin_amdgcn_exp2f(m_other - m_all) : 0.f;
+    l_run = l_run * f_mine + l_other * f_other;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[t][i] = o[t][i] * f_mine + hand[(t * 4 + i) * 256 + slot] * f_other;
+  }
+
   // lane (lr = query row, lq) holds O^T[16t + 4lq + i][row]: four consecutive dims per store
   if (row < q_len) {
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
@@ -306,13 +368,13 @@ __global__ __launch_bounds__(256, 4) void paged_prefill_kernel(
 
 // Pages: keys [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size];
 // block_size a power of two >= 16; head_dim 64 or 128.  Sequences with fewer than two query tokens
-// are skipped.
+// are skipped.  max_ctx_hint: an upper bound of the sequences' contexts if the caller knows one, else 0.
 extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, const void* key_pages,
                                                  const void* value_pages, void* out, long long out_stride,
                                                  const int* cu_q, const int* ctx_len, const int* block_table,
                                                  int table_stride, int num_seqs, int max_q_len, int kv_heads,
                                                  int groups, int head_dim, int block_size, int num_blocks,
-                                                 int window, float scale, hipStream_t stream) {
+                                                 int window, float scale, int max_ctx_hint, hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len < 2) return FE_OK;
   if (head_dim != 64 && head_dim != 128) return FE_BAD_ARGUMENT;
   if (groups < 1 || kv_heads < 1 || num_seqs > 65535) return FE_BAD_ARGUMENT;
@@ -326,12 +388,17 @@ extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, con
   const long long per_xcd = (pairs + XCDS - 1) / XCDS;
   if (per_xcd * XCDS * q_tiles > 0x7fffffffLL) return FE_BAD_ARGUMENT;
   const unsigned grid = (unsigned)(per_xcd * XCDS * q_tiles);
-#define FE_GO(DD)                                                                                                \
-  paged_prefill_kernel<DD><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
+  // two key groups a block where walks are long: portions of 256 tokens or more, or portions of a
+  // whole tile behind a context that the caller knows to be long
+  const int key_groups = (max_q_len >= 256 || (max_q_len >= 64 && max_ctx_hint >= 2048)) ? 2 : 1;
+#define FE_GO(DD, GG)                                                                                            \
+  paged_prefill_kernel<DD, GG><<<grid, 256 * GG, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,            \
       kv_heads, groups, block_shift, num_blocks, window, scale_log2, q_tiles, (int)pairs, (int)per_xcd)
-  if (head_dim == 64) FE_GO(64);
-  else FE_GO(128);
+  if (head_dim == 64 && key_groups == 1) FE_GO(64, 1);
+  else if (head_dim == 64) FE_GO(64, 2);
+  else if (key_groups == 1) FE_GO(128, 1);
+  else FE_GO(128, 2);
 #undef FE_GO
   return fe_check_launch();
 }

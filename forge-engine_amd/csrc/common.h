@@ -34,6 +34,29 @@ __device__ __forceinline__ float load_as_float(const bf16_t* p) { return bf16_to
 __device__ __forceinline__ void store_from_float(float* p, float v) { *p = v; }
 __device__ __forceinline__ void store_from_float(bf16_t* p, float v) { *p = float_to_bf16(v); }
 
+// This lane's value combined with that of lane ^ 16 or lane ^ 32 by the lane-swap instructions
+// of gfx950 (vector ALU, no trip through the LDS crossbar, which a general shuffle takes with a
+// wait behind it).  permlane16_swap(a, b) exchanges the odd rows of 16 lanes of a with the even
+// rows of b, permlane32_swap the upper half of a with the lower half of b; with a = b = v the two
+// results hold, in every lane, the values of both partners.  The sums have the same bits in both
+// partners and the same bits as v + shuffle(v).
+__device__ __forceinline__ float sum_xor16(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float sum_xor32(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float max_xor16(float v) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_xor32(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int offset = FE_WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, FE_WAVE);

@@ -563,7 +563,7 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
               _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
               c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), c_float(scale), _stream())
+              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(max_ctx or 0), _stream())
     # whatever the two fast kernels did not take goes to the general kernel
     single_left = any_single and not fast_decode
     longer_left = any_longer and not fast_prefill

@@ -976,6 +976,28 @@ def test_prefill_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size):
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("window", [None, 100, 700])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [(8, 2, 128, 16), (6, 3, 64, 32)])
+def test_prefill_attention_kernel_long_walks(ops, q_heads, kv_heads, head_dim, block_size, window):
+    """Long portions and long contexts take blocks of two key groups that walk every other tile
+    and merge at the end: walks of one tile (the second group idle), of an odd and an even number
+    of tiles, behind a long context, beside single tokens; with unowned slots poisoned."""
+    g = torch.Generator().manual_seed(45)
+    seqs = [(0, 300), (500, 257), (70, 1), (3, 2), (1000, 64), (0, 64), (61, 67)]
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                extra_width=2 * kv_heads * head_dim)
+    kw = dict(num_seqs=len(seqs), max_q_len=300, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+              scale=head_dim ** -0.5, window=window)
+    want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype), cu, ctx, table, **kw).float()
+    first = [0 if window is None else max(0, before - window + 1) for before, _ in seqs]
+    _poison_unowned_slots(kp, vp, table, first, [b + n for b, n in seqs], block_size)
+    got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV),
+                              torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
+                              cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=1, max_ctx=2048, **kw).cpu().float()
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("window", [1, 7, 64, 100])
 def test_prefill_attention_kernel_window(ops, window):
     g = torch.Generator().manual_seed(41)
