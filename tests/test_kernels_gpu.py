@@ -978,10 +978,13 @@ def test_prefill_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size):
 
 @pytest.mark.parametrize("window", [None, 100, 700])
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [(8, 2, 128, 16), (6, 3, 64, 32)])
-def test_prefill_attention_kernel_long_walks(ops, q_heads, kv_heads, head_dim, block_size, window):
-    """Long portions and long contexts take blocks of two key groups that walk every other tile
-    and merge at the end: walks of one tile (the second group idle), of an odd and an even number
-    of tiles, behind a long context, beside single tokens; with unowned slots poisoned."""
+@pytest.mark.parametrize("key_groups", [1, 2])
+def test_prefill_attention_kernel_long_walks(ops, q_heads, kv_heads, head_dim, block_size, window, key_groups, monkeypatch):
+    """Launches that leave the chip underfilled take blocks of two key groups that walk every
+    other tile and merge at the end: walks of one tile (the second group idle), of an odd and an
+    even number of tiles, behind a long context, beside single tokens; with unowned slots
+    poisoned.  Both kinds of block, forced in turn."""
+    monkeypatch.setattr(ops, "PREFILL_KEY_GROUPS", key_groups)
     g = torch.Generator().manual_seed(45)
     seqs = [(0, 300), (500, 257), (70, 1), (3, 2), (1000, 64), (0, 64), (61, 67)]
     q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
