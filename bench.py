@@ -8,8 +8,10 @@ for the benchmark context, and prints ONE JSON line: decoded tokens a second
 at batch 8 (``value``), the same at batch 1 and 64 (``points``), the prefill of
 one 2,048-token prompt, and the decode step's memory roofline.  A "step" is one
 decode step: every request's last token through the model, and the next token
-sampled (greedy) and read back.  Everything goes through the engine's own step
-function, cache and kernels.
+sampled (greedy) and read back.  The sampled tokens are fed to the next step on
+the device and read by the host while that step runs (``--no-overlap`` reads
+them before the next step is launched).  Everything goes through the engine's
+own step function, cache and kernels.
 
 Protocol (after tools/validate_l4.py:136-183 of the reference): W untimed steps,
 then K steps each bracketed by a pair of device events; the line reports their
@@ -95,6 +97,8 @@ def parse_args():
     parser.add_argument("--prompt-range", default="128,4096", help="mixed workload: prompt lengths, uniform")
     parser.add_argument("--new-tokens", type=int, default=256, help="mixed workload: tokens generated per request")
     parser.add_argument("--token-budget", type=int, default=2048, help="scheduler: tokens a step")
+    parser.add_argument("--no-overlap", dest="overlap", action="store_false",
+                        help="read every step's tokens back before the next step is launched")
     parser.add_argument("--seed", type=int, default=0)
     args = parser.parse_args()
     chosen = MODELS[args.model]
@@ -267,7 +271,20 @@ def main() -> int:
             for n, t in zip(names, tokens):
                 state[n] = t
 
-        times, wall = timed(one_step, args.warmup, args.steps)
+        # The sampled tokens go into the next step on the device, and the host reads them while
+        # that step runs (a step late): the GPU does not wait for the host between two steps.
+        placeholders = [StepEntry(n, [0], [0]) for n in names]
+        flight = {"feed": torch.tensor([state[n] for n in names], dtype=torch.int32, device=device), "unread": None}
+
+        def one_overlapped_step():
+            logits = runner.step(placeholders, device_tokens=flight["feed"])
+            both = sampler.sample_greedy_on_device(logits)
+            if flight["unread"] is not None:
+                sampler.read(flight["unread"])
+            flight["unread"], flight["feed"] = both, both[0]
+
+        overlapped = args.overlap and runner.feeds_from_device(placeholders)
+        times, wall = timed(one_overlapped_step if overlapped else one_step, args.warmup, args.steps)
         contexts = [runner.length(n) for n in names]
         for name in names:
             runner.end(name)

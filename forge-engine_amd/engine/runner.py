@@ -256,14 +256,21 @@ class ModelRunner:
         return (self.use_graphs and len(entries) <= GRAPH_MAX_REQUESTS
                 and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
 
-    def _graph_step(self, entries: list[StepEntry]) -> Tensor:
+    def _graph_step(self, entries: list[StepEntry], device_tokens: Tensor | None = None) -> Tensor:
         """A decode-only step (one token and one wanted row per request) as a
         replay of a captured HIP graph: the launches of a step cost more host
-        time than the step takes on the GPU."""
+        time than the step takes on the GPU.  With ``device_tokens`` (int32
+        [requests], on the device) the tokens of the entries are ignored and
+        those are fed instead, by a copy on the device: the host need not have
+        seen them yet."""
         cache = self.cache
         vocab = self.model.plan.vocab_size
         tokens = [e.tokens[0] for e in entries]
-        if min(tokens) < 0 or max(tokens) >= vocab:
+        if device_tokens is not None:
+            if device_tokens.dtype != torch.int32 or device_tokens.device != self.device or device_tokens.numel() < len(entries):
+                raise ValueError("device_tokens must be int32 on the runner's device, one per entry")
+            tokens = [0] * len(entries)
+        elif min(tokens) < 0 or max(tokens) >= vocab:
             raise ValueError(f"a token id is outside the vocabulary of {vocab}")
         steady = self._steady
         if (steady is not None and steady.room > 0 and len(entries) == len(steady.ids)
@@ -279,6 +286,8 @@ class ModelRunner:
             buf[4 * n + 1:6 * n + 1] += 1                    # ctx_len, ctx_before
             slot.dev.copy_(slot.host, non_blocking=True)
             slot.copied.record(torch.cuda.current_stream(self.device))
+            if device_tokens is not None:
+                slot.dev[0:n].copy_(device_tokens[0:n])
             slot.graph.replay()
             for record in steady.records:
                 record.length += 1
@@ -321,6 +330,8 @@ class ModelRunner:
             with torch.cuda.graph(graph):
                 slot.logits = self.model.forward(batch, views)
             slot.graph, slot.views, slot.batch = graph, views, batch
+        if device_tokens is not None:
+            slot.dev[0:len(entries)].copy_(device_tokens[0:len(entries)])
         slot.graph.replay()
         self.graph_replays += 1
         cache.commit_single_tokens(records)
@@ -403,14 +414,28 @@ class ModelRunner:
         return slot.logits[:sum(len(e.want) for e in entries)]
 
     @torch.inference_mode()
-    def step(self, entries: list[StepEntry]) -> Tensor:
+    def step(self, entries: list[StepEntry], device_tokens: Tensor | None = None) -> Tensor:
         """Run the entries' tokens as one batch; float32 logits [wanted, vocab]
         in the order of the entries and of each entry's ``want``.  Raises
         ``CacheCapacityError`` (and changes nothing) if pages run out.  The
         result of a step that replays a captured graph lives in a buffer that
-        the next step of the same shape overwrites."""
+        the next step of the same shape overwrites.
+
+        ``device_tokens`` (int32 [entries] on the device): for a step of single
+        tokens that replays a graph (``feeds_from_device``), the token of entry i
+        is ``device_tokens[i]`` whatever the entry holds, so that a step can be
+        launched before the host has read the tokens that the step before
+        sampled."""
         with ops.use_workspace(self.workspace):
+            if device_tokens is not None:
+                if not self._graphable(entries):
+                    raise ValueError("tokens are fed from the device only into steps of single tokens that replay a graph")
+                return self._graph_step(entries, device_tokens)
             return self._step(entries)
+
+    def feeds_from_device(self, entries: list[StepEntry]) -> bool:
+        """Whether ``step(entries, device_tokens=...)`` serves this step."""
+        return self._graphable(entries)
 
     def _step(self, entries: list[StepEntry]) -> Tensor:
         if self._graphable(entries):

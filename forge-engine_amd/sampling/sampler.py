@@ -59,6 +59,22 @@ class Sampler:
     def __init__(self, device: torch.device) -> None:
         self.device = device
 
+    def sample_greedy_on_device(self, logits: Tensor) -> Tensor:
+        """Arg-max of every row, left on the device: int32 [2, rows], the tokens and the rows'
+        status words.  Nothing is read back; ``read`` does that, whenever the host wants them
+        (a step later, if the tokens are fed to the next step on the device)."""
+        rows = logits.shape[0]
+        both = torch.empty((2, rows), dtype=torch.int32, device=self.device)
+        ops.argmax_rows(logits, both[0], both[1])
+        return both
+
+    @staticmethod
+    def read(both: Tensor) -> list[int]:
+        """The tokens of ``sample_greedy_on_device``, on the host; raises as ``sample`` does."""
+        host = both.cpu()
+        _raise_on_status(host[1].tolist())
+        return host[0].tolist()
+
     def sample(self, logits: Tensor, params: list[SamplingParams], seeds: list[int],
                draw_index: list[int]) -> list[int]:
         """One token per row.  ``seeds[r]`` and ``draw_index[r]`` (how many tokens

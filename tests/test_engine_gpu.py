@@ -179,6 +179,66 @@ def test_long_decoding_through_graphs_matches_eager_and_plain(dtype, folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tokens_fed_on_the_device_decode_like_tokens_from_the_host(dtype, folders):
+    """Greedy decoding of three requests where every step takes its tokens from the arg-max of
+    the step before without the host in between (it reads them a step late), across page edges
+    and a change of the batch: the same tokens and logits as decoding with host tokens."""
+    from forge_engine_amd.sampling.sampler import Sampler
+    name = "C"
+    config = TINY[name]
+    prompts = ru.make_requests(config, 83, (21, 9, 30))
+    _, model = load_model(folders[name], dtype=dtype, device=DEV)
+    sampler = Sampler(DEV)
+    outputs = {}
+    for mode in ("host", "device"):
+        runner = ModelRunner(model, block_size=16, block_capacity=24, num_state_slots=4)
+        last = {}
+        for k, tokens in prompts.items():
+            runner.begin(k)
+            last[k] = int(runner.step([StepEntry(k, tokens, [len(tokens) - 1])])[0].argmax())
+        names = list(prompts)
+        generated = {k: [last[k]] for k in names}
+        rows = []
+        if mode == "host":
+            for step in range(40):
+                if step == 25:
+                    names = names[:2]                      # one request leaves: another graph, other table rows
+                logits = runner.step([StepEntry(k, [generated[k][-1]], [0]) for k in names])
+                rows.append(logits.clone())
+                for k, t in zip(names, sampler.sample(logits, [SamplingParams()] * len(names), [0] * len(names), [0] * len(names))):
+                    generated[k].append(t)
+        else:
+            feed = torch.tensor([last[k] for k in names], dtype=torch.int32, device=DEV)
+            unread = []
+            for step in range(40):
+                if step == 25:
+                    names = names[:2]
+                    feed = feed[:2].contiguous()
+                entries = [StepEntry(k, [0], [0]) for k in names]
+                assert runner.feeds_from_device(entries)
+                logits = runner.step(entries, device_tokens=feed)
+                rows.append(logits.clone())
+                both = sampler.sample_greedy_on_device(logits)
+                unread.append((list(names), both))
+                feed = both[0]
+                if len(unread) > 1:                        # the host reads a step late
+                    ks, late = unread.pop(0)
+                    for k, t in zip(ks, sampler.read(late)):
+                        generated[k].append(t)
+            for ks, both in unread:
+                for k, t in zip(ks, sampler.read(both)):
+                    generated[k].append(t)
+            assert runner.graph_replays == 40
+            with pytest.raises(ValueError, match="single tokens"):
+                runner.step([StepEntry(names[0], [1, 2], [1])], device_tokens=feed)
+        outputs[mode] = (generated, torch.cat([r.flatten() for r in rows]).cpu())
+        for k in prompts:
+            runner.end(k)
+    assert outputs["host"][0] == outputs["device"][0]
+    assert torch.equal(outputs["host"][1], outputs["device"][1])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_steps_with_portions_replay_captured_graphs(name, dtype, folders):
     """A scheduler that fills its token budget repeats few step shapes; such steps (prompt portions
