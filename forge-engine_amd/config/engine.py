@@ -44,6 +44,7 @@ class SchedulerConfig:
     admission: str = "reserve"            # "reserve": worst-case pages at submit; "preempt": on demand
     max_context: int | None = None        # longest prompt + new tokens accepted (None: the pool's size)
     num_state_slots: int | None = None    # per-request state slots (None: max_requests)
+    overlap_decode: bool = True           # steady greedy decode steps take their tokens on the device; the host reads a step late
 
     def __post_init__(self) -> None:
         for name in ("max_requests", "max_batch_size", "token_budget", "block_size", "block_capacity"):

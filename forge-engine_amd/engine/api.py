@@ -58,12 +58,13 @@ def build_engine(model, *, engine_config: EngineConfig | None = None,
 
 def engine_from_folder(folder: str | Path, *, engine_config: EngineConfig | None = None,
                        scheduler_config: SchedulerConfig | None = None, dtype="bfloat16",
-                       device="cuda:0") -> ConcurrentGenerationEngine:
-    """config.json picks the model class, the safetensors files fill it."""
+                       device="cuda:0", eos_token_ids=None) -> ConcurrentGenerationEngine:
+    """config.json picks the model class, the safetensors files fill it.  ``eos_token_ids``
+    overrides the end-of-sequence tokens that config.json names."""
     device = require_gpu(device)
     _, model = load_model(folder, dtype=dtype, device=device)
     return build_engine(model, engine_config=engine_config, scheduler_config=scheduler_config,
-                        tokenizer=load_tokenizer(folder))
+                        tokenizer=load_tokenizer(folder), eos_token_ids=eos_token_ids)
 
 
 def engine_from_random(config: ModelConfig, seed: int, *, engine_config: EngineConfig | None = None,

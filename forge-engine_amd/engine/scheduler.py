@@ -11,6 +11,16 @@ and never splits a prompt; here every selected request contributes to one flat
 batch (portions of prompts beside single decoded tokens) and the token budget
 cuts prompts into portions.
 
+Overlapped decoding (``overlap_decode``).  While the same requests decode greedily step after
+step, a step is launched with the tokens that the step before sampled still on the device, and
+the host reads those tokens while the new step runs: the GPU does not wait for the scheduler
+between two steps.  What the host sees is one step late: events come a step later, and a
+request that samples its end-of-sequence token still rides in the step that was already
+launched (its result there is dropped).  A request that reaches its token limit is known in
+advance and never rides along.  Any other kind of step (a prompt portion, another set of
+requests, a sampled rather than greedy row) first reads what is in flight.  The tokens that
+requests generate are the same either way.
+
 When pages run out.  ``admission="reserve"`` (default, the reference's policy):
 a request is admitted only if the pages for its prompt plus ``max_new_tokens``
 are unreserved, so a running request can never run out; ``submit`` raises
@@ -106,6 +116,7 @@ class _Request:
     error: str | None = None
     reservation_released: bool = False
     holds_cache: bool = False
+    in_flight: bool = False                            # its last sampled token is still on the device, unread
 
     def feed(self) -> list[int]:
         return self.prompt + self.outputs
@@ -121,7 +132,7 @@ class _Request:
         return prompt[start:] + self.outputs[:start + count - len(prompt)]
 
     def remaining(self) -> int:
-        return len(self.prompt) + len(self.outputs) - self.fed
+        return len(self.prompt) + len(self.outputs) + (1 if self.in_flight else 0) - self.fed
 
 
 class ConcurrentGenerationEngine:
@@ -151,11 +162,14 @@ class ConcurrentGenerationEngine:
         self._preemptions = 0
         self._last_batch: tuple[str, ...] = ()
         self._last_tokens: tuple[int, ...] = ()
+        # the step whose sampled tokens the host has not read yet: (its requests, tokens and status on the device)
+        self._flight: tuple[list[_Request], object] | None = None
+        self.overlapped_steps = 0
 
     # ----------------------------------------------------------- properties
     @property
     def idle(self) -> bool:
-        return all(r.status.terminal for r in self._requests.values())
+        return self._flight is None and all(r.status.terminal for r in self._requests.values())
 
     @property
     def cache_pool(self):
@@ -272,11 +286,84 @@ class ConcurrentGenerationEngine:
         request.status = RequestStatus.WAITING
         self._preemptions += 1
 
+    # ------------------------------------------------- overlapped decode steps
+    def _land(self) -> list[StreamEvent]:
+        """Read the tokens of the step in flight and consume them."""
+        events: list[StreamEvent] = []
+        if self._flight is None:
+            return events
+        requests, both = self._flight
+        self._flight = None
+        try:
+            tokens = self._sampler.read(both)
+        except Exception as error:
+            for request in requests:
+                request.in_flight = False
+            events.extend(self._fail([r for r in requests if not r.status.terminal], error))
+            self._drop_terminal()
+            return events
+        for request, token in zip(requests, tokens):
+            request.in_flight = False
+            if not request.status.terminal:       # cancelled meanwhile, or ended in the step before: dropped
+                events.extend(self._consume(request, token))
+        self._drop_terminal()
+        return events
+
+    def _may_overlap(self, selected: list[tuple[_Request, int]]) -> bool:
+        """A step of single greedy tokens, every one the last of its request's history, none of
+        which ends its request by the token limit, that the runner can feed from the device."""
+        if not self._config.overlap_decode or not hasattr(self._sampler, "sample_greedy_on_device"):
+            return False
+        for request, count in selected:
+            if count != 1 or request.remaining() != 1 or not request.params.greedy:
+                return False
+            if request.sampled_tokens + (1 if request.in_flight else 0) + 1 > request.params.max_new_tokens:
+                return False
+        feeds = getattr(self._runner, "feeds_from_device", None)
+        return feeds is not None and feeds([StepEntry(r.request_id, [0], [0]) for r, _ in selected])
+
+    def _overlapped_step(self, selected: list[tuple[_Request, int]]) -> list[StreamEvent] | None:
+        """Launch the step on the tokens in flight (or, for the first of a run, on host tokens),
+        sample on the device, then read and consume the step before.  None if it cannot be done
+        (the caller then lands what is in flight and takes the plain path)."""
+        requests = [r for r, _ in selected]
+        if self._flight is not None:
+            flying, both = self._flight
+            if len(flying) != len(requests) or any(a is not b for a, b in zip(flying, requests)):
+                return None
+            entries = [StepEntry(r.request_id, [0], [0]) for r in requests]
+            feed = both[0]
+        else:
+            entries = [StepEntry(r.request_id, r.next_tokens(1), [0]) for r in requests]
+            feed = None
+        try:
+            logits = self._runner.step(entries, device_tokens=feed) if feed is not None else self._runner.step(entries)
+            launched = self._sampler.sample_greedy_on_device(logits)
+        except Exception:
+            return None                             # nothing was changed: pages are reserved all or none
+        self._last_batch = tuple(r.request_id for r in requests)
+        self._last_tokens = tuple(1 for _ in requests)
+        events = self._land()                       # the step before, read while this one runs
+        for request in requests:
+            request.fed += 1
+            request.in_flight = True
+        self._flight = (requests, launched)
+        self.overlapped_steps += 1
+        return events
+
     def step(self) -> list[StreamEvent]:
         """One model step over a fresh batch; returns what it produced."""
         selected = self._select_batch()
         self._iteration += 1
         events: list[StreamEvent] = []
+        if selected and self._may_overlap(selected):
+            produced = self._overlapped_step(selected)
+            if produced is not None:
+                return produced
+        if self._flight is not None:
+            # another kind of step follows: first learn what the step in flight sampled, then choose again
+            events.extend(self._land())
+            selected = self._select_batch()
         while True:
             self._last_batch = tuple(r.request_id for r, _ in selected)
             self._last_tokens = tuple(n for _, n in selected)

@@ -103,6 +103,46 @@ def test_scheduler_under_page_pressure_on_the_gpu(name, folders):
         assert got == plain.greedy_generate(weights, config, prompt, n), request_id
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_overlapped_decode_steps_generate_the_same_tokens(dtype, folders):
+    """Steady greedy decode steps take their tokens on the device and the host reads a step late:
+    the same tokens, finish reasons and freed pages as with every step read back at once; with
+    requests that end on an end-of-sequence token (seen a step late), on their token limit (known
+    in advance), a request cancelled while its token is in flight, and a late joiner."""
+    name = "B"          # a head of its own: greedy tokens vary instead of falling into a loop at once
+    config = TINY[name]
+    prompts = list(ru.make_requests(config, 87, (12, 30, 7, 19, 25)).values())
+    limits = [9, 40, 40, 23, 31]
+    results = {}
+    for overlap in (False, True):
+        scheduler = SchedulerConfig(block_size=8, block_capacity=64, token_budget=64, max_batch_size=8,
+                                    overlap_decode=overlap)
+        engine = engine_from_folder(folders[name], scheduler_config=scheduler, dtype=dtype)
+        if not overlap:
+            # choose an end-of-sequence token that the second request really samples, a few tokens in
+            probe = engine.generate([prompts[1]], SamplingParams(max_new_tokens=24))[0]
+            at = next(j for j in range(3, len(probe)) if probe[j] not in probe[:j])    # first seen at place j >= 3
+            results["eos"], results["stop_after"] = probe[at], at
+        engine = engine_from_folder(folders[name], scheduler_config=scheduler, dtype=dtype, eos_token_ids=[results["eos"]])
+        ids = [engine.submit(p, sampling_params=SamplingParams(max_new_tokens=n)) for p, n in zip(prompts[:4], limits[:4])]
+        steps = 0
+        while not engine.idle:
+            engine.step()
+            steps += 1
+            if steps == 6:
+                ids.append(engine.submit(prompts[4], sampling_params=SamplingParams(max_new_tokens=limits[4])))   # joins late
+            if steps == 12:
+                engine.cancel(ids[2])
+        views = [engine.request(i) for i in ids]
+        results[overlap] = [(v.status.value, v.finish_reason, v.output_token_ids if i != 2 else None) for i, v in enumerate(views)]
+        assert engine.cache_pool.allocated_pages == 0
+        assert (engine.overlapped_steps > 8) == overlap
+        assert views[1].finish_reason == "stop" and len(views[1].output_token_ids) == results["stop_after"]   # the end token is not emitted
+        assert views[0].finish_reason == "length" and len(views[0].output_token_ids) == 9
+        assert views[2].status.value == "cancelled"
+    assert results[True] == results[False]
+
+
 def test_command_line_generates(folders, capsys):
     from forge_engine_amd.cli import main
     prompt = [5, 17, 3, 200, 9]
