@@ -482,6 +482,19 @@ def generic_splits(num_seqs: int, kv_heads: int, groups: int, max_q_len: int, he
     return max(1, min(-(-GENERIC_TARGET_BLOCKS // blocks), max_ctx // (4 * key_tile), 64))
 
 
+ROWS_TARGET_BLOCKS = 1024      # blocks the vector-ALU decode attention aims at (four resident a CU)
+
+
+def rows_splits(num_decode: int, kv_heads: int, groups: int, head_dim: int, max_ctx: int | None) -> int:
+    """Runs that the vector-ALU decode attention cuts every sequence's keys into: enough for about
+    ROWS_TARGET_BLOCKS blocks, each with at least two of the kernel's key tiles."""
+    if max_ctx is None:
+        return 1
+    blocks = -(-groups // (4 if groups <= 4 else 8)) * kv_heads * max(1, num_decode)
+    key_tile = 64 if head_dim <= 64 else (32 if head_dim <= 128 else 16)
+    return max(1, min(-(-ROWS_TARGET_BLOCKS // blocks), max_ctx // (2 * key_tile), 64))
+
+
 def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tensor, cu_q: Tensor,
                     ctx_len: Tensor, block_table: Tensor, *, num_seqs: int, max_q_len: int,
                     q_heads: int, kv_heads: int, head_dim: int, scale: float,
@@ -565,9 +578,26 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
               _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
               c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
               c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(PREFILL_KEY_GROUPS), _stream())
-    # whatever the two fast kernels did not take goes to the general kernel
+    # whatever the two fast kernels did not take: single tokens go to the vector-ALU decode kernel where
+    # it can read four elements at a time, the rest to the general kernel
     single_left = any_single and not fast_decode
     longer_left = any_longer and not fast_prefill
+    item = q.element_size()
+    if (single_left and head_dim % 4 == 0 and block_size % 4 == 0 and q_stride % 4 == 0
+            and q.data_ptr() % (4 * item) == 0 and key_pages.data_ptr() % (4 * item) == 0
+            and value_pages.data_ptr() % (4 * item) == 0):
+        runs = rows_splits(num_decode, kv_heads, groups, head_dim, max_ctx)
+        part_acc = part_ml = None
+        if runs > 1:
+            part_acc = torch.empty((runs, tokens, q_heads * head_dim), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((runs, tokens, q_heads, 2), dtype=torch.float32, device=q.device)
+        _call("attention_generic", "fe_paged_attention_rows", _ptr(q), c_longlong(q_stride),
+              _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)),
+              c_int(_code(q.dtype)), _ptr(cu_q), _ptr(ctx_len), _ptr(block_table),
+              c_int(block_table.stride(0)), c_int(num_seqs), c_int(kv_heads), c_int(groups), c_int(head_dim),
+              c_int(block_size), c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(runs),
+              _ptr(part_acc), _ptr(part_ml), c_int(tokens), _stream())
+        single_left = False
     if single_left or longer_left:
         general(1 if single_left else 2, max_q_len if longer_left else 1)
     return out

@@ -305,6 +305,50 @@ def test_paged_attention_general_kernel_cuts_long_contexts_into_runs(ops, dtype,
     assert ops.generic_splits(1, 1, 1, 1, 16, 100) == 1 and ops.generic_splits(1, 8, 4, 1, 128, None) == 1
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [
+    (32, 8, 128, 16), (4, 2, 16, 4), (6, 2, 36, 12), (5, 1, 100, 20), (12, 1, 64, 8), (3, 3, 4, 4), (16, 2, 200, 16), (9, 1, 256, 32),
+])
+def test_vector_alu_decode_attention(ops, dtype, q_heads, kv_heads, head_dim, block_size, monkeypatch):
+    """Single tokens whose shapes the matrix-core decode kernel does not take (float32; bfloat16 with
+    other head sizes, pages or groups) go to the kernel that keeps keys and values out of LDS: every
+    head size that is a multiple of four (16, 32 or 64 lanes a key), up to 4 or 8 heads a block and
+    more in row tiles, pages of any multiple of four slots, any number of key runs (runs without
+    keys included), a window, contexts at the edges of pages and tiles, and NaN in every slot that
+    no live key owns."""
+    g = torch.Generator().manual_seed(14)
+    seqs = [(700, 1), (0, 1), (1023, 1), (63, 1), (64, 1), (130, 3), (15, 1)]
+    q, kp, vp, cu, ctx, table = _attention_case(g, dtype, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                extra_width=2 * kv_heads * head_dim)
+    if dtype == torch.bfloat16 and head_dim in (64, 128, 256) and q_heads // kv_heads <= 8 and block_size >= 16:
+        block_size_ok = False     # the matrix-core kernel would take these: nothing to test here
+    else:
+        block_size_ok = True
+    taken = []
+    real_call = ops._call
+    monkeypatch.setattr(ops, "_call", lambda lib, name, *a: taken.append(name) or real_call(lib, name, *a))
+    for window in (None, 100):
+        kw = dict(num_seqs=len(seqs), max_q_len=3, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+                  scale=head_dim ** -0.5, window=window)
+        want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype), cu, ctx, table, **kw).float()
+        first = [0 if window is None else max(0, before - window + 1) for before, _ in seqs]
+        kp_bad, vp_bad, table_bad = kp.clone(), vp.clone(), table.clone()
+        _poison_unowned_slots(kp_bad, vp_bad, table, first, [b + n for b, n in seqs], block_size)
+        for s, low in enumerate(first):
+            table_bad[s, :low // block_size] = -1
+        for runs in (1, 2, 5, 64):
+            monkeypatch.setattr(ops, "rows_splits", lambda *a, runs=runs: runs)
+            got = ops.paged_attention(q.to(DEV), kp_bad.to(DEV), vp_bad.to(DEV),
+                                      torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
+                                      cu.to(DEV), ctx.to(DEV), table_bad.to(DEV), num_decode=None, max_ctx=1024, **kw).cpu().float()
+            assert torch.isfinite(got).all()
+            torch.testing.assert_close(got, want, **tol(dtype))
+    assert ("fe_paged_attention_rows" in taken) == block_size_ok
+    monkeypatch.undo()
+    assert ops.rows_splits(8, 8, 4, 128, 1040) == 16 and ops.rows_splits(64, 8, 4, 128, 1040) == 2
+    assert ops.rows_splits(1, 1, 1, 16, 100) == 1 and ops.rows_splits(1, 8, 4, 128, None) == 1
+
+
 @pytest.mark.parametrize("window", [1, 5, 16, 40])
 def test_paged_attention_window(ops, window):
     g = torch.Generator().manual_seed(7)
