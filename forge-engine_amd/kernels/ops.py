@@ -300,9 +300,12 @@ def gemm_mid_parts(x: Tensor, weight: Tensor, parts: int) -> Tensor:
     return out
 
 
-def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
+def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None, stream: Tensor | None = None) -> Tensor | None:
     """The float32 product x @ weight^T (+ bias) as an update of the residual stream: [M, N], or
-    partial sums [parts, M, N] that ``add_rmsnorm`` / ``add_rows`` add up."""
+    partial sums [parts, M, N] that ``add_rmsnorm`` / ``add_rows`` add up.  Given the float32
+    ``stream`` [M, N] itself, the matrix library's product (more than 64 rows) adds into it as it
+    stores, which saves the next norm the update's bytes, and None is returned: the same float32
+    sum in the same order, stream + (x @ weight^T)."""
     _gpu(x, "x")
     _gpu(weight, "weight", contiguous=False)
     plain_bf16 = bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
@@ -318,6 +321,10 @@ def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tens
         steps = -(-weight.shape[1] // 128)
         blocks = -(-weight.shape[0] // 64)
         return gemm_mid_parts(x, weight, _mid_parts(steps, blocks))
+    if (plain_bf16 and stream is not None and x.shape[0] > SKINNY_MAX_ROWS and stream.dtype == torch.float32
+            and stream.shape == (x.shape[0], weight.shape[0]) and stream.is_contiguous()):
+        torch.addmm(stream, x, weight.t(), out_dtype=torch.float32, out=stream)
+        return None
     return linear(x, weight, bias, out_dtype=torch.float32)
 
 

@@ -111,7 +111,10 @@ class GroupedQueryAttention(Mixer):
     def cache_needs(self) -> CacheNeeds:
         return CacheNeeds(paged=PagedKV(self.num_kv_heads, self.head_dim, self.window))
 
-    def forward(self, x: Tensor, batch, cache: CacheView, writes_cache: bool = True) -> Tensor:
+    takes_stream = True
+
+    def forward(self, x: Tensor, batch, cache: CacheView, writes_cache: bool = True,
+                stream: Tensor | None = None) -> Tensor | None:
         rotary = self.position.rotary()
         inv_freq, rotary_dim = rotary if rotary is not None else (None, 0)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 1.0
@@ -128,7 +131,7 @@ class GroupedQueryAttention(Mixer):
                     batch.cu_q, batch.ctx_len, cache.block_table, q_heads=self.num_heads,
                     kv_heads=self.num_kv_heads, head_dim=self.head_dim, eps=eps, scale=self.scale,
                     window=self.window, max_ctx=batch.max_ctx)
-                return ops.linear_update(attn, self.o_weight, self.o_bias)
+                return ops.linear_update(attn, self.o_weight, self.o_bias, stream)
             qkv = ops.linear(x, self.qkv_weight, self.qkv_bias)
         else:  # another call wrote the keys and values this one reads: only q is needed
             bias = None if self.qkv_bias is None else self.qkv_bias[:self.q_size]
@@ -144,7 +147,7 @@ class GroupedQueryAttention(Mixer):
             num_seqs=batch.num_seqs, max_q_len=batch.max_q_len, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
             num_decode=batch.num_decode, max_ctx=batch.max_ctx)
-        return ops.linear_update(attn, self.o_weight, self.o_bias)   # float32 update for the residual sum
+        return ops.linear_update(attn, self.o_weight, self.o_bias, stream)   # float32 update for the residual sum
 
     def _single_tokens_only(self, batch, x: Tensor, cache: CacheView, rotary_dim: int) -> bool:
         """Every sequence of the step brings one token, and the sizes are ones that the

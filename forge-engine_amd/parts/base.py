@@ -55,9 +55,14 @@ class Residual:
         self.h = h
         self.pending: Tensor | None = None
 
-    def add(self, update: Tensor) -> None:
+    def add(self, update: Tensor | None) -> None:
+        """Leave an update pending; None: the part has added it into the stream itself."""
         self.flush()
         self.pending = update
+
+    def open(self) -> Tensor:
+        """The stream with nothing pending, for a part that adds its update itself."""
+        return self.flush()
 
     def flush(self) -> Tensor:
         if self.pending is not None:
@@ -123,18 +128,23 @@ class PositionEncoding(Part):
 
 class Mixer(Part):
     role = "mixer"
+    # True for a part whose forward takes ``stream=`` (the float32 residual stream, nothing pending):
+    # it may add its update into the stream itself, where its last product can do so for free, and
+    # then returns None instead of the update.
+    takes_stream = False
 
     def cache_needs(self) -> CacheNeeds:
         return CacheNeeds()
 
-    def forward(self, x: Tensor, batch, cache: CacheView | None, writes_cache: bool = True) -> Tensor:
+    def forward(self, x: Tensor, batch, cache: CacheView | None, writes_cache: bool = True) -> Tensor | None:
         raise NotImplementedError
 
 
 class FeedForward(Part):
     role = "feed_forward"
+    takes_stream = False   # as for a mixer
 
-    def forward(self, x: Tensor, batch) -> Tensor:
+    def forward(self, x: Tensor, batch) -> Tensor | None:
         raise NotImplementedError
 
 

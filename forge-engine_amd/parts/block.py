@@ -10,15 +10,21 @@ from .base import Block, Residual
 class PreNormBlock(Block):
     """``h += mixer(norm_in(h)); h += ffn(norm_post(h))`` (reference:
     src/forge_engine/qwen3.py:240-261).  Each add is left pending on the stream
-    and fused into the next norm."""
+    and fused into the next norm, unless the part's last product added it itself."""
 
     NORMS = ("input", "post_mixer")
 
     def forward(self, residual: Residual, batch, cache: CacheView | None, writes_cache: bool = True) -> None:
         x = self.norms["input"].forward(residual)
-        residual.add(self.mixer.forward(x, batch, cache, writes_cache))
+        if self.mixer.takes_stream:
+            residual.add(self.mixer.forward(x, batch, cache, writes_cache, stream=residual.open()))
+        else:
+            residual.add(self.mixer.forward(x, batch, cache, writes_cache))
         y = self.norms["post_mixer"].forward(residual)
-        residual.add(self.feed_forward.forward(y, batch))
+        if self.feed_forward.takes_stream:
+            residual.add(self.feed_forward.forward(y, batch, stream=residual.open()))
+        else:
+            residual.add(self.feed_forward.forward(y, batch))
 
 
 register_part("block", "pre_norm", PreNormBlock)

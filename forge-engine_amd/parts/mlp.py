@@ -43,9 +43,11 @@ class SwiGLU(FeedForward):
         else:
             raise KeyError(name)
 
-    def forward(self, x: Tensor, batch=None) -> Tensor:
+    takes_stream = True
+
+    def forward(self, x: Tensor, batch=None, stream: Tensor | None = None) -> Tensor | None:
         act = ops.linear_swiglu(x, self.gate_up_weight)
-        return ops.linear_update(act, self.down_weight)   # the update stays float32 for the residual sum
+        return ops.linear_update(act, self.down_weight, stream=stream)   # the update stays float32 for the residual sum
 
     def kernel_libraries(self):
         return {"rowwise", "gemm_f32", "gemm_skinny", "gemm_mid"}

@@ -72,8 +72,8 @@ def linear_swiglu(x, gate_up_weight):
     return (g / (1.0 + torch.exp(-g)) * u).to(x.dtype)
 
 
-def linear_update(x, weight, bias=None):
-    return linear(x, weight, bias, out_dtype=torch.float32)
+def linear_update(x, weight, bias=None, stream=None):
+    return linear(x, weight, bias, out_dtype=torch.float32)    # the stream is left to the caller's add
 
 
 def gemm_skinny(x, weight, epilogue="bf16", tiles=0, waves=0, splits=1):

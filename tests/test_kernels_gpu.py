@@ -619,6 +619,25 @@ def test_gemm_mid_parts_refuses_a_k_that_is_no_multiple_of_its_step(ops):
     torch.testing.assert_close(update.cpu(), x.float().cpu() @ w.float().cpu().T, atol=1e-3, rtol=1e-3)
 
 
+def test_linear_update_adds_into_the_stream_where_the_library_multiplies(ops):
+    """More than 64 rows: the matrix library's product adds into the float32 stream as it stores and
+    nothing is left pending; the stream then holds exactly stream + product.  Fewer rows: the update
+    comes back (in parts) and the stream is left alone."""
+    g = torch.Generator().manual_seed(31)
+    for m, n, k in ((200, 320, 256), (65, 2560, 4096)):
+        x, w = rand(g, m, k, dtype=torch.bfloat16).to(DEV), rand(g, n, k, dtype=torch.bfloat16, scale=0.05).to(DEV)
+        stream = rand(g, m, n).to(DEV)
+        before = stream.clone()
+        assert ops.linear_update(x, w, None, stream) is None
+        want = before + ops.linear_update(x, w)
+        assert torch.equal(stream, want)
+        torch.testing.assert_close(stream.cpu(), before.cpu() + x.float().cpu() @ w.float().cpu().t(), atol=2e-3, rtol=2e-3)
+    x, w = rand(g, 8, 256, dtype=torch.bfloat16).to(DEV), rand(g, 320, 256, dtype=torch.bfloat16).to(DEV)
+    stream = rand(g, 8, 320).to(DEV)
+    before = stream.clone()
+    assert ops.linear_update(x, w, None, stream) is not None and torch.equal(stream, before)
+
+
 def test_linear_update_takes_the_mid_kernel(ops):
     g = torch.Generator().manual_seed(27)
     w = rand(g, 2560, 4096, dtype=torch.bfloat16, scale=0.05).to(DEV)
