@@ -50,6 +50,7 @@
 // values' loads are moved up to the first visible key's chunk, so that no page is
 // read that was given back).
 #include "common.h"
+#include <algorithm>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
@@ -75,13 +76,35 @@ __device__ __forceinline__ void load_to_lds(const void* global, void* lds) {
                                    (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
 }
 
+// every lane gets the sum (the largest) of v over the wave, without a trip through LDS
+__device__ __forceinline__ int wave_total(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);    // lane ^ 1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);    // lane ^ 2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);   // 7 - lane within 8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true);   // 15 - lane within 16
+  auto r = __builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false);
+  v = (int)(r[0] + r[1]);
+  r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+  return __builtin_amdgcn_readfirstlane((int)(r[0] + r[1]));
+}
+__device__ __forceinline__ int wave_most(int v) {
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true));
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true));
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true));
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true));
+  auto r = __builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false);
+  v = max((int)r[0], (int)r[1]);
+  r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+  return __builtin_amdgcn_readfirstlane(max((int)r[0], (int)r[1]));
+}
+
 template <int D, int KG>
 __global__ __launch_bounds__(256 * KG, 4) void paged_prefill_kernel(   // four waves a SIMD: at most 128 registers
     const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ key_pages,
     const bf16_t* __restrict__ value_pages, bf16_t* __restrict__ out, long long out_stride,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int table_stride, int kv_heads, int groups, int block_shift, int num_blocks, int window,
-    float scale_log2, int q_tiles, int pairs, int pairs_per_xcd) {
+    float scale_log2, int num_seqs, int heads_per_xcd) {
   const int block_mask = (1 << block_shift) - 1;
   constexpr int BM = 64;
   constexpr int KC = D / 32;            // MFMA k-steps over the head dim (scores)
@@ -91,17 +114,53 @@ __global__ __launch_bounds__(256 * KG, 4) void paged_prefill_kernel(   // four w
   constexpr int VI = 8 * D / 256;       // value load instructions per wave and tile
   __shared__ __attribute__((aligned(16))) uintx4 lds[KG * (BN * CH + 8 * D)];   // per key group: a tile of keys, a tile of values
 
-  // Block id b runs on XCD b % 8.  An XCD, with its own L2, takes a run of neighbouring (sequence,
-  // head) pairs, which share keys and values; within the XCD the blocks are ordered by row tile,
-  // the last (the longest walk over the keys) first, so that the blocks a CU holds at a time are
-  // a mix of long and short walks and the long ones start early.
+  // The grid is heads x tile slots, a slot being a place for one 64-row tile of some sequence
+  // (slots >= the tiles there are: the host knows the step's query tokens, not how they are spread
+  // over the sequences), so a step whose work sits in one long portion among single tokens launches
+  // few blocks that do nothing.  Slots go round by round: first the last tile of every sequence
+  // (the longest walk over its keys), then the tile before it of every sequence that has one, and
+  // so on, so that long walks start early and the blocks a CU holds at a time are a mix.
+  // Block id b runs on XCD b % 8; with eight heads or more an XCD, with its own L2, takes a run of
+  // neighbouring heads, which share keys and values, for every slot.
   const int heads = kv_heads * groups;
-  const int local = blockIdx.x / XCDS;
-  const int pair = (blockIdx.x % XCDS) * pairs_per_xcd + local % pairs_per_xcd;
-  if (pair >= pairs) return;
-  const int q_tile = q_tiles - 1 - local / pairs_per_xcd;
-  const int seq = pair / heads;
-  const int head = pair - seq * heads;
+  int head, slot;
+  if (heads_per_xcd > 0) {
+    const int local = blockIdx.x / XCDS;
+    head = (blockIdx.x % XCDS) * heads_per_xcd + local % heads_per_xcd;
+    slot = local / heads_per_xcd;
+  } else {
+    head = blockIdx.x % heads;
+    slot = blockIdx.x / heads;
+  }
+  if (head >= heads) return;
+  int seq = 0, q_tile = -1;
+  if (num_seqs <= FE_WAVE) {
+    // lane s looks at sequence s; tiles before round r: the sum over sequences of min(tiles, r)
+    const int me = threadIdx.x & (FE_WAVE - 1);
+    const int len = cu_q[min(me, num_seqs - 1) + 1] - cu_q[min(me, num_seqs - 1)];
+    const int tiles = me < num_seqs && len >= 2 ? (len + BM - 1) / BM : 0;
+    if (slot >= wave_total(tiles)) return;
+    int lo = 0, hi = wave_most(tiles);            // the round is in [lo, hi)
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (wave_total(min(tiles, mid)) <= slot) lo = mid; else hi = mid;
+    }
+    const int rank = slot - wave_total(min(tiles, lo));          // among the sequences with a tile in this round
+    const unsigned long long in_round = __ballot(tiles > lo);
+    const int before_me = __builtin_popcountll(in_round & ((1ull << me) - 1ull));
+    const unsigned long long mine = __ballot(tiles > lo && before_me == rank);
+    seq = __builtin_amdgcn_readfirstlane(__builtin_ctzll(mine));
+    q_tile = __builtin_amdgcn_readfirstlane(__shfl(tiles, seq, FE_WAVE)) - 1 - lo;
+  } else {
+    // more sequences than lanes: sequence by sequence, every other one's tiles in rising order
+    for (int first = 0; seq < num_seqs; ++seq) {
+      const int len = cu_q[seq + 1] - cu_q[seq];
+      const int tiles = len >= 2 ? (len + BM - 1) / BM : 0;
+      if (slot < first + tiles) { q_tile = (seq & 1) ? slot - first : tiles - 1 - (slot - first); break; }
+      first += tiles;
+    }
+    if (q_tile < 0) return;
+  }
   const int hk = head / groups;
   const int q0 = cu_q[seq];
   const int q_len = cu_q[seq + 1] - q0;
@@ -368,13 +427,16 @@ __global__ __launch_bounds__(256 * KG, 4) void paged_prefill_kernel(   // four w
 
 // Pages: keys [blocks][kv_heads][block_size][D], values transposed [blocks][kv_heads][D][block_size];
 // block_size a power of two >= 16; head_dim 64 or 128.  Sequences with fewer than two query tokens
-// are skipped.  key_groups: 1 or 2 groups of four waves a block (see the top of the file), 0 lets the launch choose.
+// are skipped.  key_groups: 1 or 2 groups of four waves a block (see the top of the file), 0 lets the launch
+// choose, from total_q: the query tokens of all sequences together (the rows of q; the grid is laid out for
+// num_seqs sequences of max_q_len tokens, of which a step with one long portion fills a fraction).
 extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, const void* key_pages,
                                                  const void* value_pages, void* out, long long out_stride,
                                                  const int* cu_q, const int* ctx_len, const int* block_table,
                                                  int table_stride, int num_seqs, int max_q_len, int kv_heads,
                                                  int groups, int head_dim, int block_size, int num_blocks,
-                                                 int window, float scale, int key_groups, hipStream_t stream) {
+                                                 int window, float scale, int key_groups, int total_q,
+                                                 hipStream_t stream) {
   if (num_seqs <= 0 || max_q_len < 2) return FE_OK;
   if (head_dim != 64 && head_dim != 128) return FE_BAD_ARGUMENT;
   if (groups < 1 || kv_heads < 1 || num_seqs > 65535) return FE_BAD_ARGUMENT;
@@ -383,22 +445,26 @@ extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, con
   const float scale_log2 = scale * 1.4426950408889634f;
   int block_shift = 0;
   while ((1 << block_shift) < block_size) ++block_shift;
-  const int q_tiles = (max_q_len + 63) / 64;
-  const long long pairs = (long long)num_seqs * kv_heads * groups;
-  const long long per_xcd = (pairs + XCDS - 1) / XCDS;
-  if (per_xcd * XCDS * q_tiles > 0x7fffffffLL) return FE_BAD_ARGUMENT;
-  const unsigned grid = (unsigned)(per_xcd * XCDS * q_tiles);
+  const int heads = kv_heads * groups;
+  const int heads_per_xcd = heads >= XCDS ? (heads + XCDS - 1) / XCDS : 0;
+  if (total_q < 1) return FE_BAD_ARGUMENT;
+  // places for 64-row tiles: a sequence of n tokens has at most n / 64 + 1, and the grid does not
+  // depend on how the tokens are spread over the sequences (a captured launch serves every spread)
+  const long long slots = std::min<long long>((long long)num_seqs * ((max_q_len + 63) / 64), total_q / 64 + num_seqs);
+  const long long blocks = (heads_per_xcd ? (long long)heads_per_xcd * XCDS : heads) * slots;
+  if (blocks > 0x7fffffffLL) return FE_BAD_ARGUMENT;
+  const unsigned grid = (unsigned)blocks;
   // Two key groups a block where the launch would leave the chip underfilled (all its blocks
   // resident at once: then the longest walk sets the time, and halving it pays; measured: one
   // prompt of 2,048 tokens 72 -> 66 us, of 512 tokens 18 -> 14 us) and the portions span at least
   // two tiles; with more blocks than that one group is faster (eight prompts of 1,024 tokens:
   // 126 against 141 us).
   if (key_groups < 0 || key_groups > 2) return FE_BAD_ARGUMENT;
-  if (key_groups == 0) key_groups = (per_xcd * XCDS * q_tiles <= 1024 && max_q_len >= 128) ? 2 : 1;
+  if (key_groups == 0) key_groups = ((long long)heads * slots <= 1024 && max_q_len >= 128) ? 2 : 1;
 #define FE_GO(DD, GG)                                                                                            \
   paged_prefill_kernel<DD, GG><<<grid, 256 * GG, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,            \
-      kv_heads, groups, block_shift, num_blocks, window, scale_log2, q_tiles, (int)pairs, (int)per_xcd)
+      kv_heads, groups, block_shift, num_blocks, window, scale_log2, num_seqs, heads_per_xcd)
   if (head_dim == 64 && key_groups == 1) FE_GO(64, 1);
   else if (head_dim == 64) FE_GO(64, 2);
   else if (key_groups == 1) FE_GO(128, 1);

@@ -19,7 +19,7 @@ from .batch import StepBatch, StepEntry, build_batch, static_batch, static_batch
 GRAPH_MAX_REQUESTS = 64      # decode steps of up to this many requests replay a captured graph
 GRAPH_TABLE_STEP = 64        # block-table widths of graphs are multiples of this many pages
 GRAPH_LIMIT = 24             # captured graphs kept (least recently used goes first)
-PORTION_GRAPH_MAX_TOKENS = 1024   # steps with prompt portions of up to this many tokens may be captured
+PORTION_GRAPH_MAX_TOKENS = 4096   # steps with prompt portions of up to this many tokens may be captured
 PORTION_GRAPH_SEQ_STEP = 8        # ... for a number of sequences rounded up to a multiple of this
 PORTION_GRAPH_WANT_STEP = 8       # ... and of wanted rows likewise (none stays none)
 

@@ -584,7 +584,7 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
               _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
               c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(PREFILL_KEY_GROUPS), _stream())
+              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(PREFILL_KEY_GROUPS), c_int(tokens), _stream())
     # whatever the two fast kernels did not take: single tokens go to the vector-ALU decode kernel where
     # it can read four elements at a time, the rest to the general kernel
     single_left = any_single and not fast_decode
