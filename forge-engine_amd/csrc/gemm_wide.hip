@@ -1,0 +1,185 @@
+// bfloat16 matrix product for a few dozen to a few hundred rows of x (a step that holds a
+// portion of a prompt, or many decoding requests):
+//   out[M, N] = x[M, K] * W[N, K]^T
+// with one of three endings: float32 partial sums over parts of K ([parts][M, N]; the consumer, the
+// next norm, adds them in order), bfloat16, or silu(gate) * up as bfloat16 for a fused gate/up
+// weight.  At these row counts the product is bound by the weight's bytes and by how the rows of x
+// reach the matrix cores, not by arithmetic: the matrix library, tuned for large products, takes
+// three to four times the time the bytes need.
+//
+// Block = (64 weight rows, a part of K, a tile of MT * 16 rows of x); four waves of 16 weight rows
+// (with the gate/up ending: 16 gate rows and the 16 up rows that belong to them).  The weight goes
+// from HBM straight into MFMA operand registers, each element used by one wave only; x (shared by
+// the four waves) is staged through LDS in 64-wide steps, three stages, one barrier a step,
+// operands fetched two steps ahead, every load unconditional.  A wave needs no other wave's sums.
+// Tiles of x rows beyond the first read the weight again (from L2: the tiles of one weight tile
+// run side by side).
+//
+// MFMA 16x16x32 bf16 with A = x (16 rows), B = W^T (16 weight rows):
+//   lane l supplies A[m = l % 16][k = 8*(l / 16) .. +8], B[k = 8*(l / 16) .. +8][n = l % 16]
+//   and receives D[m = 4*(l / 16) + i][n = l % 16].
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
+
+#define WSTEP 64          // elements of K a step
+#define WIDE_ROWS 64      // weight rows (gate/up ending: output columns) a block
+
+#define EPI_PARTS 0
+#define EPI_BF16 1
+#define EPI_SWIGLU 2
+
+__device__ __forceinline__ float silu_times(float g, float u) { return g / (1.f + __expf(-g)) * u; }
+
+// LDS holds a step of x as [row][8 chunks of 16 bytes], chunk c of row r at position c ^ (r % 8):
+// the eight lanes that a 16-byte read serves in one cycle then hit eight different bank groups.
+template <int MT, int EPI>
+__global__ __launch_bounds__(256, 2) void gemm_wide_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
+    int K, long long ldw, long long ldo, int steps_per_part, long long part_stride, long long up_offset) {
+  constexpr int WF = EPI == EPI_SWIGLU ? 2 : 1;     // weight operands a wave holds: gate and up, or one
+  constexpr int XL = MT / 2;                        // 16-byte pieces of a step of x a thread fetches
+  __shared__ __attribute__((aligned(16))) bf16_t xs[3][MT * 16][WSTEP];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int lr = lane & 15;
+  const int lq = lane >> 4;
+  const int n = blockIdx.x * WIDE_ROWS + wave * 16 + lr;
+  const int m0 = blockIdx.z * MT * 16;
+  const bf16_t* wrow = w + (size_t)(n < N ? n : 0) * ldw;
+  const int steps = K / WSTEP;
+  const int first = blockIdx.y * steps_per_part;
+  const int last = min(steps, first + steps_per_part);
+
+  floatx4 acc[WF][MT];
+#pragma unroll
+  for (int f = 0; f < WF; ++f)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[f][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  if (first < last) {
+    uintx4 xr[3][XL], wr[3][WF * 2];
+    // x loader: piece p = tid + 256 i is chunk p % 8 of row p / 8.  Rows of x beyond M read row 0
+    // again: their sums are never stored.  Nothing is selected on a loaded value, so no load is
+    // waited for where it is issued.
+    auto load = [&](int step, uintx4* xdst, uintx4* wdst) {
+      step = min(step, last - 1);
+#pragma unroll
+      for (int i = 0; i < XL; ++i) {
+        const int p = tid + 256 * i;
+        const int row = m0 + (p >> 3);
+        xdst[i] = *(const uintx4*)(x + (size_t)(row < M ? row : 0) * K + step * WSTEP + (p & 7) * 8);
+      }
+#pragma unroll
+      for (int f = 0; f < WF; ++f)
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+          wdst[f * 2 + c] = *(const uintx4*)(wrow + f * up_offset + step * WSTEP + lq * 8 + c * 32);
+    };
+    auto store_x = [&](int stage, const uintx4* xsrc) {
+#pragma unroll
+      for (int i = 0; i < XL; ++i) {
+        const int p = tid + 256 * i;
+        const int row = p >> 3;
+        *(uintx4*)&xs[stage][row][((p & 7) ^ (row & 7)) * 8] = xsrc[i];
+      }
+    };
+    auto multiply = [&](int stage, const uintx4* wreg) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const int row = mt * 16 + lr;
+          const bf16x8 a = *(const bf16x8*)&xs[stage][row][((c * 4 + lq) ^ (lr & 7)) * 8];
+#pragma unroll
+          for (int f = 0; f < WF; ++f)
+            acc[f][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, wreg[f * 2 + c]), acc[f][mt], 0, 0, 0);
+        }
+      }
+    };
+
+    // Step s (counted from the part's first) has its operands in register set s % 3 and its x in
+    // LDS stage s % 3.  The loop takes three steps a round so that both are compile-time constants.
+    load(first, xr[0], wr[0]);
+    load(first + 1, xr[1], wr[1]);
+    store_x(0, xr[0]);
+    __syncthreads();
+    int step = first;
+    for (; step + 3 <= last; step += 3) {
+#pragma unroll
+      for (int u = 0; u < 3; ++u) {
+        load(step + u + 2, xr[(u + 2) % 3], wr[(u + 2) % 3]);
+        multiply(u, wr[u]);
+        store_x((u + 1) % 3, xr[(u + 1) % 3]);
+        __syncthreads();
+      }
+    }
+    const int left = last - step;          // 0 .. 2 steps, the same for every thread
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      if (u < left) {
+        if (u + 2 < left) load(step + u + 2, xr[(u + 2) % 3], wr[(u + 2) % 3]);
+        multiply(u % 3, wr[u % 3]);
+        if (u + 1 < left) {
+          store_x((u + 1) % 3, xr[(u + 1) % 3]);
+          __syncthreads();
+        }
+      }
+    }
+  }
+
+  // D[m = 4 lq + i][n = lr] of row tile mt: for each i the 16 lanes of a group write 16 neighbouring n
+  if (n < N) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = m0 + mt * 16 + lq * 4 + i;
+        if (m >= M) continue;
+        if (EPI == EPI_PARTS) ((float*)out)[(size_t)blockIdx.y * part_stride + (size_t)m * ldo + n] = acc[0][mt][i];
+        else if (EPI == EPI_BF16) ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(acc[0][mt][i]);
+        else ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(silu_times(acc[0][mt][i], acc[WF - 1][mt][i]));
+      }
+  }
+}
+
+// x [M, K] bf16 contiguous, K a multiple of 64; w [N, K] bf16 with row stride ldw, rows 16-byte aligned.
+// ending 0: out holds `parts` float32 matrices [M, N] (row stride ldo) part_stride floats apart, part s
+//   the sum over the s-th run of whole 64-steps of K; every part is written in full (zeros where a part
+//   has no steps), so the caller may add all of them up.
+// ending 1: out is bfloat16 [M, N] with row stride ldo; parts must be 1.
+// ending 2: w is a fused gate/up weight [2 N, K], gate rows first; out is bfloat16 [M, N] =
+//   silu(x gate^T) * (x up^T); parts must be 1.
+// Any M: rows are taken in tiles of row_tile = 64 or 128 (smaller tiles: more blocks, and the weight
+// read again, from L2, once per tile).
+extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int N, int K, long long ldw,
+                            long long ldo, int ending, int parts, long long part_stride, int row_tile,
+                            hipStream_t stream) {
+  if (M < 1) return FE_OK;
+  if (N < 1 || K < WSTEP || K % WSTEP || ldw < K || ldw % 8 || ldo < N) return FE_BAD_ARGUMENT;
+  if ((((uintptr_t)x) & 15) || (((uintptr_t)w) & 15)) return FE_BAD_ARGUMENT;
+  if (ending < EPI_PARTS || ending > EPI_SWIGLU) return FE_BAD_ARGUMENT;
+  if (parts < 1 || parts > 64 || (ending != EPI_PARTS && parts != 1)) return FE_BAD_ARGUMENT;
+  if (parts > 1 && part_stride < (long long)M * ldo) return FE_BAD_ARGUMENT;
+  const int steps = K / WSTEP;
+  const int per_part = (steps + parts - 1) / parts;
+  if (row_tile != 64 && row_tile != 128) return FE_BAD_ARGUMENT;
+  const int mt = row_tile / 16;
+  const long long m_tiles = (M + mt * 16 - 1) / (mt * 16);
+  if (m_tiles > 65535) return FE_BAD_ARGUMENT;
+  dim3 grid((N + WIDE_ROWS - 1) / WIDE_ROWS, parts, (unsigned)m_tiles);
+  const long long up_offset = (long long)N * ldw;
+#define FE_GO(MT, EPI)                                                                                   \
+  gemm_wide_kernel<MT, EPI><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, \
+                                                      ldw, ldo, per_part, part_stride, up_offset)
+  if (mt == 4) {
+    if (ending == EPI_PARTS) FE_GO(4, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(4, EPI_BF16); else FE_GO(4, EPI_SWIGLU);
+  } else {
+    if (ending == EPI_PARTS) FE_GO(8, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(8, EPI_BF16); else FE_GO(8, EPI_SWIGLU);
+  }
+#undef FE_GO
+  return fe_check_launch();
+}

@@ -245,6 +245,8 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
         raise KernelError(f"activation {x.dtype} does not match weight {weight.dtype}")
     if bias is None and _skinny_fits(x, weight) and out_dtype in (torch.float32, torch.bfloat16):
         return gemm_skinny(x, weight, "f32" if out_dtype == torch.float32 else "bf16")
+    if bias is None and out_dtype == torch.bfloat16 and _wide_fits(x, weight, WIDE_STORE_MAX_ROWS):
+        return gemm_wide(x, weight, "bf16", row_tile=64)
     if out_dtype == torch.float32:
         y = torch.mm(x, weight.t(), out_dtype=torch.float32)
     else:
@@ -300,6 +302,59 @@ def gemm_mid_parts(x: Tensor, weight: Tensor, parts: int) -> Tensor:
     return out
 
 
+# Measured on MI355X at Qwen3-4B's sizes against the matrix library, per call: the products back to the
+# hidden size (2560 weight rows; K = 4096 / 9728) in parts of K take 14 / 22 us at 128 rows (library 28 / 53),
+# 17 / 32 us at 256 rows (25 / 46), 21 / 43 at 384 (24 / 47) and lose from 512 rows on; the q/k/v product
+# (6144 weight rows) in row tiles of 64 takes 23 - 27 us at 96 to 256 rows (library 27 - 33); the gate/up
+# product (19456 weight rows) is the library's at every row count above 64 (55 against 52 us at 256 rows).
+WIDE_UPDATE_MAX_ROWS = 384     # most rows of x for which a product in parts of K beats the matrix library
+WIDE_STORE_MAX_ROWS = 256      # ... and a product that stores bfloat16
+WIDE_MAX_WEIGHT_ROWS = 8192    # weights with more rows fill the chip in the library's large tiles
+WIDE_TARGET_BLOCKS = 480       # blocks the product aims at when it cuts K into parts (two resident a CU)
+
+
+def _wide_fits(x: Tensor, weight: Tensor, most_rows: int) -> bool:
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2 and x.is_contiguous()
+            and MID_ROWS < x.shape[0] <= most_rows and weight.dim() == 2 and weight.stride(1) == 1
+            and weight.shape[0] <= WIDE_MAX_WEIGHT_ROWS
+            and weight.shape[1] == x.shape[1] and x.shape[1] % 64 == 0 and weight.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def gemm_wide(x: Tensor, weight: Tensor, ending: str = "bf16", parts: int = 1, row_tile: int = 0) -> Tensor:
+    """x @ weight^T for a few dozen to a few hundred bfloat16 rows: ``"parts"`` float32 partial sums
+    [parts, M, N] over runs of whole 64-steps of K, ``"bf16"`` [M, N], or ``"swiglu"``: silu(gate) * up
+    [M, N / 2] for a fused gate/up weight (gate rows first)."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(weight, "weight", torch.bfloat16, contiguous=False)
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k or k % 64 or weight.stride(1) != 1 or weight.stride(0) % 8 or not 1 <= parts <= 64:
+        raise KernelError("the product for portions takes contiguous bfloat16 rows, K a multiple of 64, at most 64 parts")
+    if ending == "parts":
+        out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
+        code, cols = 0, n
+    elif ending in ("bf16", "swiglu") and parts == 1 and (ending == "bf16" or n % 2 == 0):
+        cols = n if ending == "bf16" else n // 2
+        out = torch.empty((m, cols), dtype=torch.bfloat16, device=x.device)
+        code = 1 if ending == "bf16" else 2
+    else:
+        raise KernelError(f"no ending {ending!r} with {parts} parts")
+    _call("gemm_wide", "fe_gemm_wide", _ptr(x), _ptr(weight), _ptr(out), c_int(m), c_int(cols), c_int(k),
+          c_longlong(weight.stride(0)), c_longlong(cols), c_int(code), c_int(parts), c_longlong(m * cols),
+          c_int(row_tile or (64 if m <= 64 else 128)), _stream())
+    return out
+
+
+def _wide_parts(m: int, n: int, k: int) -> int:
+    """Parts of K for the product above: about WIDE_TARGET_BLOCKS blocks in all, at least eight 64-steps
+    a part (the kernel fetches two steps ahead), no part without steps."""
+    steps = k // 64
+    blocks = -(-n // 64) * -(-m // (64 if m <= 64 else 128))
+    parts = max(1, min(16, WIDE_TARGET_BLOCKS // blocks, steps // 8))
+    return -(-steps // -(-steps // parts))
+
+
 def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None, stream: Tensor | None = None) -> Tensor | None:
     """The float32 product x @ weight^T (+ bias) as an update of the residual stream: [M, N], or
     partial sums [parts, M, N] that ``add_rmsnorm`` / ``add_rows`` add up.  Given the float32
@@ -321,6 +376,8 @@ def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None, stream:
         steps = -(-weight.shape[1] // 128)
         blocks = -(-weight.shape[0] // 64)
         return gemm_mid_parts(x, weight, _mid_parts(steps, blocks))
+    if plain_bf16 and _wide_fits(x, weight, WIDE_UPDATE_MAX_ROWS):
+        return gemm_wide(x, weight, "parts", _wide_parts(x.shape[0], weight.shape[0], weight.shape[1]))
     if (plain_bf16 and stream is not None and x.shape[0] > SKINNY_MAX_ROWS and stream.dtype == torch.float32
             and stream.shape == (x.shape[0], weight.shape[0]) and stream.is_contiguous()):
         torch.addmm(stream, x, weight.t(), out_dtype=torch.float32, out=stream)
@@ -744,4 +801,4 @@ def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index:
           _stream())
 
 
-LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")
+LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")

@@ -158,7 +158,7 @@ class GroupedQueryAttention(Mixer):
                     rotary_dim=rotary_dim, block_size=cache.key_pages.shape[2]))
 
     def kernel_libraries(self):
-        return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny", "gemm_mid"}
+        return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
 
 
 register_part("mixer", "gqa_attention", GroupedQueryAttention)

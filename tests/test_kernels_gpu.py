@@ -574,7 +574,9 @@ def test_linear_update_routes(ops):
     assert ops.linear_update(x, many_rows).dim() == 2
     assert ops.linear_update(x[:, :1024].contiguous(), few_rows[:, :1024]).dim() == 2
     big = rand(g, 70, 4096, dtype=torch.bfloat16).to(DEV)
-    assert ops.linear_update(big, few_rows).shape == (70, 320)     # beyond 64 rows: the library
+    assert ops.linear_update(big, few_rows).shape[1:] == (70, 320)     # 65 to 384 rows: the product for portions, in parts
+    huge = rand(g, 500, 4096, dtype=torch.bfloat16).to(DEV)
+    assert ops.linear_update(huge, few_rows).shape == (500, 320)       # beyond: the library
     want = x.float().cpu() @ few_rows.float().cpu().T
     torch.testing.assert_close(ops.linear_update(x, few_rows).sum(0).cpu(), want, atol=1e-3, rtol=1e-3)
 
@@ -608,6 +610,67 @@ def test_gemm_mid_parts(ops, m, n, k, parts):
     assert torch.equal(ops.add_rows(h1, got), ops.add_rows(h2, summed))
 
 
+@pytest.mark.parametrize("m", [17, 65, 100, 128, 130, 300])
+@pytest.mark.parametrize("n,k,parts", [(2560, 4096, 8), (200, 256, 2), (1003, 1024, 3), (64, 64, 1), (70, 640, 5), (330, 9728, 16)])
+@pytest.mark.parametrize("row_tile", [64, 128])
+def test_gemm_wide_parts(ops, m, n, k, parts, row_tile):
+    """The product for portions of prompts: partial sums over parts of K (parts without steps are
+    zeros), any number of rows in tiles of 64 or 128, weight rows that are no multiple of the
+    block's 64, a weight that is a view with a longer row stride."""
+    g = torch.Generator().manual_seed(m + n + k)
+    x = rand(g, m, k, dtype=torch.bfloat16)
+    w_full = rand(g, n, k + 8, dtype=torch.bfloat16, scale=0.05)
+    w = w_full[:, :k]
+    got = ops.gemm_wide(x.to(DEV), w_full.to(DEV)[:, :k], "parts", parts, row_tile)
+    assert got.shape == (parts, m, n)
+    want = x.float() @ w.float().t()
+    torch.testing.assert_close(got.sum(0).cpu(), want, atol=1e-3 * (k / 256) ** 0.5, rtol=1e-3)
+    steps = k // 64
+    per = -(-steps // parts)
+    for part in range(parts):
+        lo, hi = part * per * 64, min(k, (part + 1) * per * 64)
+        want_part = x[:, lo:hi].float() @ w[:, lo:hi].float().t() if lo < hi else torch.zeros(m, n)
+        torch.testing.assert_close(got[part].cpu(), want_part, atol=1e-3 * (k / 256) ** 0.5, rtol=1e-3)
+
+
+@pytest.mark.parametrize("m", [20, 64, 77, 256, 260])
+@pytest.mark.parametrize("n,k", [(6144, 2560), (200, 192), (1002, 320)])
+def test_gemm_wide_stores_and_gates(ops, m, n, k):
+    g = torch.Generator().manual_seed(m * 3 + n + k)
+    x = rand(g, m, k, dtype=torch.bfloat16)
+    w = rand(g, n, k, dtype=torch.bfloat16, scale=0.05)
+    want = x.float() @ w.float().t()
+    for row_tile in (64, 128):
+        got = ops.gemm_wide(x.to(DEV), w.to(DEV), "bf16", 1, row_tile)
+        torch.testing.assert_close(got.cpu().float(), want.to(torch.bfloat16).float(), atol=2e-2, rtol=2e-2)
+        gated = ops.gemm_wide(x.to(DEV), w.to(DEV), "swiglu", 1, row_tile)
+        gate, up = want[:, :n // 2], want[:, n // 2:]
+        torch.testing.assert_close(gated.cpu().float(), (gate / (1 + torch.exp(-gate)) * up), atol=2e-2, rtol=2e-2)
+        assert gated.shape == (m, n // 2)
+
+
+def test_gemm_wide_refuses_and_routes(ops, monkeypatch):
+    x = torch.zeros(70, 200, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 200, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_wide(x, w, "parts", 2)                    # K is no multiple of 64
+    with pytest.raises(ops.KernelError):
+        ops.gemm_wide(x[:, :192].contiguous(), w[:, :192], "bf16", 2)     # a stored product has one part
+    taken = []
+    real_call = ops._call
+    monkeypatch.setattr(ops, "_call", lambda lib, name, *a: taken.append(name) or real_call(lib, name, *a))
+    g = torch.Generator().manual_seed(5)
+    x = rand(g, 100, 256, dtype=torch.bfloat16).to(DEV)
+    w = rand(g, 320, 256, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    update = ops.linear_update(x, w, None, torch.zeros(100, 320, device=DEV))
+    assert update is not None and update.dim() == 3 and taken == ["fe_gemm_wide"]
+    torch.testing.assert_close(update.sum(0).cpu(), x.float().cpu() @ w.float().cpu().t(), atol=1e-3, rtol=1e-3)
+    y = ops.linear(x, w)
+    assert taken == ["fe_gemm_wide", "fe_gemm_wide"] and y.dtype == torch.bfloat16
+    big = rand(g, 600, 256, dtype=torch.bfloat16).to(DEV)
+    assert ops.linear_update(big, w, None, torch.zeros(600, 320, device=DEV)) is None and len(taken) == 2   # the library's
+
+
 def test_gemm_mid_parts_refuses_a_k_that_is_no_multiple_of_its_step(ops):
     g = torch.Generator().manual_seed(27)
     x = rand(g, 20, 264, dtype=torch.bfloat16).to(DEV)
@@ -624,7 +687,7 @@ def test_linear_update_adds_into_the_stream_where_the_library_multiplies(ops):
     nothing is left pending; the stream then holds exactly stream + product.  Fewer rows: the update
     comes back (in parts) and the stream is left alone."""
     g = torch.Generator().manual_seed(31)
-    for m, n, k in ((200, 320, 256), (65, 2560, 4096)):
+    for m, n, k in ((500, 320, 256), (390, 2560, 4096)):
         x, w = rand(g, m, k, dtype=torch.bfloat16).to(DEV), rand(g, n, k, dtype=torch.bfloat16, scale=0.05).to(DEV)
         stream = rand(g, m, n).to(DEV)
         before = stream.clone()
@@ -647,7 +710,11 @@ def test_linear_update_takes_the_mid_kernel(ops):
         assert update.dim() == 3 and update.shape[1:] == (rows, 2560)
         want = x.float().cpu() @ w.float().cpu().T
         torch.testing.assert_close(update.sum(0).cpu(), want, atol=2e-3, rtol=2e-3)
-    assert ops.linear_update(rand(g, 65, 4096, dtype=torch.bfloat16).to(DEV), w).dim() == 2
+    more = rand(g, 65, 4096, dtype=torch.bfloat16).to(DEV)          # 65 rows and more: the product for portions, also in parts
+    update = ops.linear_update(more, w)
+    assert update.dim() == 3
+    torch.testing.assert_close(update.sum(0).cpu(), more.float().cpu() @ w.float().cpu().T, atol=2e-3, rtol=2e-3)
+    assert ops.linear_update(rand(g, 400, 4096, dtype=torch.bfloat16).to(DEV), w).dim() == 2     # the library
 
 
 def test_linear_routes_by_rows_and_dtype(ops):
