@@ -10,8 +10,12 @@
 // Block = (64 weight rows, a part of K, a tile of MT * 16 rows of x); four waves of 16 weight rows
 // (with the gate/up ending: 16 gate rows and the 16 up rows that belong to them).  The weight goes
 // from HBM straight into MFMA operand registers, each element used by one wave only; x (shared by
-// the four waves) is staged through LDS in 64-wide steps, three stages, one barrier a step,
-// operands fetched two steps ahead, every load unconditional.  A wave needs no other wave's sums.
+// the four waves) is staged through LDS in 64-wide steps, two stages, one barrier a step; operands
+// are fetched four steps ahead (eight gained nothing), every load unconditional.  A wave needs no
+// other wave's sums.  What bounds the kernel, measured over tile shapes and row counts: the bytes
+// that all blocks together pull into their CUs (the weight once per row tile, x once per 64 weight
+// rows, the partial sums), at about 8 TB/s for the whole chip, so only a launch that keeps every CU
+// busy streams the weight at the memory's speed: hence the parts of K where a weight has few rows.
 // Tiles of x rows beyond the first read the weight again (from L2: the tiles of one weight tile
 // run side by side).
 //
@@ -35,13 +39,13 @@ __device__ __forceinline__ float silu_times(float g, float u) { return g / (1.f 
 
 // LDS holds a step of x as [row][8 chunks of 16 bytes], chunk c of row r at position c ^ (r % 8):
 // the eight lanes that a 16-byte read serves in one cycle then hit eight different bank groups.
-template <int MT, int EPI>
+template <int MT, int EPI, int R>
 __global__ __launch_bounds__(256, 2) void gemm_wide_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
     int K, long long ldw, long long ldo, int steps_per_part, long long part_stride, long long up_offset) {
   constexpr int WF = EPI == EPI_SWIGLU ? 2 : 1;     // weight operands a wave holds: gate and up, or one
   constexpr int XL = MT / 2;                        // 16-byte pieces of a step of x a thread fetches
-  __shared__ __attribute__((aligned(16))) bf16_t xs[3][MT * 16][WSTEP];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][WSTEP];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -61,11 +65,12 @@ __global__ __launch_bounds__(256, 2) void gemm_wide_kernel(
     for (int mt = 0; mt < MT; ++mt) acc[f][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   if (first < last) {
-    uintx4 xr[3][XL], wr[3][WF * 2];
+    static_assert(R % 2 == 0, "a round of the loop is a whole number of LDS stage rotations");
+    uintx4 xr[R][XL], wr[R][WF * 2];
     // x loader: piece p = tid + 256 i is chunk p % 8 of row p / 8.  Rows of x beyond M read row 0
     // again: their sums are never stored.  Nothing is selected on a loaded value, so no load is
-    // waited for where it is issued.
-    auto load = [&](int step, uintx4* xdst, uintx4* wdst) {
+    // waited for where it is issued; a step beyond the part's end reads the last step again.
+    auto load_x = [&](int step, uintx4* xdst) {
       step = min(step, last - 1);
 #pragma unroll
       for (int i = 0; i < XL; ++i) {
@@ -73,6 +78,9 @@ __global__ __launch_bounds__(256, 2) void gemm_wide_kernel(
         const int row = m0 + (p >> 3);
         xdst[i] = *(const uintx4*)(x + (size_t)(row < M ? row : 0) * K + step * WSTEP + (p & 7) * 8);
       }
+    };
+    auto load_w = [&](int step, uintx4* wdst) {
+      step = min(step, last - 1);
 #pragma unroll
       for (int f = 0; f < WF; ++f)
 #pragma unroll
@@ -101,30 +109,37 @@ __global__ __launch_bounds__(256, 2) void gemm_wide_kernel(
       }
     };
 
-    // Step s (counted from the part's first) has its operands in register set s % 3 and its x in
-    // LDS stage s % 3.  The loop takes three steps a round so that both are compile-time constants.
-    load(first, xr[0], wr[0]);
-    load(first + 1, xr[1], wr[1]);
+    // Step s (counted from the part's first) has its operands in register sets s % R: the weight's,
+    // fetched R - 1 steps ahead, feed the MFMAs directly; those of x, fetched R steps ahead, go to
+    // LDS stage s % 2 one step before they are used (a step's arithmetic is far shorter than a trip
+    // to memory, what is stored to LDS has to have arrived, and a launch of few blocks keeps the
+    // memory busy only through what each block has in flight).  The loop takes R steps a round so
+    // that all of these are compile-time constants; one barrier a step.
+#pragma unroll
+    for (int u = 0; u < R - 1; ++u) load_w(first + u, wr[u]);
+#pragma unroll
+    for (int u = 0; u < R; ++u) load_x(first + u, xr[u]);
     store_x(0, xr[0]);
     __syncthreads();
+    // The rounds are straight-line code: where branches meet, every load in flight would be waited for.
     int step = first;
-    for (; step + 3 <= last; step += 3) {
+    for (; step + R <= last; step += R) {
 #pragma unroll
-      for (int u = 0; u < 3; ++u) {
-        load(step + u + 2, xr[(u + 2) % 3], wr[(u + 2) % 3]);
-        multiply(u, wr[u]);
-        store_x((u + 1) % 3, xr[(u + 1) % 3]);
+      for (int u = 0; u < R; ++u) {
+        load_w(step + u + R - 1, wr[(u + R - 1) % R]);
+        load_x(step + u + R, xr[u]);
+        multiply(u % 2, wr[u]);
+        store_x((u + 1) % 2, xr[(u + 1) % R]);
         __syncthreads();
       }
     }
-    const int left = last - step;          // 0 .. 2 steps, the same for every thread
+    const int left = last - step;          // 0 .. R - 1 steps, the same for every thread; their operands are on their way
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < R - 1; ++u) {
       if (u < left) {
-        if (u + 2 < left) load(step + u + 2, xr[(u + 2) % 3], wr[(u + 2) % 3]);
-        multiply(u % 3, wr[u % 3]);
+        multiply(u % 2, wr[u]);
         if (u + 1 < left) {
-          store_x((u + 1) % 3, xr[(u + 1) % 3]);
+          store_x((u + 1) % 2, xr[(u + 1) % R]);
           __syncthreads();
         }
       }
@@ -172,13 +187,13 @@ extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int 
   if (m_tiles > 65535) return FE_BAD_ARGUMENT;
   dim3 grid((N + WIDE_ROWS - 1) / WIDE_ROWS, parts, (unsigned)m_tiles);
   const long long up_offset = (long long)N * ldw;
-#define FE_GO(MT, EPI)                                                                                   \
-  gemm_wide_kernel<MT, EPI><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, \
+#define FE_GO(MT, EPI, R)                                                                                   \
+  gemm_wide_kernel<MT, EPI, R><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, \
                                                       ldw, ldo, per_part, part_stride, up_offset)
   if (mt == 4) {
-    if (ending == EPI_PARTS) FE_GO(4, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(4, EPI_BF16); else FE_GO(4, EPI_SWIGLU);
+    if (ending == EPI_PARTS) FE_GO(4, EPI_PARTS, 4); else if (ending == EPI_BF16) FE_GO(4, EPI_BF16, 4); else FE_GO(4, EPI_SWIGLU, 4);
   } else {
-    if (ending == EPI_PARTS) FE_GO(8, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(8, EPI_BF16); else FE_GO(8, EPI_SWIGLU);
+    if (ending == EPI_PARTS) FE_GO(8, EPI_PARTS, 4); else if (ending == EPI_BF16) FE_GO(8, EPI_BF16, 4); else FE_GO(8, EPI_SWIGLU, 4);
   }
 #undef FE_GO
   return fe_check_launch();

@@ -246,7 +246,7 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
     if bias is None and _skinny_fits(x, weight) and out_dtype in (torch.float32, torch.bfloat16):
         return gemm_skinny(x, weight, "f32" if out_dtype == torch.float32 else "bf16")
     if bias is None and out_dtype == torch.bfloat16 and _wide_fits(x, weight, WIDE_STORE_MAX_ROWS):
-        return gemm_wide(x, weight, "bf16", row_tile=64)
+        return gemm_wide(x, weight, "bf16", row_tile=64 if x.shape[0] <= 128 else 128)
     if out_dtype == torch.float32:
         y = torch.mm(x, weight.t(), out_dtype=torch.float32)
     else:
@@ -305,7 +305,8 @@ def gemm_mid_parts(x: Tensor, weight: Tensor, parts: int) -> Tensor:
 # Measured on MI355X at Qwen3-4B's sizes against the matrix library, per call: the products back to the
 # hidden size (2560 weight rows; K = 4096 / 9728) in parts of K take 14 / 22 us at 128 rows (library 28 / 53),
 # 17 / 32 us at 256 rows (25 / 46), 21 / 43 at 384 (24 / 47) and lose from 512 rows on; the q/k/v product
-# (6144 weight rows) in row tiles of 64 takes 23 - 27 us at 96 to 256 rows (library 27 - 33); the gate/up
+# (6144 weight rows) takes 18 - 20 us at 96 and 128 rows in row tiles of 64 and 23 - 26 us at 192 and 256 rows
+# in tiles of 128 (library 24 and 27 - 33); the gate/up
 # product (19456 weight rows) is the library's at every row count above 64 (55 against 52 us at 256 rows).
 WIDE_UPDATE_MAX_ROWS = 384     # most rows of x for which a product in parts of K beats the matrix library
 WIDE_STORE_MAX_ROWS = 256      # ... and a product that stores bfloat16
