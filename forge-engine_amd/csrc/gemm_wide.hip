@@ -29,7 +29,6 @@ typedef __attribute__((ext_vector_type(4))) float floatx4;
 typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 
 #define WSTEP 64          // elements of K a step
-#define WIDE_ROWS 64      // weight rows (gate/up ending: output columns) a block
 
 #define EPI_PARTS 0
 #define EPI_BF16 1
@@ -39,19 +38,20 @@ __device__ __forceinline__ float silu_times(float g, float u) { return g / (1.f 
 
 // LDS holds a step of x as [row][8 chunks of 16 bytes], chunk c of row r at position c ^ (r % 8):
 // the eight lanes that a 16-byte read serves in one cycle then hit eight different bank groups.
-template <int MT, int EPI, int R>
-__global__ __launch_bounds__(256, 2) void gemm_wide_kernel(
+template <int MT, int EPI, int R, int WPB>
+__global__ __launch_bounds__(64 * WPB, 2) void gemm_wide_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
     int K, long long ldw, long long ldo, int steps_per_part, long long part_stride, long long up_offset) {
   constexpr int WF = EPI == EPI_SWIGLU ? 2 : 1;     // weight operands a wave holds: gate and up, or one
-  constexpr int XL = MT / 2;                        // 16-byte pieces of a step of x a thread fetches
+  constexpr int XL = 2 * MT / WPB;                  // 16-byte pieces of a step of x a thread fetches
+  constexpr int THREADS = 64 * WPB;
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][WSTEP];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int lr = lane & 15;
   const int lq = lane >> 4;
-  const int n = blockIdx.x * WIDE_ROWS + wave * 16 + lr;
+  const int n = blockIdx.x * (16 * WPB) + wave * 16 + lr;
   const int m0 = blockIdx.z * MT * 16;
   const bf16_t* wrow = w + (size_t)(n < N ? n : 0) * ldw;
   const int steps = K / WSTEP;
@@ -67,14 +67,14 @@ __global__ __launch_bounds__(256, 2) void gemm_wide_kernel(
   if (first < last) {
     static_assert(R % 2 == 0, "a round of the loop is a whole number of LDS stage rotations");
     uintx4 xr[R][XL], wr[R][WF * 2];
-    // x loader: piece p = tid + 256 i is chunk p % 8 of row p / 8.  Rows of x beyond M read row 0
+    // x loader: piece p = tid + THREADS i is chunk p % 8 of row p / 8.  Rows of x beyond M read row 0
     // again: their sums are never stored.  Nothing is selected on a loaded value, so no load is
     // waited for where it is issued; a step beyond the part's end reads the last step again.
     auto load_x = [&](int step, uintx4* xdst) {
       step = min(step, last - 1);
 #pragma unroll
       for (int i = 0; i < XL; ++i) {
-        const int p = tid + 256 * i;
+        const int p = tid + THREADS * i;
         const int row = m0 + (p >> 3);
         xdst[i] = *(const uintx4*)(x + (size_t)(row < M ? row : 0) * K + step * WSTEP + (p & 7) * 8);
       }
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256, 2) void gemm_wide_kernel(
     auto store_x = [&](int stage, const uintx4* xsrc) {
 #pragma unroll
       for (int i = 0; i < XL; ++i) {
-        const int p = tid + 256 * i;
+        const int p = tid + THREADS * i;
         const int row = p >> 3;
         *(uintx4*)&xs[stage][row][((p & 7) ^ (row & 7)) * 8] = xsrc[i];
       }
@@ -169,10 +169,11 @@ __global__ __launch_bounds__(256, 2) void gemm_wide_kernel(
 // ending 2: w is a fused gate/up weight [2 N, K], gate rows first; out is bfloat16 [M, N] =
 //   silu(x gate^T) * (x up^T); parts must be 1.
 // Any M: rows are taken in tiles of row_tile = 64 or 128 (smaller tiles: more blocks, and the weight
-// read again, from L2, once per tile).
+// read again, from L2, once per tile).  block_rows = 64 or 32: the weight rows (gate/up ending: output
+// columns) a block of four or two waves takes; 32 gives a launch of few blocks twice as many.
 extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int N, int K, long long ldw,
                             long long ldo, int ending, int parts, long long part_stride, int row_tile,
-                            hipStream_t stream) {
+                            int block_rows, hipStream_t stream) {
   if (M < 1) return FE_OK;
   if (N < 1 || K < WSTEP || K % WSTEP || ldw < K || ldw % 8 || ldo < N) return FE_BAD_ARGUMENT;
   if ((((uintptr_t)x) & 15) || (((uintptr_t)w) & 15)) return FE_BAD_ARGUMENT;
@@ -185,15 +186,22 @@ extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int 
   const int mt = row_tile / 16;
   const long long m_tiles = (M + mt * 16 - 1) / (mt * 16);
   if (m_tiles > 65535) return FE_BAD_ARGUMENT;
-  dim3 grid((N + WIDE_ROWS - 1) / WIDE_ROWS, parts, (unsigned)m_tiles);
+  if (block_rows != 64 && block_rows != 32) return FE_BAD_ARGUMENT;
+  dim3 grid((N + block_rows - 1) / block_rows, parts, (unsigned)m_tiles);
   const long long up_offset = (long long)N * ldw;
-#define FE_GO(MT, EPI, R)                                                                                   \
-  gemm_wide_kernel<MT, EPI, R><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, \
-                                                      ldw, ldo, per_part, part_stride, up_offset)
+#define FE_GO(MT, EPI)                                                                                         \
+  do {                                                                                                         \
+    if (block_rows == 64)                                                                                      \
+      gemm_wide_kernel<MT, EPI, 4, 4><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, \
+                                                                ldw, ldo, per_part, part_stride, up_offset);   \
+    else                                                                                                       \
+      gemm_wide_kernel<MT, EPI, 4, 2><<<grid, 128, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, \
+                                                                ldw, ldo, per_part, part_stride, up_offset);   \
+  } while (0)
   if (mt == 4) {
-    if (ending == EPI_PARTS) FE_GO(4, EPI_PARTS, 4); else if (ending == EPI_BF16) FE_GO(4, EPI_BF16, 4); else FE_GO(4, EPI_SWIGLU, 4);
+    if (ending == EPI_PARTS) FE_GO(4, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(4, EPI_BF16); else FE_GO(4, EPI_SWIGLU);
   } else {
-    if (ending == EPI_PARTS) FE_GO(8, EPI_PARTS, 4); else if (ending == EPI_BF16) FE_GO(8, EPI_BF16, 4); else FE_GO(8, EPI_SWIGLU, 4);
+    if (ending == EPI_PARTS) FE_GO(8, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(8, EPI_BF16); else FE_GO(8, EPI_SWIGLU);
   }
 #undef FE_GO
   return fe_check_launch();

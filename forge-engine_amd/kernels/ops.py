@@ -245,8 +245,9 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
         raise KernelError(f"activation {x.dtype} does not match weight {weight.dtype}")
     if bias is None and _skinny_fits(x, weight) and out_dtype in (torch.float32, torch.bfloat16):
         return gemm_skinny(x, weight, "f32" if out_dtype == torch.float32 else "bf16")
-    if bias is None and out_dtype == torch.bfloat16 and _wide_fits(x, weight, WIDE_STORE_MAX_ROWS):
-        return gemm_wide(x, weight, "bf16", row_tile=64 if x.shape[0] <= 128 else 128)
+    if bias is None and out_dtype == torch.bfloat16 and _wide_fits(x, weight, WIDE_STORE_MAX_ROWS, SKINNY_MAX_ROWS + 1):
+        rows = x.shape[0]        # up to 64 rows: blocks of 32 weight rows, so that the launch has twice the blocks
+        return gemm_wide(x, weight, "bf16", row_tile=64 if rows <= 128 else 128, block_rows=32 if rows <= 64 else 64)
     if out_dtype == torch.float32:
         y = torch.mm(x, weight.t(), out_dtype=torch.float32)
     else:
@@ -306,7 +307,8 @@ def gemm_mid_parts(x: Tensor, weight: Tensor, parts: int) -> Tensor:
 # hidden size (2560 weight rows; K = 4096 / 9728) in parts of K take 14 / 22 us at 128 rows (library 28 / 53),
 # 17 / 32 us at 256 rows (25 / 46), 21 / 43 at 384 (24 / 47) and lose from 512 rows on; the q/k/v product
 # (6144 weight rows) takes 18 - 20 us at 96 and 128 rows in row tiles of 64 and 23 - 26 us at 192 and 256 rows
-# in tiles of 128 (library 24 and 27 - 33); the gate/up
+# in tiles of 128 (library 24 and 27 - 33), 15 - 16 us at 32 and 64 rows in blocks of 32 weight rows (library
+# 20 - 23); the gate/up
 # product (19456 weight rows) is the library's at every row count above 64 (55 against 52 us at 256 rows).
 WIDE_UPDATE_MAX_ROWS = 384     # most rows of x for which a product in parts of K beats the matrix library
 WIDE_STORE_MAX_ROWS = 256      # ... and a product that stores bfloat16
@@ -314,15 +316,16 @@ WIDE_MAX_WEIGHT_ROWS = 8192    # weights with more rows fill the chip in the lib
 WIDE_TARGET_BLOCKS = 480       # blocks the product aims at when it cuts K into parts (two resident a CU)
 
 
-def _wide_fits(x: Tensor, weight: Tensor, most_rows: int) -> bool:
+def _wide_fits(x: Tensor, weight: Tensor, most_rows: int, least_rows: int = MID_ROWS + 1) -> bool:
     return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2 and x.is_contiguous()
-            and MID_ROWS < x.shape[0] <= most_rows and weight.dim() == 2 and weight.stride(1) == 1
+            and least_rows <= x.shape[0] <= most_rows and weight.dim() == 2 and weight.stride(1) == 1
             and weight.shape[0] <= WIDE_MAX_WEIGHT_ROWS
             and weight.shape[1] == x.shape[1] and x.shape[1] % 64 == 0 and weight.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def gemm_wide(x: Tensor, weight: Tensor, ending: str = "bf16", parts: int = 1, row_tile: int = 0) -> Tensor:
+def gemm_wide(x: Tensor, weight: Tensor, ending: str = "bf16", parts: int = 1, row_tile: int = 0,
+              block_rows: int = 64) -> Tensor:
     """x @ weight^T for a few dozen to a few hundred bfloat16 rows: ``"parts"`` float32 partial sums
     [parts, M, N] over runs of whole 64-steps of K, ``"bf16"`` [M, N], or ``"swiglu"``: silu(gate) * up
     [M, N / 2] for a fused gate/up weight (gate rows first)."""
@@ -343,7 +346,7 @@ def gemm_wide(x: Tensor, weight: Tensor, ending: str = "bf16", parts: int = 1, r
         raise KernelError(f"no ending {ending!r} with {parts} parts")
     _call("gemm_wide", "fe_gemm_wide", _ptr(x), _ptr(weight), _ptr(out), c_int(m), c_int(cols), c_int(k),
           c_longlong(weight.stride(0)), c_longlong(cols), c_int(code), c_int(parts), c_longlong(m * cols),
-          c_int(row_tile or (64 if m <= 64 else 128)), _stream())
+          c_int(row_tile or (64 if m <= 64 else 128)), c_int(block_rows), _stream())
     return out
 
 

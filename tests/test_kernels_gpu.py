@@ -621,7 +621,7 @@ def test_gemm_wide_parts(ops, m, n, k, parts, row_tile):
     x = rand(g, m, k, dtype=torch.bfloat16)
     w_full = rand(g, n, k + 8, dtype=torch.bfloat16, scale=0.05)
     w = w_full[:, :k]
-    got = ops.gemm_wide(x.to(DEV), w_full.to(DEV)[:, :k], "parts", parts, row_tile)
+    got = ops.gemm_wide(x.to(DEV), w_full.to(DEV)[:, :k], "parts", parts, row_tile, 32 if m == 100 else 64)
     assert got.shape == (parts, m, n)
     want = x.float() @ w.float().t()
     torch.testing.assert_close(got.sum(0).cpu(), want, atol=1e-3 * (k / 256) ** 0.5, rtol=1e-3)
@@ -640,10 +640,10 @@ def test_gemm_wide_stores_and_gates(ops, m, n, k):
     x = rand(g, m, k, dtype=torch.bfloat16)
     w = rand(g, n, k, dtype=torch.bfloat16, scale=0.05)
     want = x.float() @ w.float().t()
-    for row_tile in (64, 128):
-        got = ops.gemm_wide(x.to(DEV), w.to(DEV), "bf16", 1, row_tile)
+    for row_tile, block_rows in ((64, 64), (128, 64), (64, 32), (128, 32)):      # blocks of four waves or two
+        got = ops.gemm_wide(x.to(DEV), w.to(DEV), "bf16", 1, row_tile, block_rows)
         torch.testing.assert_close(got.cpu().float(), want.to(torch.bfloat16).float(), atol=2e-2, rtol=2e-2)
-        gated = ops.gemm_wide(x.to(DEV), w.to(DEV), "swiglu", 1, row_tile)
+        gated = ops.gemm_wide(x.to(DEV), w.to(DEV), "swiglu", 1, row_tile, block_rows)
         gate, up = want[:, :n // 2], want[:, n // 2:]
         torch.testing.assert_close(gated.cpu().float(), (gate / (1 + torch.exp(-gate)) * up), atol=2e-2, rtol=2e-2)
         assert gated.shape == (m, n // 2)
