@@ -129,7 +129,9 @@ def test_add_rows_and_swiglu(ops, dtype):
 @pytest.mark.parametrize("m,n,k", [(1, 1, 1), (3, 70, 50), (65, 129, 96), (130, 64, 2560), (17, 1003, 200), (5, 33, 7),
                                    # up to 16 rows with K a multiple of four: the weight-streaming variant
                                    (1, 9003, 2560), (3, 70, 52), (4, 2560, 4096), (8, 2560, 9728), (7, 1003, 200), (16, 330, 1028),
-                                   (13, 6, 4), (9, 5, 1024)])
+                                   (13, 6, 4), (9, 5, 1024),
+                                   # up to 8 rows and K from 1,024: the rows of A stay in registers (K in one, two or three passes)
+                                   (8, 1003, 2560), (5, 7, 1024), (8, 2561, 3072), (2, 600, 4096), (8, 300, 6148), (6, 131, 12292), (1, 70, 1500)])
 def test_gemm_f32(ops, m, n, k):
     g = torch.Generator().manual_seed(4)
     a, b, bias = rand(g, m, k), rand(g, n, k), rand(g, n)
@@ -138,12 +140,13 @@ def test_gemm_f32(ops, m, n, k):
     torch.testing.assert_close(got, want, atol=1e-4 * math.sqrt(k), rtol=1e-5)
     # a row's result does not depend on the rows beside it
     alone = ops.gemm_nt_f32(a[:1].to(DEV).contiguous(), b.to(DEV), bias.to(DEV)).cpu()
-    if m <= 16 or k % 4:
+    if (m <= 8 or k < 1024 or k % 4) and (m <= 16 or k % 4):
         assert torch.equal(alone[0], got[0])        # the same variant, whose order of sums depends on K alone
     else:                                           # few rows stream the weight, many rows take tiles: another order of the same sums
         torch.testing.assert_close(alone[0], got[0], atol=1e-5 * math.sqrt(k), rtol=1e-5)
-    for rows in (2, 5, 9, 16):                      # every variant for few rows gives the same bits
-        if rows < m <= 16:
+    resident = lambda rows: rows <= 8 and k >= 1024 and k % 4 == 0      # the variant that keeps A in registers
+    for rows in (2, 5, 9, 16):                      # the variants for few rows give the same bits within their kind
+        if rows < m <= 16 and resident(rows) == resident(m):
             part = ops.gemm_nt_f32(a[:rows].to(DEV).contiguous(), b.to(DEV), bias.to(DEV)).cpu()
             assert torch.equal(part, got[:rows])
 
