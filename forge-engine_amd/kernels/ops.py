@@ -310,7 +310,11 @@ def gemm_mid_parts(x: Tensor, weight: Tensor, parts: int) -> Tensor:
 # in tiles of 128 (library 24 and 27 - 33), 15 - 16 us at 32 and 64 rows in blocks of 32 weight rows (library
 # 20 - 23); the gate/up
 # product (19456 weight rows) is the library's at every row count above 64 (55 against 52 us at 256 rows).
-WIDE_UPDATE_MAX_ROWS = 384     # most rows of x for which a product in parts of K beats the matrix library
+WIDE_UPDATE_MAX_ROWS = 384     # most rows of x for which a product in parts of K beats the matrix library ...
+WIDE_UPDATE_SURE_ROWS = 128    # ... for weights of up to WIDE_UPDATE_FEW_WEIGHT_ROWS rows; up to this many rows it does for every
+WIDE_UPDATE_FEW_WEIGHT_ROWS = 3072   # weight measured (hidden sizes 2560, 4096, 5120: 13 - 30 us against 21 - 45 at the output
+                                     # projection, 22 - 85 against 54 - 181 at the down projection, 128 rows); at 256 rows the
+                                     # hidden size 4096 is the library's by a tenth, at 384 rows 4096 and 5120 by a sixth
 WIDE_STORE_MAX_ROWS = 256      # ... and a product that stores bfloat16
 WIDE_MAX_WEIGHT_ROWS = 8192    # weights with more rows fill the chip in the library's large tiles
 WIDE_TARGET_BLOCKS = 480       # blocks the product aims at when it cuts K into parts (two resident a CU)
@@ -380,7 +384,8 @@ def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None, stream:
         steps = -(-weight.shape[1] // 128)
         blocks = -(-weight.shape[0] // 64)
         return gemm_mid_parts(x, weight, _mid_parts(steps, blocks))
-    if plain_bf16 and _wide_fits(x, weight, WIDE_UPDATE_MAX_ROWS):
+    if plain_bf16 and _wide_fits(x, weight, WIDE_UPDATE_MAX_ROWS if weight.shape[0] <= WIDE_UPDATE_FEW_WEIGHT_ROWS
+                                 else WIDE_UPDATE_SURE_ROWS):
         return gemm_wide(x, weight, "parts", _wide_parts(x.shape[0], weight.shape[0], weight.shape[1]))
     if (plain_bf16 and stream is not None and x.shape[0] > SKINNY_MAX_ROWS and stream.dtype == torch.float32
             and stream.shape == (x.shape[0], weight.shape[0]) and stream.is_contiguous()):
