@@ -117,12 +117,13 @@ def static_batch_size(num_seqs: int, widths, num_tokens: int | None = None, num_
 
 
 def static_batch(flat: Tensor, *, num_tokens: int, num_seqs: int, num_wanted: int, widths, max_q_len: int,
-                 max_ctx: int) -> StepBatch:
+                 max_ctx: int, num_decode: int | None = None) -> StepBatch:
     """The batch of a captured step: views into a device buffer at fixed addresses, laid out as
     ``build_batch`` lays a batch out, for ``num_seqs`` sequences of which some may be empty.
     What the kernels cannot read from the buffer is a bound (``max_q_len``, ``max_ctx``) or
-    unknown (how many sequences bring one token); the host-side lists are not filled in, so a
-    model with a part that reads them is not captured."""
+    unknown (how many sequences bring one token, unless the caller knows that none ever does:
+    ``num_decode=0``); the host-side lists are not filled in, so a model with a part that reads
+    them is not captured."""
     sizes = [num_tokens, num_tokens, num_tokens, num_seqs + 1, num_seqs, num_seqs, num_seqs, num_wanted]
     views, offset = [], 0
     for size in sizes:
@@ -134,6 +135,6 @@ def static_batch(flat: Tensor, *, num_tokens: int, num_seqs: int, num_wanted: in
         offset += num_seqs * width
     return StepBatch(
         num_tokens=num_tokens, num_seqs=num_seqs, num_wanted=num_wanted, max_q_len=max_q_len, max_ctx=max_ctx,
-        num_decode=None, token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
+        num_decode=num_decode, token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
         ctx_len=views[4], ctx_before=views[5], state_slots=views[6], want_rows=views[7],
         block_tables=block_tables, request_ids=[], q_lens=[], ctx_before_host=[], state_slots_host=[])

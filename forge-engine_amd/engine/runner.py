@@ -363,7 +363,8 @@ class ModelRunner:
         seqs = -(-len(entries) // PORTION_GRAPH_SEQ_STEP) * PORTION_GRAPH_SEQ_STEP
         wanted = sum(len(e.want) for e in entries)
         wanted = -(-wanted // PORTION_GRAPH_WANT_STEP) * PORTION_GRAPH_WANT_STEP
-        return tokens, seqs, wanted
+        singles = any(len(e.tokens) == 1 for e in entries)    # a step without single tokens launches no kernel for them
+        return tokens, seqs, wanted, singles
 
     def _portion_graph_step(self, entries: list[StepEntry], shape) -> Tensor | None:
         """A step with prompt portions as a replay of a captured graph, once its shape (token
@@ -399,7 +400,8 @@ class ModelRunner:
         slot.copied.record(torch.cuda.current_stream(self.device))
         if slot.graph is None:
             batch = static_batch(slot.dev, num_tokens=shape[0], num_seqs=shape[1], num_wanted=shape[2],
-                                 widths=widths, max_q_len=shape[0], max_ctx=widths[0] * self.block_size if widths else 0)
+                                 widths=widths, max_q_len=shape[0], max_ctx=widths[0] * self.block_size if widths else 0,
+                                 num_decode=None if shape[3] else 0)
             views = self.cache_views(batch)
             self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()
