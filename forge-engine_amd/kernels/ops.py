@@ -304,20 +304,20 @@ def gemm_mid_parts(x: Tensor, weight: Tensor, parts: int) -> Tensor:
 
 
 # Measured on MI355X at Qwen3-4B's sizes against the matrix library, per call: the products back to the
-# hidden size (2560 weight rows; K = 4096 / 9728) in parts of K take 14 / 22 us at 128 rows (library 28 / 53),
-# 17 / 32 us at 256 rows (25 / 46), 21 / 43 at 384 (24 / 47) and lose from 512 rows on; the q/k/v product
+# hidden size (2560 weight rows; K = 4096 / 9728) in parts of K take 10 / 20 us at 128 rows (library 28 / 53),
+# 14 / 30 us at 256 rows (25 / 46), 18 / 41 at 384 (24 / 47) and lose from 512 rows on; the q/k/v product
 # (6144 weight rows) takes 18 - 20 us at 96 and 128 rows in row tiles of 64 and 23 - 26 us at 192 and 256 rows
 # in tiles of 128 (library 24 and 27 - 33), 15 - 16 us at 32 and 64 rows in blocks of 32 weight rows (library
-# 20 - 23); the gate/up
-# product (19456 weight rows) is the library's at every row count above 64 (55 against 52 us at 256 rows).
+# 20 - 23); the gate/up product (19456 weight rows) is the library's at every row count above 64 (55 against
+# 52 us at 256 rows).
 WIDE_UPDATE_MAX_ROWS = 384     # most rows of x for which a product in parts of K beats the matrix library ...
-WIDE_UPDATE_SURE_ROWS = 128    # ... for weights of up to WIDE_UPDATE_FEW_WEIGHT_ROWS rows; up to this many rows it does for every
-WIDE_UPDATE_FEW_WEIGHT_ROWS = 3072   # weight measured (hidden sizes 2560, 4096, 5120: 13 - 30 us against 21 - 45 at the output
-                                     # projection, 22 - 85 against 54 - 181 at the down projection, 128 rows); at 256 rows the
-                                     # hidden size 4096 is the library's by a tenth, at 384 rows 4096 and 5120 by a sixth
+WIDE_UPDATE_SURE_ROWS = 256    # ... for weights of up to WIDE_UPDATE_FEW_WEIGHT_ROWS rows; up to this many rows it does for every
+WIDE_UPDATE_FEW_WEIGHT_ROWS = 3072   # weight measured (hidden sizes 2560, 4096, 5120 at 256 rows: output projection 14 / 21 / 45 us
+                                     # against 25 / 26 / 73, down projection 30 / 55 / 146 against 46 / 59 / 178); at 384 rows the
+                                     # hidden sizes 4096 and 5120 are the library's by a tenth
 WIDE_STORE_MAX_ROWS = 256      # ... and a product that stores bfloat16
 WIDE_MAX_WEIGHT_ROWS = 8192    # weights with more rows fill the chip in the library's large tiles
-WIDE_TARGET_BLOCKS = 480       # blocks the product aims at when it cuts K into parts (two resident a CU)
+WIDE_CUS = 256                 # the product's blocks run one a CU, round after round: the parts of K are chosen to fill the rounds
 
 
 def _wide_fits(x: Tensor, weight: Tensor, most_rows: int, least_rows: int = MID_ROWS + 1) -> bool:
@@ -355,12 +355,19 @@ def gemm_wide(x: Tensor, weight: Tensor, ending: str = "bf16", parts: int = 1, r
 
 
 def _wide_parts(m: int, n: int, k: int) -> int:
-    """Parts of K for the product above: about WIDE_TARGET_BLOCKS blocks in all, at least eight 64-steps
-    a part (the kernel fetches two steps ahead), no part without steps."""
+    """Parts of K for the product above.  Its blocks run one a CU in rounds, so the count of parts is
+    the one whose blocks fill their rounds best (measured at 40 to 160 blocks a part: 240 blocks beat
+    280 and 320, 480 beat 160 and 320), the smaller of near equals (every part writes and the consumer
+    reads a partial sum of the whole result), at least eight 64-steps a part, no part without steps."""
     steps = k // 64
-    blocks = -(-n // 64) * -(-m // (64 if m <= 64 else 128))
-    parts = max(1, min(16, WIDE_TARGET_BLOCKS // blocks, steps // 8))
-    return -(-steps // -(-steps // parts))
+    base = -(-n // 64) * -(-m // (64 if m <= 64 else 128))
+    best, best_fill = 1, 0.0
+    for parts in range(1, max(1, min(16, steps // 8)) + 1):
+        blocks = base * parts
+        fill = blocks / (-(-blocks // WIDE_CUS) * WIDE_CUS) - 0.02 * parts
+        if fill > best_fill + 1e-9:
+            best, best_fill = parts, fill
+    return -(-steps // -(-steps // best))
 
 
 def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None, stream: Tensor | None = None) -> Tensor | None:
