@@ -33,6 +33,7 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 #define EPI_PARTS 0
 #define EPI_BF16 1
 #define EPI_SWIGLU 2
+#define EPI_SWIGLU_HALF 3     // a wave's 16 weight rows are 8 gate rows and the 8 up rows that belong to them
 
 __device__ __forceinline__ float silu_times(float g, float u) { return g / (1.f + __expf(-g)) * u; }
 
@@ -42,18 +43,22 @@ template <int MT, int EPI, int R, int WPB>
 __global__ __launch_bounds__(64 * WPB, 2) void gemm_wide_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N,
     int K, long long ldw, long long ldo, int steps_per_part, long long part_stride, long long up_offset) {
-  constexpr int WF = EPI == EPI_SWIGLU ? 2 : 1;     // weight operands a wave holds: gate and up, or one
-  constexpr int XL = 2 * MT / WPB;                  // 16-byte pieces of a step of x a thread fetches
+  constexpr int WF = EPI == EPI_SWIGLU ? 2 : 1;     // weight operands a wave holds: a gate tile and an up tile, or one
   constexpr int THREADS = 64 * WPB;
+  constexpr int PIECES = MT * 128;                  // 16-byte pieces of a step of x
+  constexpr int XL = (PIECES + THREADS - 1) / THREADS;   // ... that a thread fetches (where the threads do not divide them, the last piece more than once)
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][WSTEP];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int lr = lane & 15;
   const int lq = lane >> 4;
-  const int n = blockIdx.x * (16 * WPB) + wave * 16 + lr;
+  // the weight row this lane feeds and the output column it receives: the wave's 16 rows, or, with the
+  // half-tile gate/up ending, 8 gate rows (lanes with lr < 8) and the 8 up rows of the same columns
+  const int n = EPI == EPI_SWIGLU_HALF ? blockIdx.x * (8 * WPB) + wave * 8 + (lr & 7)
+                                       : blockIdx.x * (16 * WPB) + wave * 16 + lr;
   const int m0 = blockIdx.z * MT * 16;
-  const bf16_t* wrow = w + (size_t)(n < N ? n : 0) * ldw;
+  const bf16_t* wrow = w + (size_t)(n < N ? n : 0) * ldw + (EPI == EPI_SWIGLU_HALF && lr >= 8 ? up_offset : 0);
   const int steps = K / WSTEP;
   const int first = blockIdx.y * steps_per_part;
   const int last = min(steps, first + steps_per_part);
@@ -74,7 +79,7 @@ __global__ __launch_bounds__(64 * WPB, 2) void gemm_wide_kernel(
       step = min(step, last - 1);
 #pragma unroll
       for (int i = 0; i < XL; ++i) {
-        const int p = tid + THREADS * i;
+        const int p = min(tid + THREADS * i, PIECES - 1);
         const int row = m0 + (p >> 3);
         xdst[i] = *(const uintx4*)(x + (size_t)(row < M ? row : 0) * K + step * WSTEP + (p & 7) * 8);
       }
@@ -90,7 +95,7 @@ __global__ __launch_bounds__(64 * WPB, 2) void gemm_wide_kernel(
     auto store_x = [&](int stage, const uintx4* xsrc) {
 #pragma unroll
       for (int i = 0; i < XL; ++i) {
-        const int p = tid + THREADS * i;
+        const int p = min(tid + THREADS * i, PIECES - 1);
         const int row = p >> 3;
         *(uintx4*)&xs[stage][row][((p & 7) ^ (row & 7)) * 8] = xsrc[i];
       }
@@ -153,9 +158,14 @@ __global__ __launch_bounds__(64 * WPB, 2) void gemm_wide_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int m = m0 + mt * 16 + lq * 4 + i;
-        if (m >= M) continue;
+        if (EPI != EPI_SWIGLU_HALF && m >= M) continue;      // (the half-tile ending exchanges between lanes first)
         if (EPI == EPI_PARTS) ((float*)out)[(size_t)blockIdx.y * part_stride + (size_t)m * ldo + n] = acc[0][mt][i];
         else if (EPI == EPI_BF16) ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(acc[0][mt][i]);
+        else if (EPI == EPI_SWIGLU_HALF) {
+          // the lane 8 further in its row of 16 holds the up projection of this lane's column (and the other way round)
+          const float other = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(acc[0][mt][i]), 0x128, 0xF, 0xF, true));
+          if (lr < 8 && m < M) ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(silu_times(acc[0][mt][i], other));
+        }
         else ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(silu_times(acc[0][mt][i], acc[WF - 1][mt][i]));
       }
   }
@@ -167,7 +177,11 @@ __global__ __launch_bounds__(64 * WPB, 2) void gemm_wide_kernel(
 //   has no steps), so the caller may add all of them up.
 // ending 1: out is bfloat16 [M, N] with row stride ldo; parts must be 1.
 // ending 2: w is a fused gate/up weight [2 N, K], gate rows first; out is bfloat16 [M, N] =
-//   silu(x gate^T) * (x up^T); parts must be 1.
+//   silu(x gate^T) * (x up^T); parts must be 1.  A wave multiplies 16 gate rows and their 16 up rows.
+// ending 3: the same result with 8 gate rows and their 8 up rows a wave (one weight operand, the two halves
+//   of a result tile meet by a lane exchange), so that a block takes 8 columns a wave: block_rows = 32 to 64
+//   in steps of 8 (four to eight waves) is then the block's columns, chosen so that the blocks fill rounds of
+//   one a CU.
 // Any M: rows are taken in tiles of row_tile = 64 or 128 (smaller tiles: more blocks, and the weight
 // read again, from L2, once per tile).  block_rows = 64 or 32: the weight rows (gate/up ending: output
 // columns) a block of four or two waves takes; 32 gives a launch of few blocks twice as many.
@@ -177,7 +191,7 @@ extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int 
   if (M < 1) return FE_OK;
   if (N < 1 || K < WSTEP || K % WSTEP || ldw < K || ldw % 8 || ldo < N) return FE_BAD_ARGUMENT;
   if ((((uintptr_t)x) & 15) || (((uintptr_t)w) & 15)) return FE_BAD_ARGUMENT;
-  if (ending < EPI_PARTS || ending > EPI_SWIGLU) return FE_BAD_ARGUMENT;
+  if (ending < EPI_PARTS || ending > EPI_SWIGLU_HALF) return FE_BAD_ARGUMENT;
   if (parts < 1 || parts > 64 || (ending != EPI_PARTS && parts != 1)) return FE_BAD_ARGUMENT;
   if (parts > 1 && part_stride < (long long)M * ldo) return FE_BAD_ARGUMENT;
   const int steps = K / WSTEP;
@@ -186,23 +200,34 @@ extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int 
   const int mt = row_tile / 16;
   const long long m_tiles = (M + mt * 16 - 1) / (mt * 16);
   if (m_tiles > 65535) return FE_BAD_ARGUMENT;
-  if (block_rows != 64 && block_rows != 32) return FE_BAD_ARGUMENT;
+  if (ending == EPI_SWIGLU_HALF ? (block_rows < 32 || block_rows > 64 || block_rows % 8) : (block_rows != 64 && block_rows != 32))
+    return FE_BAD_ARGUMENT;
   dim3 grid((N + block_rows - 1) / block_rows, parts, (unsigned)m_tiles);
   const long long up_offset = (long long)N * ldw;
-#define FE_GO(MT, EPI)                                                                                         \
-  do {                                                                                                         \
-    if (block_rows == 64)                                                                                      \
-      gemm_wide_kernel<MT, EPI, 4, 4><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, \
-                                                                ldw, ldo, per_part, part_stride, up_offset);   \
-    else                                                                                                       \
-      gemm_wide_kernel<MT, EPI, 4, 2><<<grid, 128, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, \
-                                                                ldw, ldo, per_part, part_stride, up_offset);   \
+#define FE_LAUNCH(MT, EPI, WPB)                                                                                  \
+  gemm_wide_kernel<MT, EPI, 4, WPB><<<grid, 64 * WPB, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, \
+                                                                    ldw, ldo, per_part, part_stride, up_offset)
+#define FE_GO(MT, EPI)                                  \
+  do {                                                  \
+    if (block_rows == 64) FE_LAUNCH(MT, EPI, 4);        \
+    else FE_LAUNCH(MT, EPI, 2);                         \
+  } while (0)
+#define FE_HALF(MT)                                                                                              \
+  do {                                                                                                           \
+    const int waves = block_rows / 8;                                                                            \
+    if (waves == 4) FE_LAUNCH(MT, EPI_SWIGLU_HALF, 4); else if (waves == 5) FE_LAUNCH(MT, EPI_SWIGLU_HALF, 5);  \
+    else if (waves == 6) FE_LAUNCH(MT, EPI_SWIGLU_HALF, 6); else if (waves == 7) FE_LAUNCH(MT, EPI_SWIGLU_HALF, 7); \
+    else FE_LAUNCH(MT, EPI_SWIGLU_HALF, 8);                                                                      \
   } while (0)
   if (mt == 4) {
-    if (ending == EPI_PARTS) FE_GO(4, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(4, EPI_BF16); else FE_GO(4, EPI_SWIGLU);
+    if (ending == EPI_PARTS) FE_GO(4, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(4, EPI_BF16);
+    else if (ending == EPI_SWIGLU) FE_GO(4, EPI_SWIGLU); else FE_HALF(4);
   } else {
-    if (ending == EPI_PARTS) FE_GO(8, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(8, EPI_BF16); else FE_GO(8, EPI_SWIGLU);
+    if (ending == EPI_PARTS) FE_GO(8, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(8, EPI_BF16);
+    else if (ending == EPI_SWIGLU) FE_GO(8, EPI_SWIGLU); else FE_HALF(8);
   }
+#undef FE_HALF
 #undef FE_GO
+#undef FE_LAUNCH
   return fe_check_launch();
 }

@@ -650,6 +650,29 @@ def test_gemm_wide_stores_and_gates(ops, m, n, k):
         gate, up = want[:, :n // 2], want[:, n // 2:]
         torch.testing.assert_close(gated.cpu().float(), (gate / (1 + torch.exp(-gate)) * up), atol=2e-2, rtol=2e-2)
         assert gated.shape == (m, n // 2)
+    # the ending that takes 8 gate rows and their 8 up rows a wave, blocks of four to eight waves
+    for width in (32, 40, 48, 56, 64):
+        gated = ops.gemm_wide(x.to(DEV), w.to(DEV), "swiglu_half", 1, 64 if width != 48 else 128, width)
+        torch.testing.assert_close(gated.cpu().float(), (gate / (1 + torch.exp(-gate)) * up), atol=2e-2, rtol=2e-2)
+
+
+def test_linear_swiglu_routes_by_rows(ops, monkeypatch):
+    """Up to 16 rows: the streaming kernel; 17 to 64: the product that pairs gate and up rows within a
+    wave; more: the matrix library and the gate kernel.  All give the plain result."""
+    g = torch.Generator().manual_seed(33)
+    w = rand(g, 2 * 328, 256, dtype=torch.bfloat16, scale=0.05)
+    taken = []
+    real_call = ops._call
+    monkeypatch.setattr(ops, "_call", lambda lib, name, *a: taken.append(name) or real_call(lib, name, *a))
+    for rows, name in ((8, "fe_gemm_skinny"), (17, "fe_gemm_wide"), (64, "fe_gemm_wide"), (65, "fe_swiglu")):
+        x = rand(g, rows, 256, dtype=torch.bfloat16)
+        taken.clear()
+        got = ops.linear_swiglu(x.to(DEV), w.to(DEV)).cpu().float()
+        assert taken[-1] == name, taken
+        y = x.float() @ w.float().t()
+        gate, up = y[:, :328], y[:, 328:]
+        torch.testing.assert_close(got, gate / (1 + torch.exp(-gate)) * up, atol=2e-2, rtol=2e-2)
+    assert ops._gate_block_columns(9728) == 40 and ops._gate_block_columns(12288) == 48
 
 
 def test_gemm_wide_refuses_and_routes(ops, monkeypatch):
