@@ -69,14 +69,34 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// The same over the data-parallel lane permutes and the lane swaps: no trip through the LDS
+// crossbar (six of them, each with a wait behind it, in the forms above).  Another order of the
+// same additions, so not for code whose bits another kernel has to reproduce.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));    // lane ^ 1
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));    // lane ^ 2
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));   // 7 - lane within 8
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));   // 15 - lane within 16
+  return sum_xor32(sum_xor16(v));
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true)));
+  return max_xor32(max_xor16(v));
+}
+
 // Sum over a block of up to 1024 threads; `scratch` holds one float per wave
-// (at least 16).  Every thread gets the total.  Contains two barriers.
+// (at least 16).  Every thread gets the total.  Contains two barriers, or one where nothing
+// has used `scratch` before (SCRATCH_IS_FRESH).
+template <bool SCRATCH_IS_FRESH = false>
 __device__ __forceinline__ float block_sum(float v, float* scratch) {
   const int lane = threadIdx.x & (FE_WAVE - 1);
   const int wave = threadIdx.x / FE_WAVE;
   const int waves = (blockDim.x + FE_WAVE - 1) / FE_WAVE;
-  v = wave_sum(v);
-  __syncthreads();
+  v = wave_sum_dpp(v);
+  if (!SCRATCH_IS_FRESH) __syncthreads();
   if (lane == 0) scratch[wave] = v;
   __syncthreads();
   float total = 0.f;
@@ -88,7 +108,7 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   const int lane = threadIdx.x & (FE_WAVE - 1);
   const int wave = threadIdx.x / FE_WAVE;
   const int waves = (blockDim.x + FE_WAVE - 1) / FE_WAVE;
-  v = wave_max(v);
+  v = wave_max_dpp(v);
   __syncthreads();
   if (lane == 0) scratch[wave] = v;
   __syncthreads();

@@ -68,7 +68,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
     }
     sumsq += v * v;
   }
-  const float total = block_sum(sumsq, scratch);
+  const float total = block_sum<true>(sumsq, scratch);
   const float inv = rsqrtf(total / (float)hidden + eps);
   TO* orow = out + (size_t)r * hidden;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_regs_kernel(
       sumsq += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
     }
   }
-  const float total = block_sum(sumsq, scratch);
+  const float total = block_sum<true>(sumsq, scratch);
   const float inv = rsqrtf(total / (float)hidden + eps);
   TO* orow = out + (size_t)r * hidden;
 #pragma unroll
