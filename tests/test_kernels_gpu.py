@@ -1132,6 +1132,33 @@ def test_prefill_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size):
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("num_seqs", [40, 64, 65, 130])
+def test_prefill_attention_kernel_places_every_tile(ops, num_seqs):
+    """The kernel's grid holds a place for every 64-row tile there may be (the host knows only the
+    step's tokens and sequences) and every block finds its sequence and tile on the device: up to 64
+    sequences by a search with a lane a sequence, more one after the other.  Sequences of every
+    kind side by side: empty ones (a captured step pads with them), single tokens, one to four tiles,
+    with and without cached context."""
+    g = torch.Generator().manual_seed(50 + num_seqs)
+    lengths = torch.randint(0, 7, (num_seqs,), generator=g).tolist()
+    seqs = []
+    for kind in lengths:
+        q_len = {0: 0, 1: 1, 2: 2, 3: 64, 4: 65, 5: 130, 6: 200}[kind]
+        before = int(torch.randint(0, 90, (1,), generator=g)) if kind % 2 else 0
+        seqs.append((before if q_len else 16, q_len))
+    q_heads, kv_heads, head_dim, block_size = 8, 2, 64, 16
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                extra_width=2 * kv_heads * head_dim)
+    kw = dict(num_seqs=len(seqs), max_q_len=200, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+              scale=head_dim ** -0.5)
+    want = refs.paged_attention(q, kp, vp, torch.empty(q.shape[0], q_heads * head_dim, dtype=q.dtype), cu, ctx, table, **kw).float()
+    got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV),
+                              torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
+                              cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=None, max_ctx=300, **kw).cpu().float()
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("window", [None, 100, 700])
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [(8, 2, 128, 16), (6, 3, 64, 32)])
 @pytest.mark.parametrize("key_groups", [1, 2])
