@@ -184,7 +184,8 @@ __global__ __launch_bounds__(64 * WPB, 2) void gemm_wide_kernel(
 //   one a CU.
 // Any M: rows are taken in tiles of row_tile = 64 or 128 (smaller tiles: more blocks, and the weight
 // read again, from L2, once per tile).  block_rows = 64 or 32: the weight rows (gate/up ending: output
-// columns) a block of four or two waves takes; 32 gives a launch of few blocks twice as many.
+// columns) a block of four or two waves takes; 32 gives a launch of few blocks twice as many; 128 (eight
+// waves, plain endings) halves how often x is read.
 extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int N, int K, long long ldw,
                             long long ldo, int ending, int parts, long long part_stride, int row_tile,
                             int block_rows, hipStream_t stream) {
@@ -200,7 +201,7 @@ extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int 
   const int mt = row_tile / 16;
   const long long m_tiles = (M + mt * 16 - 1) / (mt * 16);
   if (m_tiles > 65535) return FE_BAD_ARGUMENT;
-  if (ending == EPI_SWIGLU_HALF ? (block_rows < 32 || block_rows > 64 || block_rows % 8) : (block_rows != 64 && block_rows != 32))
+  if (ending == EPI_SWIGLU_HALF ? (block_rows < 32 || block_rows > 64 || block_rows % 8) : (block_rows != 128 && block_rows != 64 && block_rows != 32))
     return FE_BAD_ARGUMENT;
   dim3 grid((N + block_rows - 1) / block_rows, parts, (unsigned)m_tiles);
   const long long up_offset = (long long)N * ldw;
@@ -209,7 +210,8 @@ extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int 
                                                                     ldw, ldo, per_part, part_stride, up_offset)
 #define FE_GO(MT, EPI)                                  \
   do {                                                  \
-    if (block_rows == 64) FE_LAUNCH(MT, EPI, 4);        \
+    if (block_rows == 128) FE_LAUNCH(MT, EPI, 8);       \
+    else if (block_rows == 64) FE_LAUNCH(MT, EPI, 4);   \
     else FE_LAUNCH(MT, EPI, 2);                         \
   } while (0)
 #define FE_HALF(MT)                                                                                              \

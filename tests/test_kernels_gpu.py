@@ -624,7 +624,7 @@ def test_gemm_wide_parts(ops, m, n, k, parts, row_tile):
     x = rand(g, m, k, dtype=torch.bfloat16)
     w_full = rand(g, n, k + 8, dtype=torch.bfloat16, scale=0.05)
     w = w_full[:, :k]
-    got = ops.gemm_wide(x.to(DEV), w_full.to(DEV)[:, :k], "parts", parts, row_tile, 32 if m == 100 else 64)
+    got = ops.gemm_wide(x.to(DEV), w_full.to(DEV)[:, :k], "parts", parts, row_tile, {100: 32, 130: 128, 300: 128}.get(m, 64))
     assert got.shape == (parts, m, n)
     want = x.float() @ w.float().t()
     torch.testing.assert_close(got.sum(0).cpu(), want, atol=1e-3 * (k / 256) ** 0.5, rtol=1e-3)
