@@ -87,7 +87,7 @@ def parse_args():
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
     parser.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
     parser.add_argument("--points", default=None, help="other decode batch sizes to report")
-    parser.add_argument("--phase", choices=("all", "decode", "prefill"), default="all",
+    parser.add_argument("--phase", choices=("all", "decode", "prefill", "micro"), default="all",
                         help="run one phase only (for profiles); the record then holds that phase alone")
     parser.add_argument("--through", choices=("step", "scheduler"), default="step",
                         help="decode by calling the step function, or through the scheduler's step()")
@@ -137,11 +137,69 @@ def spread(times_ms: list[float]) -> dict:
             "max": round(ordered[-1], 4)}
 
 
+def micro_benchmarks() -> int:
+    """The three kernel measurements that the reference publishes (docs/benchmarks.md:27-29,
+    results/l4-v0.1.0.json:51-65; one NVIDIA L4), with its shapes and its protocol
+    (tools/validate_l4.py:136-183: 10 warm-up calls, 50 timed ones, a pair of device events around
+    each call, the median), on this engine's kernels.  A call is timed as the reference times it,
+    from the host, so a few microseconds of every figure are the launch."""
+    import torch
+
+    from forge_engine_amd.kernels import ops
+
+    device = torch.device("cuda:0")
+    generator = torch.Generator(device=device).manual_seed(0)
+
+    def rand(*shape, dtype=torch.bfloat16):
+        return torch.randn(*shape, generator=generator, device=device, dtype=torch.float32).to(dtype)
+
+    def measure(fn):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(50)]
+        for begin, end in events:
+            begin.record()
+            fn()
+            end.record()
+        torch.cuda.synchronize()
+        return spread([begin.elapsed_time(end) for begin, end in events])
+
+    record = {"phase": "micro", "protocol": "10 warm-up, 50 timed, device events around each call, milliseconds"}
+
+    # residual add + RMSNorm, [512, 2560]: the stream is float32 here, the update and the result bfloat16
+    stream, update = rand(512, 2560, dtype=torch.float32), rand(512, 2560)
+    weight, normed = rand(2560, dtype=torch.float32), torch.empty(512, 2560, dtype=torch.bfloat16, device=device)
+    record["residual_add_rms_norm_512x2560"] = dict(measure(lambda: ops.add_rmsnorm(stream, update, weight, 1e-6, normed)),
+                                                    reference_l4_ms=0.0850)
+
+    def paged(context, q_tokens, q_heads, kv_heads):
+        pages = -(-context // 16)
+        keys, values = rand(pages + 1, kv_heads, 16, 128), rand(pages + 1, kv_heads, 128, 16)
+        q = rand(q_tokens, q_heads * 128)
+        out = torch.empty(q_tokens, q_heads * 128, dtype=torch.bfloat16, device=device)
+        cu = torch.tensor([0, q_tokens], dtype=torch.int32, device=device)
+        ctx = torch.tensor([context], dtype=torch.int32, device=device)
+        table = torch.arange(pages, dtype=torch.int32, device=device).view(1, pages)
+        return lambda: ops.paged_attention(q, keys, values, out, cu, ctx, table, num_seqs=1, max_q_len=q_tokens,
+                                           q_heads=q_heads, kv_heads=kv_heads, head_dim=128, scale=128 ** -0.5,
+                                           num_decode=1 if q_tokens == 1 else 0, max_ctx=context)
+
+    # causal attention of a 128-token prompt, 8 heads of 128 (the reference's [1, 8, 128, 128]), over the paged cache
+    record["causal_prefill_1x8x128x128"] = dict(measure(paged(128, 128, 8, 8)), reference_l4_ms=0.0891)
+    # one decoded token over 127 cached keys and its own, 32 query heads, 8 kv heads of 128, pages of 16
+    record["paged_gqa_decode_past127_q32_kv8"] = dict(measure(paged(128, 1, 32, 8)), reference_l4_ms=0.1004)
+    print(json.dumps(record))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2
+    if args.phase == "micro":
+        return micro_benchmarks()
     import torch
 
     from forge_engine_amd.config import SchedulerConfig, load_model_config
