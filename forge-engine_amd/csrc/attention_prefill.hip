@@ -308,18 +308,19 @@ __global__ __launch_bounds__(256 * KG, 4) void paged_prefill_kernel(   // four w
       // lane (lr = query row, lq): st[blk][h][i] = score of key key_base + 32 blk + 8lq + 4h + i
       const bool edge = key_base + BN - 1 > wave_lo || (window > 0 && key_base < pos_hi - window + 1);
       float s[16];
-      float mx = -INFINITY;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        float v = st[j >> 3][(j >> 2) & 1][j & 3];
-        if (edge) {
+      for (int j = 0; j < 16; ++j) s[j] = st[j >> 3][(j >> 2) & 1][j & 3];
+      if (edge) {          // one branch a tile, not one a score: the tiles in the middle of a walk skip all of it
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
           const int key = key_base + 32 * (j >> 3) + 8 * lq + (j & 7);
           const bool visible = key <= row_pos && (window <= 0 || key > row_pos - window);
-          v = visible ? v : -INFINITY;
+          s[j] = visible ? s[j] : -INFINITY;
         }
-        s[j] = v;
-        mx = fmaxf(mx, v);
       }
+      float mx = s[0];
+#pragma unroll
+      for (int j = 1; j < 16; ++j) mx = fmaxf(mx, s[j]);
       mx = max_xor16(mx);
       mx = max_xor32(mx);
       const float m_new = fmaxf(m_run, mx * scale_log2);   // the scale is positive
