@@ -16,7 +16,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 
 from .allocator import BlockAllocator, CacheCapacityError, StateSlotPool
-from .spec import CacheNeeds, PagedKV
+from .spec import CacheNeeds
 
 NO_PAGE = -1
 

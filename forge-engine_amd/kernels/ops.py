@@ -8,7 +8,6 @@ implementation: without a GPU or without the compiled library a call raises.
 
 from __future__ import annotations
 
-import ctypes
 import threading
 from ctypes import c_float, c_int, c_longlong, c_void_p
 
