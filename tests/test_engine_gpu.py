@@ -1073,6 +1073,35 @@ def test_schedules_at_the_large_widths(mode, dtype, wide_folder, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_portions_at_the_large_widths(dtype, wide_folder, tmp_path):
+    """Portions of 65 to 400 tokens at the widths of the large model: the row counts at which the
+    products for portions of prompts run (parts of K in row tiles of 128, the stored q/k/v product in
+    tiles of 64 and 128, blocks of eight waves for the long K) and, beyond them, the matrix library
+    that adds into the stream as it stores; a step of two portions beside each other; the second and
+    later portions read what the first left in the cache.  Logits at each portion's last token."""
+    folder, config, weights = wide_folder
+    requests = ru.make_requests(config, 73, (700, 330, 129))
+    trace = ru.TraceBuilder(False)
+    a, b, c = (requests[key] for key in sorted(requests))
+    ida, idb, idc = sorted(requests)
+    trace.step([(ida, a[:130])])                         # 130 rows
+    trace.step([(ida, a[130:330]), (idb, b[:65])])       # 265 rows in one step, two requests
+    trace.step([(ida, a[330:700])], end=[ida])           # 370 rows
+    trace.step([(idb, b[65:330])], end=[idb])            # 265 rows
+    trace.step([(idc, c[:100])])                         # 100 rows
+    trace.step([(idc, c[100:129])], end=[idc])
+    rows = {key for keys in trace.rows.values() for key in keys}
+    got = ru.run_trace(folder, dtype, trace, tmp_path, block_size=16)
+    want = {}
+    for request_id, tokens in requests.items():
+        positions = sorted(position for rid, position in rows if rid == request_id)
+        for row, position in zip(plain.forward(weights, config, tokens, rows=positions), positions):
+            want[(request_id, position)] = row
+    assert len(want) == 7
+    ru.compare(got, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_scheduler_with_sixty_four_rows_at_the_large_widths(dtype, wide_folder):
     """Forty requests through the scheduler at its largest batch (64 requests a step, 256 tokens):
     prompts are cut into portions beside decoded tokens, and decode steps of 17 to 40 rows replay
