@@ -461,7 +461,10 @@ extern "C" int fe_paged_attention_prefill(const void* q, long long q_stride, con
   // two tiles; with more blocks than that one group is faster (eight prompts of 1,024 tokens:
   // 126 against 141 us).
   if (key_groups < 0 || key_groups > 2) return FE_BAD_ARGUMENT;
-  if (key_groups == 0) key_groups = ((long long)heads * slots <= 1024 && max_q_len >= 128) ? 2 : 1;
+  // (counted by the tiles that the tokens can fill, not by the grid: a captured launch is laid out
+  // for more sequences than a step brings, and a block without a tile ends at once)
+  const long long filled = std::min<long long>(slots, (total_q + 63) / 64);
+  if (key_groups == 0) key_groups = ((long long)heads * filled <= 1024 && max_q_len >= 128) ? 2 : 1;
 #define FE_GO(DD, GG)                                                                                            \
   paged_prefill_kernel<DD, GG><<<grid, 256 * GG, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)key_pages, \
       (const bf16_t*)value_pages, (bf16_t*)out, out_stride, cu_q, ctx_len, block_table, table_stride,            \
