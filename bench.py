@@ -309,7 +309,7 @@ def main() -> int:
     capacity = max(args.batch * -(-args.context // args.block_size), max(batches) * per_request,
                    -(-(args.prefill_tokens + 1) // args.block_size))
     runner = ModelRunner(model, block_size=args.block_size, block_capacity=capacity,
-                         num_state_slots=max(batches) + 1)
+                         num_state_slots=max(batches) + 1, eager_sightings=1)   # the timed loops repeat one shape
 
     def decode_run(batch):
         names = [f"d{batch}_{i}" for i in range(batch)]

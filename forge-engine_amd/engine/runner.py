@@ -22,6 +22,13 @@ GRAPH_LIMIT = 24             # captured graphs kept (least recently used goes fi
 PORTION_GRAPH_MAX_TOKENS = 4096   # steps with prompt portions of up to this many tokens may be captured
 PORTION_GRAPH_SEQ_STEP = 8        # ... for a number of sequences rounded up to a multiple of this
 PORTION_GRAPH_WANT_STEP = 8       # ... and of wanted rows likewise (none stays none)
+# A capture costs two more runs of the step (the warm-up and the replay after a capture that runs
+# nothing), and a replay saves the host's launches only: measured 0.2 ms a step, 3 % of a step of 256
+# tokens and 1 % of one of 2,048.  So a shape is captured once it has come this often, the more often
+# the larger the step: a workload of mixed prompts repeats few of its large shapes, and capturing each
+# on its second sighting cost it 6 % of its time.
+PORTION_GRAPH_SIGHTINGS = 2       # a shape is captured on this sighting ...
+PORTION_GRAPH_SIGHTINGS_PER = 128  # ... plus one for every so many tokens of the step
 
 
 class _DecodeGraph:
@@ -148,8 +155,12 @@ class _PortionGraph:
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, *, block_size: int, block_capacity: int,
-                 num_state_slots: int, use_graphs: bool = True) -> None:
+                 num_state_slots: int, use_graphs: bool = True, eager_sightings: int | None = None) -> None:
+        """``eager_sightings``: how often a shape of a step with prompt portions runs eagerly before
+        it is captured (None: by the step's size, see ``PORTION_GRAPH_SIGHTINGS``; a loop that repeats
+        one shape, a benchmark for instance, passes 1)."""
         self.model = model
+        self.eager_sightings = eager_sightings
         self.use_graphs = use_graphs and model.ctx.device.type == "cuda" and model.graph_safe
         self._graphs: dict[tuple, _DecodeGraph] = {}
         self._steady: _SteadyDecode | None = None
@@ -369,8 +380,8 @@ class ModelRunner:
     def _portion_graph_step(self, entries: list[StepEntry], shape) -> Tensor | None:
         """A step with prompt portions as a replay of a captured graph, once its shape (token
         count, sequence and wanted-row counts rounded up, table widths rounded up) has come
-        before: a scheduler that fills its token budget repeats few shapes.  None if the step
-        is to run eagerly (first sighting of a shape)."""
+        often enough: a scheduler that fills its token budget repeats few shapes.  None if the
+        step is to run eagerly (the first sightings of a shape)."""
         cache = self.cache
         self._check(entries)
         records = [cache.request(e.request_id) for e in entries]
@@ -386,7 +397,10 @@ class ModelRunner:
             if len(self._portion_seen) >= 4 * GRAPH_LIMIT:
                 self._portion_seen.pop(next(iter(self._portion_seen)))
             self._portion_seen[key] = seen + 1
-            if seen == 0:
+            eager = self.eager_sightings
+            if eager is None:
+                eager = PORTION_GRAPH_SIGHTINGS - 1 + shape[0] // PORTION_GRAPH_SIGHTINGS_PER
+            if seen < eager:
                 return None
             if len(self._portion_graphs) >= GRAPH_LIMIT:
                 self._portion_graphs.pop(next(iter(self._portion_graphs)))
