@@ -613,7 +613,7 @@ def test_gemm_mid_parts(ops, m, n, k, parts):
     assert torch.equal(ops.add_rows(h1, got), ops.add_rows(h2, summed))
 
 
-@pytest.mark.parametrize("m", [17, 65, 100, 128, 130, 300])
+@pytest.mark.parametrize("m", [17, 33, 64, 65, 100, 128, 130, 300])
 @pytest.mark.parametrize("n,k,parts", [(2560, 4096, 8), (200, 256, 2), (1003, 1024, 3), (64, 64, 1), (70, 640, 5), (330, 9728, 16)])
 @pytest.mark.parametrize("row_tile", [64, 128])
 def test_gemm_wide_parts(ops, m, n, k, parts, row_tile):
@@ -727,20 +727,30 @@ def test_linear_update_adds_into_the_stream_where_the_library_multiplies(ops):
     assert ops.linear_update(x, w, None, stream) is not None and torch.equal(stream, before)
 
 
-def test_linear_update_takes_the_mid_kernel(ops):
+def test_linear_update_is_in_parts_from_17_rows(ops, monkeypatch):
+    taken = []
+    real_call = ops._call
+    monkeypatch.setattr(ops, "_call", lambda lib, name, *a: taken.append(name) or real_call(lib, name, *a))
     g = torch.Generator().manual_seed(27)
     w = rand(g, 2560, 4096, dtype=torch.bfloat16, scale=0.05).to(DEV)
     for rows in (17, 40, 64):
         x = rand(g, rows, 4096, dtype=torch.bfloat16).to(DEV)
         update = ops.linear_update(x, w)
         assert update.dim() == 3 and update.shape[1:] == (rows, 2560)
+        assert update.shape[0] == 6 and taken[-1] == "fe_gemm_wide"      # 40 blocks a part: six parts fill 240 CUs
         want = x.float().cpu() @ w.float().cpu().T
         torch.testing.assert_close(update.sum(0).cpu(), want, atol=2e-3, rtol=2e-3)
-    more = rand(g, 65, 4096, dtype=torch.bfloat16).to(DEV)          # 65 rows and more: the product for portions, also in parts
+    more = rand(g, 65, 4096, dtype=torch.bfloat16).to(DEV)          # 65 rows and more: the same product, tiles of 128 rows
     update = ops.linear_update(more, w)
-    assert update.dim() == 3
+    assert update.dim() == 3 and taken[-1] == "fe_gemm_wide"
     torch.testing.assert_close(update.sum(0).cpu(), more.float().cpu() @ w.float().cpu().T, atol=2e-3, rtol=2e-3)
     assert ops.linear_update(rand(g, 400, 4096, dtype=torch.bfloat16).to(DEV), w).dim() == 2     # the library
+    # a weight of more rows than the product for portions takes: the product for 17 to 64 rows
+    tall = rand(g, 8256, 1024, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    x = rand(g, 40, 1024, dtype=torch.bfloat16).to(DEV)
+    update = ops.linear_update(x, tall)
+    assert update.dim() == 3 and taken[-1] == "fe_gemm_mid_parts"
+    torch.testing.assert_close(update.sum(0).cpu(), x.float().cpu() @ tall.float().cpu().T, atol=2e-3, rtol=2e-3)
 
 
 def test_linear_routes_by_rows_and_dtype(ops):
