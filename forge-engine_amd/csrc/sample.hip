@@ -1,7 +1,6 @@
-// Sampling over float32 logits rows: argmax, and a draw from
-// softmax(logits / temperature) by inverse CDF with a counter-based generator.
-// One block of 1024 threads per row; entries equal to -inf have probability 0
-// (that is how filters remove tokens).  Each row also gets a status word:
+// Sampling over float32 logits rows: argmax, and a draw from softmax(logits / temperature)
+// after top-k, top-p and min-p by inverse CDF with a counter-based generator, one block of
+// 1024 threads per row.  Each row also gets a status word:
 //   bit 0: a NaN was seen, bit 1: +inf was seen, bit 2: no finite entry.
 #include "common.h"
 #include "sample_api.h"
@@ -9,28 +8,6 @@
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_WAVES (SAMPLE_THREADS / FE_WAVE)
-
-__device__ __forceinline__ int row_status(const float* row, int vocab, float* scratch_f, int* scratch_i) {
-  int flags = 0;
-  int finite = 0;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float v = row[i];
-    if (v != v) flags |= 1;
-    else if (v == INFINITY) flags |= 2;
-    else if (v != -INFINITY) finite = 1;
-  }
-  // OR-reduce through LDS
-  __syncthreads();
-  if (threadIdx.x == 0) { scratch_i[0] = 0; scratch_i[1] = 0; }
-  __syncthreads();
-  if (flags) atomicOr(&scratch_i[0], flags);
-  if (finite) atomicOr(&scratch_i[1], 1);
-  __syncthreads();
-  int result = scratch_i[0];
-  if (!scratch_i[1]) result |= 4;
-  (void)scratch_f;
-  return result;
-}
 
 // tokens[row] = index of the largest entry; the lowest index wins ties.  Two
 // stages so that a few long rows still fill the chip: ARGMAX_PARTS blocks per
@@ -131,84 +108,288 @@ __device__ __forceinline__ uint32_t philox_first_word(uint32_t c0, uint32_t c1, 
   return c0;
 }
 
-// For each row: weights w_i = exp((x_i - max) / temperature); the uniform
-// u = (philox(counter = draw index, key = seed) >> 8) * 2^-24 picks the first
-// token whose running sum of weights exceeds u * total.  Thread t owns the
-// contiguous range [t * chunk, (t + 1) * chunk) so that the running sum follows
-// the token order.
-__global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(
-    const float* __restrict__ logits, long long row_stride, int vocab,
-    const float* __restrict__ temperatures, const unsigned long long* __restrict__ seeds,
-    const unsigned long long* __restrict__ draw_index, int* __restrict__ tokens,
-    int* __restrict__ status) {
-  __shared__ float red[SAMPLE_WAVES];
-  __shared__ int flags[2];
-  __shared__ float sums[SAMPLE_THREADS];
-  __shared__ int chosen;
+// ---------------------------------------------------------------------------------------------
+// One launch for rows that each bring parameters of their own: arg-max (temperature 0), or a draw
+// from softmax(logits / temperature) after top-k, top-p and min-p, in that order, each a threshold
+// on the logit: with f_i = (x_i - max) / temperature (so the largest is 0) and e_i = exp(f_i),
+//   top-k  keeps the k largest f (all of those equal to the k-th),
+//   top-p  keeps a token if the e of all larger tokens, over the e of the top-k set, is <= top_p,
+//   min-p  keeps a token if e_i >= min_p (its probability over the largest one's),
+// and the draw takes the first kept token, in token order, whose running sum of e exceeds u times
+// the total, u = (philox(counter = draw index, key = seed) >> 8) * 2^-24.
+//
+// Sums of e are sums of integers, e_i * 2^40 cut to 64 bits: they do not depend on the order of
+// the additions, so histograms by atomic adds and reductions of any shape give the same bits in
+// every run, and the place where a running sum crosses its target is exact.  A token whose e is
+// below 2^-40 of the largest one's weighs nothing.
+//
+// Thresholds are found in the space of keys: y_i = -f_i >= 0, key = the bits of y (the order of
+// non-negative floats is the order of their bits; -inf logits give y = +inf, the largest key).
+// A histogram of 2,048 bins (first linear in y up to 32, then an even split of the chosen bin's
+// range of keys, until the range is one key) holds counts for top-k or masses for top-p; a scan
+// over the bins finds the bin in which the count reaches k or the mass passes top_p * total.
+// One block of 1,024 threads a row; wave w reads the w-th sixteenth of the row, 256 entries a trip.
+struct SampleRowParams {
+  float temperature;           // 0: arg-max
+  int top_k;                   // 0: no limit
+  float top_p;                 // >= 1: no limit
+  float min_p;                 // 0: no limit
+  unsigned long long seed;
+  unsigned long long draw_index;
+};
+static_assert(sizeof(SampleRowParams) == FE_SAMPLE_PARAM_WORDS * 4, "the host packs eight words a row");
+
+#define FILTER_BINS 2048
+#define WEIGHT_SCALE 1099511627776.0f      // 2^40
+#define KEY_END 0x7f800001u                // one past the key of +inf
+
+struct FilterShared {
+  unsigned long long mass[FILTER_BINS];
+  unsigned int count[FILTER_BINS];
+  unsigned long long wave_sum[SAMPLE_WAVES];
+  float wave_best[SAMPLE_WAVES];
+  int wave_arg[SAMPLE_WAVES];
+  int wave_flags[SAMPLE_WAVES];
+  unsigned long long found_before;
+  unsigned long long target;
+  int found_bin;
+  int pick_wave;
+};
+
+// f(index, value) for every entry of the row that this thread owns: wave w owns
+// [w * segment, (w + 1) * segment), a trip takes 256 entries, a lane four neighbours.
+template <class F>
+__device__ __forceinline__ void visit_row(const float* __restrict__ row, int vocab, int segment, F f) {
+  const int lane = threadIdx.x & (FE_WAVE - 1), wave = threadIdx.x / FE_WAVE;
+  const int begin = wave * segment;
+  const int end = min(vocab, begin + segment);
+  const bool aligned = (((uintptr_t)row) & 15) == 0;
+  for (int at = begin + 4 * lane; at < end; at += 256) {
+    if (aligned && at + 3 < end) {
+      const float4 v = *(const float4*)(row + at);
+      f(at, v.x); f(at + 1, v.y); f(at + 2, v.z); f(at + 3, v.w);
+    } else {
+      for (int c = 0; c < 4 && at + c < end; ++c) f(at + c, row[at + c]);
+    }
+  }
+}
+
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+  for (int offset = FE_WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, FE_WAVE);
+  return v;
+}
+
+// Every thread gets the block's total (two barriers).
+__device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v, FilterShared& sh) {
+  v = wave_sum_u64(v);
+  __syncthreads();
+  if ((threadIdx.x & (FE_WAVE - 1)) == 0) sh.wave_sum[threadIdx.x / FE_WAVE] = v;
+  __syncthreads();
+  unsigned long long total = 0;
+  for (int w = 0; w < SAMPLE_WAVES; ++w) total += sh.wave_sum[w];
+  return total;
+}
+
+__device__ __forceinline__ unsigned long long weight_of(float y) {
+  return (unsigned long long)(expf(-y) * WEIGHT_SCALE);
+}
+
+__device__ __forceinline__ int first_bin(float y) { return (int)fminf(y * 64.f, (float)(FILTER_BINS - 1)); }
+
+// The bin in which the running total over the bins, in order, reaches the target: by counts the
+// bin with before < target <= before + own, by masses the bin with before <= target < before + own.
+// Leaves the bin in sh.found_bin (-1 if there is none) and the total before it in sh.found_before.
+template <bool BY_MASS>
+__device__ __forceinline__ void find_crossing(FilterShared& sh, unsigned long long target) {
+  const int t = threadIdx.x, lane = t & (FE_WAVE - 1), wave = t / FE_WAVE;
+  const unsigned long long a0 = BY_MASS ? sh.mass[2 * t] : sh.count[2 * t];
+  const unsigned long long a1 = BY_MASS ? sh.mass[2 * t + 1] : sh.count[2 * t + 1];
+  const unsigned long long own = a0 + a1;
+  unsigned long long upto = own;
+#pragma unroll
+  for (int offset = 1; offset < FE_WAVE; offset <<= 1) {
+    const unsigned long long other = __shfl_up(upto, offset, FE_WAVE);
+    if (lane >= offset) upto += other;
+  }
+  __syncthreads();                       // whoever still reads what the call before left has done so
+  if (lane == FE_WAVE - 1) sh.wave_sum[wave] = upto;
+  if (t == 0) sh.found_bin = -1;
+  __syncthreads();
+  unsigned long long before = upto - own;
+  for (int w = 0; w < wave; ++w) before += sh.wave_sum[w];
+  const unsigned long long before1 = before + a0;
+  const bool hit0 = BY_MASS ? (before <= target && target < before + a0) : (before < target && target <= before + a0);
+  const bool hit1 = BY_MASS ? (before1 <= target && target < before1 + a1) : (before1 < target && target <= before1 + a1);
+  if (hit0) { sh.found_bin = 2 * t; sh.found_before = before; }
+  else if (hit1) { sh.found_bin = 2 * t + 1; sh.found_before = before1; }
+  __syncthreads();
+}
+
+// The key at which the running count (top-k) or mass (top-p) over the keys, in order, reaches the
+// target, given the first histogram (already in sh) and the target.
+template <bool BY_MASS>
+__device__ __forceinline__ unsigned int find_key(const float* __restrict__ row, int vocab, int segment, float mx,
+                                                 float inv_t, unsigned long long target, FilterShared& sh) {
+  find_crossing<BY_MASS>(sh, target);
+  int bin = sh.found_bin;
+  if (bin < 0) return KEY_END - 1;              // cannot happen (the target lies below the total); keeps everything
+  target -= sh.found_before;
+  unsigned int lo = __float_as_uint((float)bin * (1.f / 64.f));
+  unsigned int hi = bin == FILTER_BINS - 1 ? KEY_END : __float_as_uint((float)(bin + 1) * (1.f / 64.f));
+  while (hi - lo > 1) {
+    const unsigned int span = hi - lo;
+    const int shift = span <= FILTER_BINS ? 0 : 32 - __clz((span - 1) >> 11);    // (span - 1) >> shift < 2048
+    __syncthreads();
+    for (int i = threadIdx.x; i < FILTER_BINS; i += SAMPLE_THREADS) {
+      if (BY_MASS) sh.mass[i] = 0; else sh.count[i] = 0;
+    }
+    __syncthreads();
+    visit_row(row, vocab, segment, [&](int, float v) {
+      const float y = (mx - v) * inv_t;
+      const unsigned int key = __float_as_uint(y);
+      if (key >= lo && key < hi) {
+        const unsigned int sub = (key - lo) >> shift;
+        if (BY_MASS) atomicAdd(&sh.mass[sub], weight_of(y)); else atomicAdd(&sh.count[sub], 1u);
+      }
+    });
+    __syncthreads();
+    find_crossing<BY_MASS>(sh, target);
+    bin = sh.found_bin;
+    if (bin < 0) return hi - 1;
+    target -= sh.found_before;
+    lo += (unsigned int)bin << shift;
+    hi = min(hi, lo + (1u << shift));
+  }
+  return lo;
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_filtered_rows_kernel(
+    const float* __restrict__ logits, long long row_stride, int vocab, const SampleRowParams* __restrict__ params,
+    int* __restrict__ tokens, int* __restrict__ status) {
+  __shared__ FilterShared sh;
   const int row_id = blockIdx.x;
   const float* row = logits + (size_t)row_id * row_stride;
-  const int st = row_status(row, vocab, red, flags);
-  if (st) {  // nothing sensible to draw from; the host raises on the status
-    if (threadIdx.x == 0) { tokens[row_id] = 0; status[row_id] = st; }
+  const int lane = threadIdx.x & (FE_WAVE - 1), wave = threadIdx.x / FE_WAVE;
+  const int segment = (vocab + SAMPLE_WAVES * 256 - 1) / (SAMPLE_WAVES * 256) * 256;
+  const SampleRowParams p = params[row_id];
+
+  // the largest entry (lowest index among equals) and what the guards look for
+  float bv = -INFINITY;
+  int bi = 0x7fffffff, flags = 0;
+  visit_row(row, vocab, segment, [&](int i, float v) {
+    if (v != v) flags |= 1;
+    else if (v == INFINITY) flags |= 2;
+    else if (v != -INFINITY) flags |= 8;
+    argmax_merge(bv, bi, v, i);
+  });
+#pragma unroll
+  for (int offset = FE_WAVE / 2; offset > 0; offset >>= 1) {
+    argmax_merge(bv, bi, __shfl_xor(bv, offset, FE_WAVE), __shfl_xor(bi, offset, FE_WAVE));
+    flags |= __shfl_xor(flags, offset, FE_WAVE);
+  }
+  if (lane == 0) { sh.wave_best[wave] = bv; sh.wave_arg[wave] = bi; sh.wave_flags[wave] = flags; }
+  __syncthreads();
+  bv = sh.wave_best[0]; bi = sh.wave_arg[0]; flags = sh.wave_flags[0];
+  for (int w = 1; w < SAMPLE_WAVES; ++w) { argmax_merge(bv, bi, sh.wave_best[w], sh.wave_arg[w]); flags |= sh.wave_flags[w]; }
+  const int st = (flags & 3) | ((flags & 8) ? 0 : 4);
+  if (st || !(p.temperature > 0.f)) {     // nothing sensible to draw from (the host raises on the status), or arg-max
+    if (threadIdx.x == 0) { tokens[row_id] = st || bi == 0x7fffffff ? 0 : bi; status[row_id] = st; }
     return;
   }
-  const float inv_t = 1.f / temperatures[row_id];
-  float mx = -INFINITY;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) mx = fmaxf(mx, row[i]);
-  mx = block_max(mx, red);
+  const float mx = bv, inv_t = 1.f / p.temperature;
 
-  const int chunk = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-  const int begin = threadIdx.x * chunk;
-  const int end = min(vocab, begin + chunk);
-  float local = 0.f;
-  for (int i = begin; i < end; ++i) local += expf((row[i] - mx) * inv_t);
-  sums[threadIdx.x] = local;
-  if (threadIdx.x == 0) chosen = -1;
+  unsigned int key_limit = KEY_END - 1;       // keys up to this one stay
+  if (p.top_k > 0 && p.top_k < vocab) {
+    for (int i = threadIdx.x; i < FILTER_BINS; i += SAMPLE_THREADS) sh.count[i] = 0;
+    __syncthreads();
+    visit_row(row, vocab, segment, [&](int, float v) { atomicAdd(&sh.count[first_bin((mx - v) * inv_t)], 1u); });
+    __syncthreads();
+    key_limit = find_key<false>(row, vocab, segment, mx, inv_t, (unsigned long long)p.top_k, sh);
+  }
+  if (p.top_p < 1.f) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < FILTER_BINS; i += SAMPLE_THREADS) sh.mass[i] = 0;
+    __syncthreads();
+    unsigned long long within = 0;          // the mass of what top-k left
+    visit_row(row, vocab, segment, [&](int, float v) {
+      const float y = (mx - v) * inv_t;
+      const unsigned long long w = weight_of(y);
+      atomicAdd(&sh.mass[first_bin(y)], w);
+      if (__float_as_uint(y) <= key_limit) within += w;
+    });
+    within = block_sum_u64(within, sh);     // its barriers also end the histogram
+    const unsigned long long target = (unsigned long long)((double)within * (double)p.top_p);
+    // what lies past top-k comes after every key that top-k keeps and cannot move the crossing
+    key_limit = min(key_limit, find_key<true>(row, vocab, segment, mx, inv_t, target, sh));
+  }
+
+  // the draw: totals of the kept weights per wave, the wave in which the running sum passes the
+  // target, then that wave walks its part of the row again
+  const float min_e = p.min_p;
+  auto kept_weight = [&](float v) -> unsigned long long {
+    const float y = (mx - v) * inv_t;
+    if (__float_as_uint(y) > key_limit) return 0ull;
+    const float e = expf(-y);
+    return e >= min_e ? (unsigned long long)(e * WEIGHT_SCALE) : 0ull;
+  };
+  unsigned long long mine = 0;
+  visit_row(row, vocab, segment, [&](int, float v) { mine += kept_weight(v); });
+  mine = wave_sum_u64(mine);
+  __syncthreads();
+  if (lane == 0) sh.wave_sum[wave] = mine;
   __syncthreads();
   if (threadIdx.x == 0) {
-    // serial scan over 1024 partial sums: a fixed order, negligible time
-    float total = 0.f;
-    for (int t = 0; t < SAMPLE_THREADS; ++t) total += sums[t];
-    const unsigned long long seed = seeds[row_id];
-    const unsigned long long index = draw_index[row_id];
-    const uint32_t word = philox_first_word((uint32_t)index, (uint32_t)(index >> 32), 0u, 0u,
-                                            (uint32_t)seed, (uint32_t)(seed >> 32));
-    const float u = (float)(word >> 8) * (1.0f / 16777216.0f);
-    const float target = u * total;
-    float running = 0.f;
-    int owner = -1, last_nonzero = -1;
-    for (int t = 0; t < SAMPLE_THREADS; ++t) {
-      const float s = sums[t];
-      if (s > 0.f) last_nonzero = t;
-      if (owner < 0 && running + s > target) { owner = t; break; }
-      running += s;
-    }
-    if (owner < 0) {  // rounding pushed the target past the total: last token with weight
-      owner = last_nonzero;
-      running = -1.f;  // marks "take the last nonzero entry of the range"
-    }
-    red[0] = running;
-    red[1] = target;
-    chosen = owner;
-    if (owner < 0) { tokens[row_id] = 0; status[row_id] = 4; }
+    unsigned long long total = 0;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) total += sh.wave_sum[w];
+    const uint32_t word = philox_first_word((uint32_t)p.draw_index, (uint32_t)(p.draw_index >> 32), 0u, 0u,
+                                            (uint32_t)p.seed, (uint32_t)(p.seed >> 32));
+    const unsigned long long u24 = word >> 8;
+    // floor(total * u24 / 2^24) from the 128-bit product
+    const unsigned long long target = (__umul64hi(total, u24) << 40) | ((total * u24) >> 24);
+    unsigned long long before = 0;
+    int w = 0;
+    while (w < SAMPLE_WAVES - 1 && before + sh.wave_sum[w] <= target) before += sh.wave_sum[w++];
+    sh.pick_wave = w;
+    sh.found_before = before;
+    sh.target = target;
   }
   __syncthreads();
-  if (threadIdx.x == chosen) {
-    float running = red[0];
-    const float target = red[1];
-    int pick = -1, last = -1;
-    for (int i = begin; i < end; ++i) {
-      const float w = expf((row[i] - mx) * inv_t);
-      if (w > 0.f) last = i;
-      if (running >= 0.f) {
-        running += w;
-        if (running > target) { pick = i; break; }
-      }
+  if (wave != sh.pick_wave) return;
+  unsigned long long before = sh.found_before;
+  const unsigned long long target = sh.target;
+  const int begin = wave * segment, end = min(vocab, begin + segment);
+  for (int base = begin; base < end; base += 256) {       // the same order as visit_row's
+    const int at = base + 4 * lane;
+    unsigned long long w4[4];
+    unsigned long long own = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) { w4[c] = at + c < end ? kept_weight(row[at + c]) : 0ull; own += w4[c]; }
+    unsigned long long upto = own;
+#pragma unroll
+    for (int offset = 1; offset < FE_WAVE; offset <<= 1) {
+      const unsigned long long other = __shfl_up(upto, offset, FE_WAVE);
+      if (lane >= offset) upto += other;
     }
-    if (pick < 0) pick = last;
-    tokens[row_id] = pick < 0 ? 0 : pick;
-    status[row_id] = 0;
+    const unsigned long long trip = __shfl(upto, FE_WAVE - 1, FE_WAVE);
+    if (before + trip > target) {
+      const unsigned long long hits = __ballot(before + upto > target);
+      if (lane == __ffsll((long long)hits) - 1) {
+        unsigned long long running = before + upto - own;
+        int pick = at;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          running += w4[c];
+          if (running > target) { pick = at + c; break; }
+        }
+        tokens[row_id] = pick;
+        status[row_id] = 0;
+      }
+      return;
+    }
+    before += trip;
   }
+  if (lane == 0) { tokens[row_id] = bi; status[row_id] = 0; }    // cannot happen: the target lies below the total
 }
 
 // scratch: at least rows * 32 * 3 four-byte words (partial maxima, indices, flags).
@@ -255,13 +436,11 @@ extern "C" int fe_argmax_rows_static(const float* logits, long long row_stride, 
   return fe_argmax_rows(logits, row_stride, rows, vocab, tokens, status, scratch, stream);
 }
 
-extern "C" int fe_sample_rows(const float* logits, long long row_stride, int rows, int vocab,
-                              const float* temperatures, const unsigned long long* seeds,
-                              const unsigned long long* draw_index, int* tokens, int* status,
-                              hipStream_t stream) {
+extern "C" int fe_sample_filtered_rows(const float* logits, long long row_stride, int rows, int vocab,
+                                       const void* params, int* tokens, int* status, hipStream_t stream) {
   if (rows <= 0) return FE_OK;
-  if (vocab <= 0 || row_stride < vocab) return FE_BAD_ARGUMENT;
-  sample_rows_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, row_stride, vocab, temperatures, seeds,
-                                                          draw_index, tokens, status);
+  if (vocab <= 0 || row_stride < vocab || !params || (((uintptr_t)params) & 7)) return FE_BAD_ARGUMENT;
+  sample_filtered_rows_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, row_stride, vocab,
+                                                                   (const SampleRowParams*)params, tokens, status);
   return fe_check_launch();
 }

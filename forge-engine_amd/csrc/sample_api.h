@@ -6,6 +6,9 @@
 // Most rows that fe_argmax_rows_static takes in one call.
 #define FE_ARGMAX_STATIC_MAX_ROWS 1024
 
+// Four-byte words of parameters that fe_sample_filtered_rows reads per row.
+#define FE_SAMPLE_PARAM_WORDS 8
+
 extern "C" {
 
 // tokens[r] = argmax(logits[r]) (lowest index among equals); status bits: 1 NaN, 2 +inf, 4 no finite
@@ -26,10 +29,17 @@ int fe_argmax_rows(const float* logits, long long row_stride, int rows, int voca
 int fe_argmax_rows_static(const float* logits, long long row_stride, int rows, int vocab, int* tokens,
                           int* status, hipStream_t stream);
 
-// tokens[r] drawn from softmax(logits[r] / temperatures[r]) with the uniform
-// philox(counter = draw_index[r], key = seeds[r]); entries equal to -inf have probability 0.
-int fe_sample_rows(const float* logits, long long row_stride, int rows, int vocab, const float* temperatures,
-                   const unsigned long long* seeds, const unsigned long long* draw_index, int* tokens,
-                   int* status, hipStream_t stream);
+// One launch for rows with parameters of their own.  params: rows x FE_SAMPLE_PARAM_WORDS four-byte
+// words, 8-byte aligned: temperature (float; 0 asks for the arg-max), top_k (int; 0 = no limit),
+// top_p (float; >= 1 = no limit), min_p (float; 0 = no limit), seed (64 bits), draw index (64 bits).
+// tokens[r] is drawn from softmax(logits[r] / temperature) restricted, in this order, to the top_k
+// largest entries (with every entry equal to the k-th), to the entries before which at most top_p
+// of that set's probability lies, and to those with at least min_p of the largest probability; the
+// first kept token, in token order, whose running probability exceeds the uniform
+// philox(counter = draw index, key = seed) is taken.  Status bits as for fe_argmax_rows, judged on
+// the logits before any filter.  Probabilities are summed as 64-bit integers (2^-40 of the largest
+// one's), so the result does not depend on the order of the sums.
+int fe_sample_filtered_rows(const float* logits, long long row_stride, int rows, int vocab, const void* params,
+                            int* tokens, int* status, hipStream_t stream);
 
 }  // extern "C"

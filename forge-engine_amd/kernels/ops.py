@@ -11,6 +11,7 @@ from __future__ import annotations
 import threading
 from ctypes import c_float, c_int, c_longlong, c_void_p
 
+import numpy as np
 import torch
 from torch import Tensor
 
@@ -20,6 +21,8 @@ FE_F32 = 0
 FE_BF16 = 1
 _STATUS = {1: "bad argument", 2: "launch failed"}
 _DTYPE_CODE = {torch.float32: FE_F32, torch.bfloat16: FE_BF16}
+_SAMPLE_PARAMS = np.dtype([("temperature", "<f4"), ("top_k", "<i4"), ("top_p", "<f4"), ("min_p", "<f4"),
+                           ("seed", "<u8"), ("draw", "<u8")])
 
 
 class KernelError(RuntimeError):
@@ -821,24 +824,36 @@ def argmax_rows_static(logits: Tensor, tokens: Tensor, status: Tensor) -> None:
           c_int(vocab), _ptr(tokens), _ptr(status), _stream())
 
 
-def sample_rows(logits: Tensor, temperatures: Tensor, seeds: Tensor, draw_index: Tensor,
-                tokens: Tensor, status: Tensor) -> None:
-    """Draw tokens[r] from softmax(logits[r] / temperatures[r]) with the uniform
-    philox(counter=draw_index[r], key=seeds[r]); -inf entries have probability 0."""
-    _gpu(logits, "logits", torch.float32)
-    _gpu(temperatures, "temperatures", torch.float32)
-    _gpu(seeds, "seeds", torch.int64)
-    _gpu(draw_index, "draw_index", torch.int64)
+SAMPLE_PARAM_WORDS = 8      # per row: temperature, top_k, top_p, min_p (four-byte words), seed, draw index (eight bytes each)
+
+
+def pack_sample_params(rows) -> Tensor:
+    """int32 [rows, SAMPLE_PARAM_WORDS] on the host for ``sample_filtered_rows`` from tuples
+    (temperature, top_k or None, top_p, min_p, seed, draw index); temperature 0 asks for the arg-max."""
+    packed = np.zeros(len(rows), dtype=_SAMPLE_PARAMS)
+    for i, (temperature, top_k, top_p, min_p, seed, draw) in enumerate(rows):
+        packed[i] = (temperature, top_k or 0, top_p, min_p, seed & (2**64 - 1), draw & (2**64 - 1))
+    return torch.from_numpy(packed.view(np.int32).reshape(len(rows), SAMPLE_PARAM_WORDS))
+
+
+def sample_filtered_rows(logits: Tensor, params: Tensor, tokens: Tensor, status: Tensor) -> None:
+    """tokens[r]: the arg-max of logits[r], or a draw from softmax(logits[r] / temperature) after
+    top-k, top-p and min-p (in the order of the reference, src/forge_engine/sampling.py:83-140) with
+    the uniform philox(counter=draw index, key=seed); ``params`` as ``pack_sample_params`` lays
+    them out, on the device.  status[r]: bit 0 NaN, bit 1 +inf, bit 2 no finite entry."""
+    _gpu(logits, "logits", torch.float32, contiguous=False)
+    _gpu(params, "params", torch.int32)
     _gpu(tokens, "tokens", torch.int32)
     _gpu(status, "status", torch.int32)
     rows, vocab = logits.shape
-    for name, t in (("temperatures", temperatures), ("seeds", seeds), ("draw_index", draw_index),
-                    ("tokens", tokens), ("status", status)):
-        if t.numel() != rows:
-            raise KernelError(f"{name} needs one entry per row")
-    _call("sample", "fe_sample_rows", _ptr(logits), c_longlong(logits.stride(0)), c_int(rows),
-          c_int(vocab), _ptr(temperatures), _ptr(seeds), _ptr(draw_index), _ptr(tokens), _ptr(status),
-          _stream())
+    if logits.stride(1) != 1 or logits.stride(0) < vocab:
+        raise KernelError("logits rows must be contiguous")
+    if params.shape != (rows, SAMPLE_PARAM_WORDS) or params.data_ptr() % 8:
+        raise KernelError(f"params must be int32 [rows, {SAMPLE_PARAM_WORDS}], 8-byte aligned")
+    if tokens.numel() != rows or status.numel() != rows:
+        raise KernelError("tokens and status need one entry per row")
+    _call("sample", "fe_sample_filtered_rows", _ptr(logits), c_longlong(logits.stride(0)), c_int(rows),
+          c_int(vocab), _ptr(params), _ptr(tokens), _ptr(status), _stream())
 
 
 LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")

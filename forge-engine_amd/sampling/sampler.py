@@ -1,13 +1,15 @@
 """Token selection over float32 logits rows.
 
-Greedy rows take the argmax kernel.  Other rows are filtered in the order of
-the reference (src/forge_engine/sampling.py:83-140): temperature, top-k, top-p,
-min-p; the draw itself is the inverse-CDF kernel with a counter-based
+Greedy batches take the argmax kernel.  Otherwise one kernel takes every row
+with its own parameters and filters in the order of the reference
+(src/forge_engine/sampling.py:83-140): temperature, top-k, top-p, min-p, each
+as a threshold on the logit, then draws by inverse CDF with a counter-based
 generator, so the n-th token of a request depends only on (seed, n) and the
 logits, not on what else was in the batch or on how often the request was
 preempted.  NaN, +inf or a row without a finite entry raise, as in
 sampling.py:62-70; the check runs inside the kernels and comes back with the
-tokens in one transfer.
+tokens in one transfer.  ``filter_logits`` is the same filter on whole tensors
+(what the kernel keeps, for callers that want the filtered logits themselves).
 """
 
 from __future__ import annotations
@@ -85,53 +87,15 @@ class Sampler:
         if not (len(params) == len(seeds) == len(draw_index) == rows):
             raise ValueError("one parameter set, seed and draw index per logits row is needed")
         both = torch.empty((2, rows), dtype=torch.int32, device=self.device)   # one transfer brings both back
-        tokens, status = both[0], both[1]
-        greedy = [r for r in range(rows) if params[r].greedy]
-        drawn = [r for r in range(rows) if not params[r].greedy]
-        if not drawn:
-            ops.argmax_rows(logits, tokens, status)
+        if all(p.greedy for p in params):
+            ops.argmax_rows(logits, both[0], both[1])
         else:
-            self._mixed(logits, params, seeds, draw_index, greedy, drawn, tokens, status)
+            # one launch for all rows, each with its own parameters (greedy rows among them), fed by
+            # one transfer: filters and draw run in the kernel, on the logits where they lie
+            packed = ops.pack_sample_params([
+                (0.0 if p.greedy else p.temperature, p.top_k, p.top_p, p.min_p, seeds[r], draw_index[r])
+                for r, p in enumerate(params)])
+            ops.sample_filtered_rows(logits.float(), packed.to(self.device), both[0], both[1])
         host = both.cpu()
         _raise_on_status(host[1].tolist())
         return host[0].tolist()
-
-    def _mixed(self, logits, params, seeds, draw_index, greedy, drawn, tokens, status) -> None:
-        if greedy:
-            index = torch.tensor(greedy, device=self.device)
-            t = torch.empty(len(greedy), dtype=torch.int32, device=self.device)
-            s = torch.empty(len(greedy), dtype=torch.int32, device=self.device)
-            ops.argmax_rows(logits.index_select(0, index).contiguous(), t, s)
-            tokens[index] = t
-            status[index] = s
-        groups: dict[tuple, list[int]] = {}
-        for r in drawn:
-            p = params[r]
-            groups.setdefault((p.temperature, p.top_k, p.top_p, p.min_p), []).append(r)
-        for key, members in groups.items():
-            p = params[members[0]]
-            index = torch.tensor(members, device=self.device)
-            rows = logits.index_select(0, index).contiguous()
-            filtered = p.top_k is not None or p.top_p < 1.0 or p.min_p > 0.0
-            if filtered:
-                check_t = torch.empty(len(members), dtype=torch.int32, device=self.device)
-                check_s = torch.empty(len(members), dtype=torch.int32, device=self.device)
-                ops.argmax_rows(rows, check_t, check_s)     # the guards see the logits before any filter
-                rows = filter_logits(rows, p).contiguous()  # temperature already applied
-                temperature = 1.0
-            else:
-                temperature = p.temperature
-            t = torch.empty(len(members), dtype=torch.int32, device=self.device)
-            s = torch.empty(len(members), dtype=torch.int32, device=self.device)
-            ops.sample_rows(
-                rows, torch.full((len(members),), temperature, dtype=torch.float32, device=self.device),
-                torch.tensor([_as_int64(seeds[r]) for r in members], dtype=torch.int64, device=self.device),
-                torch.tensor([draw_index[r] for r in members], dtype=torch.int64, device=self.device), t, s)
-            tokens[index] = t
-            status[index] = check_s if filtered else s
-
-
-def _as_int64(seed: int) -> int:
-    """Seeds are 64-bit keys; values above 2^63 wrap into the signed range."""
-    seed &= (1 << 64) - 1
-    return seed - (1 << 64) if seed >= (1 << 63) else seed

@@ -185,12 +185,50 @@ def uniform_from(counter: int, key: int) -> float:
     return (philox_first_word(counter, key) >> 8) / 16777216.0
 
 
-def sample_rows(logits, temperatures, seeds, draw_index, tokens, status):
-    """Inverse CDF over softmax(logits / T) in float64 with the same uniform as
-    the kernel; the kernel's float32 running sum may pick a neighbour when the
-    target falls within rounding of a boundary (tests allow for that)."""
-    for r in range(logits.shape[0]):
-        row = logits[r].double()
+def kept_after_filters(row, temperature, top_k, top_p, min_p):
+    """(weights, kept) of one row in float64 after temperature, top-k, top-p, min-p in the order and
+    with the rules of the reference (src/forge_engine/sampling.py:83-140): e_i = exp((x_i - max) / T);
+    top-k keeps the k largest; top-p keeps a token if the probability of all larger ones, within what
+    top-k left, is <= top_p; min-p keeps e_i >= min_p (the largest e is 1)."""
+    # the logit as the kernel forms it, in float32: (max - x) * (1 / T); everything after it in float64
+    y = (row.float().max() - row.float()) * torch.tensor(1.0, dtype=torch.float32).div(temperature)
+    x = -y.double()
+    e = torch.exp(x)
+    kept = torch.ones_like(e, dtype=torch.bool)
+    if top_k and top_k < len(row):
+        kth = torch.topk(x, top_k).values[-1]
+        kept &= x >= kth
+    if top_p < 1.0:
+        masked = torch.where(kept, e, torch.zeros_like(e))
+        order = torch.argsort(x, descending=True, stable=True)
+        before = masked[order].cumsum(0) - masked[order]
+        keep_sorted = before <= top_p * masked.sum()
+        by_p = torch.zeros_like(kept)
+        by_p[order] = keep_sorted
+        kept &= by_p
+    if min_p > 0.0:
+        kept &= e >= min_p
+    return e, kept
+
+
+def unpack_sample_params(params):
+    """Rows of (temperature, top_k, top_p, min_p, seed, draw index) from the packed int32 words."""
+    words = params.cpu().contiguous()
+    floats = words.view(torch.float32)
+    rows = []
+    for r in range(words.shape[0]):
+        low = [int(v) & 0xFFFFFFFF for v in words[r, 4:8]]
+        rows.append((float(floats[r, 0]), int(words[r, 1]), float(floats[r, 2]), float(floats[r, 3]),
+                     low[0] | (low[1] << 32), low[2] | (low[3] << 32)))
+    return rows
+
+
+def sample_filtered_rows(logits, params, tokens, status):
+    """Arg-max (temperature 0), or the filters above and an inverse CDF in float64 over what they
+    kept, in token order, with the same uniform as the kernel; the kernel's sums of 2^-40 steps may
+    pick a neighbour when the target falls within rounding of a boundary (tests allow for that)."""
+    for r, (temperature, top_k, top_p, min_p, seed, draw) in enumerate(unpack_sample_params(params)):
+        row = logits[r]
         flags = 0
         if torch.isnan(row).any():
             flags |= 1
@@ -202,10 +240,12 @@ def sample_rows(logits, temperatures, seeds, draw_index, tokens, status):
         if flags:
             tokens[r] = 0
             continue
-        weights = torch.exp((row - row.max()) / float(temperatures[r]))
-        cdf = weights.cumsum(0)
-        u = uniform_from(int(draw_index[r]) & (2**64 - 1), int(seeds[r]) & (2**64 - 1))
-        target = u * float(cdf[-1])
+        if not temperature > 0:
+            tokens[r] = int(torch.argmax(row))
+            continue
+        e, kept = kept_after_filters(row, temperature, top_k, top_p, min_p)
+        cdf = torch.where(kept, e, torch.zeros_like(e)).cumsum(0)
+        target = uniform_from(draw, seed) * float(cdf[-1])
         pick = int(torch.searchsorted(cdf, torch.tensor(target, dtype=torch.float64), right=True))
         tokens[r] = min(pick, logits.shape[1] - 1)
 
@@ -219,7 +259,7 @@ def linear_in_parts(x, weight):
 
 
 NAMES = ("decode_prepare_supported", "linear_in_parts", "embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_update", "linear_swiglu", "gemm_skinny",
-         "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_rows")
+         "qk_norm_rope_write", "paged_attention", "argmax_rows", "sample_filtered_rows")
 
 
 def install(monkeypatch):

@@ -408,23 +408,25 @@ def test_argmax_rows(ops):
     assert status.cpu().tolist() == [0, 0, 1, 4, 2]
 
 
-def test_sample_rows_follows_the_distribution(ops):
+def sample_params(ops, rows):
+    return ops.pack_sample_params(rows).to(DEV)
+
+
+def test_sampling_follows_the_distribution(ops):
     vocab, draws = 37, 4000
     g = torch.Generator().manual_seed(11)
     row = rand(g, vocab, scale=2.0)
     row[5] = float("-inf")
     logits = row.repeat(draws, 1).to(DEV)
-    temps = torch.full((draws,), 0.8, device=DEV)
-    seeds = torch.full((draws,), 1234, dtype=torch.int64, device=DEV)
-    index = torch.arange(draws, dtype=torch.int64, device=DEV)
+    params = sample_params(ops, [(0.8, None, 1.0, 0.0, 1234, i) for i in range(draws)])
     tokens = torch.zeros(draws, dtype=torch.int32, device=DEV)
     status = torch.zeros(draws, dtype=torch.int32, device=DEV)
-    ops.sample_rows(logits, temps, seeds, index, tokens, status)
+    ops.sample_filtered_rows(logits, params, tokens, status)
     assert int(status.sum()) == 0
     got = tokens.cpu()
     # same uniforms, float64 inverse CDF: equal except where the target sits within rounding of a boundary
     want = torch.zeros(draws, dtype=torch.int32)
-    refs.sample_rows(logits.cpu(), temps.cpu(), seeds.cpu(), index.cpu(), want, torch.zeros(draws, dtype=torch.int32))
+    refs.sample_filtered_rows(logits.cpu(), params.cpu(), want, torch.zeros(draws, dtype=torch.int32))
     assert (got != want).sum() <= 2
     assert (got == 5).sum() == 0
     probs = torch.softmax(row / 0.8, 0)
@@ -435,20 +437,104 @@ def test_sample_rows_follows_the_distribution(ops):
     assert chi2 < 2.0 * int(mask.sum()) + 20
     # a second run with the same seeds and counters repeats the draws; another seed does not
     again = torch.zeros_like(tokens)
-    ops.sample_rows(logits, temps, seeds, index, again, status)
+    ops.sample_filtered_rows(logits, params, again, status)
     assert torch.equal(again.cpu(), got)
-    ops.sample_rows(logits, temps, seeds + 1, index, again, status)
+    ops.sample_filtered_rows(logits, sample_params(ops, [(0.8, None, 1.0, 0.0, 1235, i) for i in range(draws)]), again, status)
     assert not torch.equal(again.cpu(), got)
 
 
-def test_sample_rows_low_temperature_is_argmax(ops):
+def test_sampling_at_low_temperature_is_argmax(ops):
     g = torch.Generator().manual_seed(12)
     logits = rand(g, 8, 1003).to(DEV)
     tokens = torch.zeros(8, dtype=torch.int32, device=DEV)
     status = torch.zeros(8, dtype=torch.int32, device=DEV)
-    ops.sample_rows(logits, torch.full((8,), 1e-4, device=DEV), torch.arange(8, dtype=torch.int64, device=DEV),
-                    torch.zeros(8, dtype=torch.int64, device=DEV), tokens, status)
+    ops.sample_filtered_rows(logits, sample_params(ops, [(1e-4, None, 1.0, 0.0, r, 0) for r in range(8)]), tokens, status)
     assert torch.equal(tokens.cpu().long(), logits.cpu().argmax(-1))
+
+
+FILTERS = [(0.7, 5, 1.0, 0.0), (1.3, None, 0.6, 0.0), (0.9, None, 1.0, 0.1), (0.5, 20, 0.8, 0.05), (1.0, 1, 1.0, 0.0),
+           (1.1, 300, 0.95, 0.0), (0.8, None, 0.999, 0.001), (2.0, 50, 0.3, 0.0)]
+
+
+@pytest.mark.parametrize("vocab", [37, 1003, 4097, 151936])
+def test_sampling_filters_keep_what_the_reference_keeps(ops, vocab):
+    """Rows of their own parameters in one launch (greedy ones among them): every draw equals the
+    float64 inverse CDF over what the reference's filters keep, with the same uniform, but for a
+    few whose target lies within rounding of a boundary; a kept set that differed by one token
+    would shift every draw behind it."""
+    g = torch.Generator().manual_seed(vocab)
+    shapes = FILTERS + [(0.0, None, 1.0, 0.0)]
+    per = 24 if vocab > 10000 else 120
+    rows, base = [], []
+    for f, (t, k, p, m) in enumerate(shapes):
+        row = rand(g, vocab, scale=3.0)
+        if vocab > 50:
+            row[7] = float("-inf")
+        for d in range(per):
+            rows.append((t, k, p, m, 1000 + f, d))
+            base.append(row)
+    logits = torch.stack(base)
+    wide = torch.full((len(rows), vocab + 3), 9.0)          # rows that are a view with a longer stride
+    wide[:, :vocab] = logits
+    tokens = torch.zeros(len(rows), dtype=torch.int32, device=DEV)
+    status = torch.ones(len(rows), dtype=torch.int32, device=DEV)
+    params = sample_params(ops, rows)
+    ops.sample_filtered_rows(wide.to(DEV)[:, :vocab], params, tokens, status)
+    assert int(status.sum()) == 0
+    want = torch.zeros(len(rows), dtype=torch.int32)
+    refs.sample_filtered_rows(logits, params.cpu(), want, torch.zeros(len(rows), dtype=torch.int32))
+    got = tokens.cpu()
+    assert (got != want).sum() <= max(2, len(rows) // 200), (got != want).nonzero().flatten().tolist()
+    for f, (t, k, p, m) in enumerate(shapes):       # nothing outside what the filters keep is ever drawn
+        picks = got[f * per:(f + 1) * per].long()
+        if t == 0.0:
+            assert (picks == int(base[f * per].argmax())).all()
+            continue
+        _, kept = refs.kept_after_filters(base[f * per], t, k or 0, p, m)
+        assert kept[picks].all()
+    again = torch.zeros_like(tokens)
+    ops.sample_filtered_rows(wide.to(DEV)[:, :vocab], params, again, status)
+    assert torch.equal(again.cpu(), got)
+
+
+def test_sampling_thresholds_at_equal_and_extreme_logits(ops):
+    """Equal logits (every key in one bin down to the last level), a far maximum (all mass in one
+    token), and -inf everywhere but two entries: the searches end and the draws stay inside."""
+    vocab = 5000
+    flat = torch.zeros(vocab)
+    peak = torch.full((vocab,), -50.0)
+    peak[4321] = 30.0
+    two = torch.full((vocab,), float("-inf"))
+    two[17], two[4000] = 1.0, 1.0
+    cases = [(flat, (1.0, 10, 0.5, 0.0)), (flat, (1.0, None, 0.5, 0.2)), (peak, (1.0, 40, 0.9, 0.0)), (peak, (5.0, None, 0.99, 0.0)),
+             (two, (1.0, 5, 0.9, 0.1)), (two, (0.7, None, 0.4, 0.0))]
+    per = 64
+    rows = [(t, k, p, m, 7 + c, d) for c, (_, (t, k, p, m)) in enumerate(cases) for d in range(per)]
+    logits = torch.stack([row for row, _ in cases for _ in range(per)]).to(DEV)
+    tokens = torch.zeros(len(rows), dtype=torch.int32, device=DEV)
+    status = torch.ones(len(rows), dtype=torch.int32, device=DEV)
+    ops.sample_filtered_rows(logits, sample_params(ops, rows), tokens, status)
+    assert int(status.sum()) == 0
+    got = tokens.cpu().view(len(cases), per)
+    assert len(set(got[0].tolist())) > 20 and len(set(got[1].tolist())) > 20     # equal logits: ties all stay
+    assert (got[2] == 4321).all() and (got[3] == 4321).all()
+    for c in (4, 5):
+        assert set(got[c].tolist()) <= {17, 4000}
+    assert set(got[4].tolist()) == {17, 4000}          # top_p 0.9 keeps both halves
+    assert set(got[5].tolist()) == {17, 4000}          # equal keys stay together: ties are kept
+
+
+def test_sampling_reports_bad_rows(ops):
+    logits = torch.zeros(4, 100)
+    logits[1, 3] = float("nan")
+    logits[2, 5] = float("inf")
+    logits[3] = float("-inf")
+    tokens = torch.zeros(4, dtype=torch.int32, device=DEV)
+    status = torch.zeros(4, dtype=torch.int32, device=DEV)
+    ops.sample_filtered_rows(logits.to(DEV), sample_params(ops, [(0.9, 5, 0.9, 0.0, 1, 0)] * 4), tokens, status)
+    assert status.cpu().tolist() == [0, 1, 2, 4]
+    with pytest.raises(ops.KernelError):
+        ops.sample_filtered_rows(logits.to(DEV), sample_params(ops, [(0.9, 5, 0.9, 0.0, 1, 0)] * 3), tokens, status)
 
 
 def test_kernels_refuse_what_they_cannot_do(ops):

@@ -57,6 +57,29 @@ def test_filters_equal_the_plain_implementation(seed):
         torch.testing.assert_close(got, want)
 
 
+@pytest.mark.parametrize("seed", range(5))
+def test_the_kernel_reference_keeps_what_the_plain_filters_keep(seed):
+    """The thresholds that the sampling kernel is tested against (kernel_refs.kept_after_filters)
+    against the filters written from the reference's text, on rows without equal logits."""
+    g = torch.Generator().manual_seed(100 + seed)
+    logits = torch.randn(6, 300, generator=g) * 3
+    for t, k, p, m in ((0.7, 5, 1.0, 0.0), (1.3, None, 0.6, 0.0), (0.9, None, 1.0, 0.1), (0.5, 20, 0.8, 0.05), (1.0, 1, 1.0, 0.0),
+                       (1.1, 200, 0.95, 0.0), (2.0, 50, 0.3, 0.0)):
+        want = torch.isfinite(plain.filter_logits(logits, t, k, p, m))
+        for r in range(logits.shape[0]):
+            _, kept = kernel_refs.kept_after_filters(logits[r], t, k or 0, p, m)
+            assert torch.equal(kept, want[r]), (t, k, p, m, r)
+
+
+def test_sample_parameters_are_packed_as_the_kernel_reads_them():
+    from forge_engine_amd.kernels import ops
+    packed = ops.pack_sample_params([(0.5, None, 1.0, 0.0, 2**64 - 1, 5), (0.0, 40, 0.9, 0.05, 7, 2**40 + 3)])
+    assert packed.shape == (2, ops.SAMPLE_PARAM_WORDS) and packed.dtype == torch.int32
+    rows = kernel_refs.unpack_sample_params(packed)
+    assert rows[0] == (0.5, 0, 1.0, 0.0, 2**64 - 1, 5)
+    assert rows[1][0] == 0.0 and rows[1][1] == 40 and abs(rows[1][2] - 0.9) < 1e-6 and rows[1][4:] == (7, 2**40 + 3)
+
+
 def test_sampler_routes_rows_and_raises_on_bad_logits(monkeypatch):
     kernel_refs.install(monkeypatch)
     sampler = Sampler(torch.device("cpu"))
