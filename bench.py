@@ -189,6 +189,18 @@ def micro_benchmarks() -> int:
     record["causal_prefill_1x8x128x128"] = dict(measure(paged(128, 128, 8, 8)), reference_l4_ms=0.0891)
     # one decoded token over 127 cached keys and its own, 32 query heads, 8 kv heads of 128, pages of 16
     record["paged_gqa_decode_past127_q32_kv8"] = dict(measure(paged(128, 1, 32, 8)), reference_l4_ms=0.1004)
+
+    # beside the reference's three: a sampling call for 8 and 64 rows of a 151,936-token vocabulary with
+    # temperature, top-k, top-p and min-p (parameters packed and sent, the kernel's launches, tokens read back)
+    from forge_engine_amd.sampling import SamplingParams
+    from forge_engine_amd.sampling.sampler import Sampler
+
+    sampler = Sampler(device)
+    for rows in (8, 64):
+        logits = rand(rows, 151936, dtype=torch.float32) * 3
+        params = [SamplingParams(temperature=0.8, top_k=50, top_p=0.9, min_p=0.05, seed=1)] * rows
+        seeds, draws = list(range(rows)), [3] * rows
+        record[f"sample_top_k_top_p_min_p_{rows}x151936"] = measure(lambda: sampler.sample(logits, params, seeds, draws))
     print(json.dumps(record))
     return 0
 

@@ -836,11 +836,20 @@ def pack_sample_params(rows) -> Tensor:
     return torch.from_numpy(packed.view(np.int32).reshape(len(rows), SAMPLE_PARAM_WORDS))
 
 
-def sample_filtered_rows(logits: Tensor, params: Tensor, tokens: Tensor, status: Tensor) -> None:
+SAMPLE_MAX_SPLIT = 32                # most slices of a row, a block each
+SAMPLE_SCRATCH_BYTES_PER_ROW = 76800
+SAMPLE_TARGET_BLOCKS = 1024          # slices of all rows together: four blocks of 256 threads a CU
+
+
+def sample_filtered_rows(logits: Tensor, params: Tensor, tokens: Tensor, status: Tensor,
+                         any_top_k: bool = True, any_top_p: bool = True) -> None:
     """tokens[r]: the arg-max of logits[r], or a draw from softmax(logits[r] / temperature) after
     top-k, top-p and min-p (in the order of the reference, src/forge_engine/sampling.py:83-140) with
     the uniform philox(counter=draw index, key=seed); ``params`` as ``pack_sample_params`` lays
-    them out, on the device.  status[r]: bit 0 NaN, bit 1 +inf, bit 2 no finite entry."""
+    them out, on the device.  status[r]: bit 0 NaN, bit 1 +inf, bit 2 no finite entry.
+    ``any_top_k`` / ``any_top_p``: whether any row limits by top-k / top-p (each search is up to
+    four launches that rows without it sit out; saying no where a row does ask leaves that row
+    unfinished, which raises)."""
     _gpu(logits, "logits", torch.float32, contiguous=False)
     _gpu(params, "params", torch.int32)
     _gpu(tokens, "tokens", torch.int32)
@@ -852,8 +861,15 @@ def sample_filtered_rows(logits: Tensor, params: Tensor, tokens: Tensor, status:
         raise KernelError(f"params must be int32 [rows, {SAMPLE_PARAM_WORDS}], 8-byte aligned")
     if tokens.numel() != rows or status.numel() != rows:
         raise KernelError("tokens and status need one entry per row")
+    if rows == 0:
+        return
+    # slices of at least 4,096 entries, about SAMPLE_TARGET_BLOCKS blocks in all
+    split = max(1, min(SAMPLE_MAX_SPLIT, -(-SAMPLE_TARGET_BLOCKS // rows), vocab // 4096))
+    scratch = torch.empty(rows * SAMPLE_SCRATCH_BYTES_PER_ROW, dtype=torch.uint8, device=logits.device)
+    launches = 3 + (4 if any_top_k else 0) + (4 if any_top_p else 0)
     _call("sample", "fe_sample_filtered_rows", _ptr(logits), c_longlong(logits.stride(0)), c_int(rows),
-          c_int(vocab), _ptr(params), _ptr(tokens), _ptr(status), _stream())
+          c_int(vocab), _ptr(params), _ptr(tokens), _ptr(status), _ptr(scratch), c_int(split), c_int(launches),
+          _stream())
 
 
 LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")

@@ -49,6 +49,8 @@ def filter_logits(logits: Tensor, params: SamplingParams) -> Tensor:
 
 def _raise_on_status(status: list[int]) -> None:
     for flags in status:
+        if flags & 8:
+            raise RuntimeError("the sampling kernel was given too few launches for a row's filters")
         if flags & 1:
             raise ValueError("logits must not contain NaN")
         if flags & 2:
@@ -95,7 +97,9 @@ class Sampler:
             packed = ops.pack_sample_params([
                 (0.0 if p.greedy else p.temperature, p.top_k, p.top_p, p.min_p, seeds[r], draw_index[r])
                 for r, p in enumerate(params)])
-            ops.sample_filtered_rows(logits.float(), packed.to(self.device), both[0], both[1])
+            ops.sample_filtered_rows(logits.float(), packed.to(self.device), both[0], both[1],
+                                     any_top_k=any(p.top_k is not None for p in params if not p.greedy),
+                                     any_top_p=any(p.top_p < 1.0 for p in params if not p.greedy))
         host = both.cpu()
         _raise_on_status(host[1].tolist())
         return host[0].tolist()

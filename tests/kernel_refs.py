@@ -223,7 +223,7 @@ def unpack_sample_params(params):
     return rows
 
 
-def sample_filtered_rows(logits, params, tokens, status):
+def sample_filtered_rows(logits, params, tokens, status, any_top_k=True, any_top_p=True):
     """Arg-max (temperature 0), or the filters above and an inverse CDF in float64 over what they
     kept, in token order, with the same uniform as the kernel; the kernel's sums of 2^-40 steps may
     pick a neighbour when the target falls within rounding of a boundary (tests allow for that)."""

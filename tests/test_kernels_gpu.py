@@ -456,12 +456,14 @@ FILTERS = [(0.7, 5, 1.0, 0.0), (1.3, None, 0.6, 0.0), (0.9, None, 1.0, 0.1), (0.
            (1.1, 300, 0.95, 0.0), (0.8, None, 0.999, 0.001), (2.0, 50, 0.3, 0.0)]
 
 
-@pytest.mark.parametrize("vocab", [37, 1003, 4097, 151936])
-def test_sampling_filters_keep_what_the_reference_keeps(ops, vocab):
-    """Rows of their own parameters in one launch (greedy ones among them): every draw equals the
-    float64 inverse CDF over what the reference's filters keep, with the same uniform, but for a
-    few whose target lies within rounding of a boundary; a kept set that differed by one token
-    would shift every draw behind it."""
+@pytest.mark.parametrize("vocab,blocks", [(37, 1024), (1003, 1024), (4097, 1024), (151936, 1024), (151936, 100000),
+                                          (20000, 100000), (9000, 100000)])
+def test_sampling_filters_keep_what_the_reference_keeps(ops, monkeypatch, vocab, blocks):
+    """Rows of their own parameters in one call (greedy ones among them), a row in 1, 2, 4, 5 or 32
+    slices: every draw equals the float64 inverse CDF over what the reference's filters keep, with
+    the same uniform, but for a few whose target lies within rounding of a boundary; a kept set that
+    differed by one token would shift every draw behind it."""
+    monkeypatch.setattr(ops, "SAMPLE_TARGET_BLOCKS", blocks)
     g = torch.Generator().manual_seed(vocab)
     shapes = FILTERS + [(0.0, None, 1.0, 0.0)]
     per = 24 if vocab > 10000 else 120
@@ -533,6 +535,10 @@ def test_sampling_reports_bad_rows(ops):
     status = torch.zeros(4, dtype=torch.int32, device=DEV)
     ops.sample_filtered_rows(logits.to(DEV), sample_params(ops, [(0.9, 5, 0.9, 0.0, 1, 0)] * 4), tokens, status)
     assert status.cpu().tolist() == [0, 1, 2, 4]
+    # told that no row limits by top-k or top-p, the call leaves out those launches: the row that does is not through
+    ops.sample_filtered_rows(logits.to(DEV), sample_params(ops, [(0.9, 5, 0.9, 0.0, 1, 0)] * 4), tokens, status,
+                             any_top_k=False, any_top_p=False)
+    assert status.cpu().tolist() == [8, 1, 2, 4]
     with pytest.raises(ops.KernelError):
         ops.sample_filtered_rows(logits.to(DEV), sample_params(ops, [(0.9, 5, 0.9, 0.0, 1, 0)] * 3), tokens, status)
 
