@@ -97,6 +97,8 @@ def parse_args():
     parser.add_argument("--prompt-range", default="128,4096", help="mixed workload: prompt lengths, uniform")
     parser.add_argument("--new-tokens", type=int, default=256, help="mixed workload: tokens generated per request")
     parser.add_argument("--token-budget", type=int, default=2048, help="scheduler: tokens a step")
+    parser.add_argument("--sampled", action="store_true",
+                        help="through the scheduler: draw with temperature 0.8, top-k 50, top-p 0.9 instead of the arg-max")
     parser.add_argument("--no-overlap", dest="overlap", action="store_false",
                         help="read every step's tokens back before the next step is launched")
     parser.add_argument("--seed", type=int, default=0)
@@ -364,10 +366,12 @@ def main() -> int:
         """The same decode steps through the scheduler: requests are admitted with their prompts,
         stepped until every one decodes, then K calls of step() are timed."""
         scheduler = SchedulerConfig(max_requests=batch, max_batch_size=batch, token_budget=max(args.token_budget, batch),
-                                    block_size=args.block_size, block_capacity=capacity)
+                                    block_size=args.block_size, block_capacity=capacity, overlap_decode=args.overlap)
         engine = ConcurrentGenerationEngine(runner, sampler, greedy, scheduler, eos_token_ids=())
-        budget = SamplingParams(max_new_tokens=args.steps + args.warmup + 4 + joining)
-        ids = [engine.submit(random_tokens(args.prompt_len), sampling_params=budget) for _ in range(batch)]
+        limit = args.steps + args.warmup + 4 + joining
+        drawn = dict(temperature=0.8, top_k=50, top_p=0.9) if args.sampled else {}
+        ids = [engine.submit(random_tokens(args.prompt_len), sampling_params=SamplingParams(max_new_tokens=limit, seed=i, **drawn))
+               for i in range(batch)]
         while any(n != 1 for n in engine.snapshot().last_batch_tokens) or len(engine.snapshot().last_batch) != batch:
             engine.step()
         times, wall = timed(engine.step, args.warmup, args.steps)

@@ -11,14 +11,15 @@ and never splits a prompt; here every selected request contributes to one flat
 batch (portions of prompts beside single decoded tokens) and the token budget
 cuts prompts into portions.
 
-Overlapped decoding (``overlap_decode``).  While the same requests decode greedily step after
-step, a step is launched with the tokens that the step before sampled still on the device, and
+Overlapped decoding (``overlap_decode``).  While the same requests decode step after step
+(greedily or with draws: a draw is keyed by the request's seed and the count of its tokens, which
+the host knows without reading any), a step is launched with the tokens that the step before sampled still on the device, and
 the host reads those tokens while the new step runs: the GPU does not wait for the scheduler
 between two steps.  What the host sees is one step late: events come a step later, and a
 request that samples its end-of-sequence token still rides in the step that was already
 launched (its result there is dropped).  A request that reaches its token limit is known in
 advance and never rides along.  Any other kind of step (a prompt portion, another set of
-requests, a sampled rather than greedy row) first reads what is in flight.  The tokens that
+requests) first reads what is in flight.  The tokens that
 requests generate are the same either way.
 
 When pages run out.  ``admission="reserve"`` (default, the reference's policy):
@@ -310,12 +311,12 @@ class ConcurrentGenerationEngine:
         return events
 
     def _may_overlap(self, selected: list[tuple[_Request, int]]) -> bool:
-        """A step of single greedy tokens, every one the last of its request's history, none of
-        which ends its request by the token limit, that the runner can feed from the device."""
-        if not self._config.overlap_decode or not hasattr(self._sampler, "sample_greedy_on_device"):
+        """A step of single tokens, every one the last of its request's history, none of which
+        ends its request by the token limit, that the runner can feed from the device."""
+        if not self._config.overlap_decode or not hasattr(self._sampler, "sample_on_device"):
             return False
         for request, count in selected:
-            if count != 1 or request.remaining() != 1 or not request.params.greedy:
+            if count != 1 or request.remaining() != 1:
                 return False
             if request.sampled_tokens + (1 if request.in_flight else 0) + 1 > request.params.max_new_tokens:
                 return False
@@ -338,7 +339,10 @@ class ConcurrentGenerationEngine:
             feed = None
         try:
             logits = self._runner.step(entries, device_tokens=feed) if feed is not None else self._runner.step(entries)
-            launched = self._sampler.sample_greedy_on_device(logits)
+            # a request with a token in flight has drawn one more than it has consumed
+            launched = self._sampler.sample_on_device(
+                logits, [r.params for r in requests], [r.seed for r in requests],
+                [r.sampled_tokens + (1 if r.in_flight else 0) for r in requests])
         except Exception:
             return None                             # nothing was changed: pages are reserved all or none
         self._last_batch = tuple(r.request_id for r in requests)

@@ -62,6 +62,28 @@ def _raise_on_status(status: list[int]) -> None:
 class Sampler:
     def __init__(self, device: torch.device) -> None:
         self.device = device
+        # the rows' parameters go to the device from pinned memory without the host waiting for the
+        # stream (a copy from pageable memory waits for everything queued before it, the step
+        # included); two buffers in turn, each free again once its last copy has run
+        self._staging: list[tuple[Tensor, torch.cuda.Event] | None] = [None, None]
+        self._turn = 0
+
+    def _to_device(self, packed: Tensor) -> Tensor:
+        if self.device.type != "cuda":
+            return packed.to(self.device)
+        self._turn ^= 1
+        slot = self._staging[self._turn]
+        if slot is None or slot[0].shape[0] < packed.shape[0]:
+            rows = max(64, 2 * packed.shape[0])
+            slot = (torch.empty((rows, packed.shape[1]), dtype=packed.dtype, pin_memory=True), torch.cuda.Event())
+            self._staging[self._turn] = slot
+        else:
+            slot[1].synchronize()
+        host = slot[0][:packed.shape[0]]
+        host.copy_(packed)
+        on_device = host.to(self.device, non_blocking=True)
+        slot[1].record(torch.cuda.current_stream(self.device))
+        return on_device
 
     def sample_greedy_on_device(self, logits: Tensor) -> Tensor:
         """Arg-max of every row, left on the device: int32 [2, rows], the tokens and the rows'
@@ -79,27 +101,33 @@ class Sampler:
         _raise_on_status(host[1].tolist())
         return host[0].tolist()
 
-    def sample(self, logits: Tensor, params: list[SamplingParams], seeds: list[int],
-               draw_index: list[int]) -> list[int]:
-        """One token per row.  ``seeds[r]`` and ``draw_index[r]`` (how many tokens
-        the request has drawn so far) key the generator of row r."""
+    def sample_on_device(self, logits: Tensor, params: list[SamplingParams], seeds: list[int],
+                         draw_index: list[int]) -> Tensor:
+        """One token per row, left on the device: int32 [2, rows], the tokens and the rows' status
+        words, for ``read``.  ``seeds[r]`` and ``draw_index[r]`` (how many tokens the request has
+        drawn so far) key the generator of row r."""
         rows = logits.shape[0]
-        if rows == 0:
-            return []
         if not (len(params) == len(seeds) == len(draw_index) == rows):
             raise ValueError("one parameter set, seed and draw index per logits row is needed")
         both = torch.empty((2, rows), dtype=torch.int32, device=self.device)   # one transfer brings both back
+        if rows == 0:
+            return both
         if all(p.greedy for p in params):
             ops.argmax_rows(logits, both[0], both[1])
         else:
-            # one launch for all rows, each with its own parameters (greedy rows among them), fed by
-            # one transfer: filters and draw run in the kernel, on the logits where they lie
+            # all rows in one call, each with its own parameters (greedy rows among them), fed by one
+            # transfer: filters and draw run in the kernel, on the logits where they lie
             packed = ops.pack_sample_params([
                 (0.0 if p.greedy else p.temperature, p.top_k, p.top_p, p.min_p, seeds[r], draw_index[r])
                 for r, p in enumerate(params)])
-            ops.sample_filtered_rows(logits.float(), packed.to(self.device), both[0], both[1],
+            ops.sample_filtered_rows(logits.float(), self._to_device(packed), both[0], both[1],
                                      any_top_k=any(p.top_k is not None for p in params if not p.greedy),
                                      any_top_p=any(p.top_p < 1.0 for p in params if not p.greedy))
-        host = both.cpu()
-        _raise_on_status(host[1].tolist())
-        return host[0].tolist()
+        return both
+
+    def sample(self, logits: Tensor, params: list[SamplingParams], seeds: list[int],
+               draw_index: list[int]) -> list[int]:
+        """One token per row, on the host (``sample_on_device``, read at once)."""
+        if logits.shape[0] == 0:
+            return []
+        return self.read(self.sample_on_device(logits, params, seeds, draw_index))

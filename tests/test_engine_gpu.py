@@ -103,12 +103,18 @@ def test_scheduler_under_page_pressure_on_the_gpu(name, folders):
         assert got == plain.greedy_generate(weights, config, prompt, n), request_id
 
 
+@pytest.mark.parametrize("sampled", [False, True])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_overlapped_decode_steps_generate_the_same_tokens(dtype, folders):
-    """Steady greedy decode steps take their tokens on the device and the host reads a step late:
+def test_overlapped_decode_steps_generate_the_same_tokens(dtype, sampled, folders):
+    """Steady decode steps (greedy, or drawn with temperature, top-k and top-p from seeded
+    generators) take their tokens on the device and the host reads a step late:
     the same tokens, finish reasons and freed pages as with every step read back at once; with
     requests that end on an end-of-sequence token (seen a step late), on their token limit (known
     in advance), a request cancelled while its token is in flight, and a late joiner."""
+    def sampling(limit, seed):
+        if sampled:
+            return SamplingParams(temperature=0.9, top_k=20, top_p=0.95, seed=seed, max_new_tokens=limit)
+        return SamplingParams(max_new_tokens=limit)
     name = "B"          # a head of its own: greedy tokens vary instead of falling into a loop at once
     config = TINY[name]
     prompts = list(ru.make_requests(config, 87, (12, 30, 7, 19, 25)).values())
@@ -120,17 +126,17 @@ def test_overlapped_decode_steps_generate_the_same_tokens(dtype, folders):
         engine = engine_from_folder(folders[name], scheduler_config=scheduler, dtype=dtype)
         if not overlap:
             # choose an end-of-sequence token that the second request really samples, a few tokens in
-            probe = engine.generate([prompts[1]], SamplingParams(max_new_tokens=24))[0]
+            probe = engine.generate([prompts[1]], sampling(24, 101))[0]
             at = next(j for j in range(3, len(probe)) if probe[j] not in probe[:j])    # first seen at place j >= 3
             results["eos"], results["stop_after"] = probe[at], at
         engine = engine_from_folder(folders[name], scheduler_config=scheduler, dtype=dtype, eos_token_ids=[results["eos"]])
-        ids = [engine.submit(p, sampling_params=SamplingParams(max_new_tokens=n)) for p, n in zip(prompts[:4], limits[:4])]
+        ids = [engine.submit(p, sampling_params=sampling(n, 100 + i)) for i, (p, n) in enumerate(zip(prompts[:4], limits[:4]))]
         steps = 0
         while not engine.idle:
             engine.step()
             steps += 1
             if steps == 6:
-                ids.append(engine.submit(prompts[4], sampling_params=SamplingParams(max_new_tokens=limits[4])))   # joins late
+                ids.append(engine.submit(prompts[4], sampling_params=sampling(limits[4], 104)))   # joins late
             if steps == 12:
                 engine.cancel(ids[2])
         views = [engine.request(i) for i in ids]
