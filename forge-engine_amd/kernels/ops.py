@@ -832,7 +832,7 @@ def pack_sample_params(rows) -> Tensor:
     (temperature, top_k or None, top_p, min_p, seed, draw index); temperature 0 asks for the arg-max."""
     packed = np.zeros(len(rows), dtype=_SAMPLE_PARAMS)
     for i, (temperature, top_k, top_p, min_p, seed, draw) in enumerate(rows):
-        packed[i] = (temperature, top_k or 0, top_p, min_p, seed & (2**64 - 1), draw & (2**64 - 1))
+        packed[i] = (temperature, min(top_k or 0, 2**31 - 1), top_p, min_p, seed & (2**64 - 1), draw & (2**64 - 1))
     return torch.from_numpy(packed.view(np.int32).reshape(len(rows), SAMPLE_PARAM_WORDS))
 
 
