@@ -319,6 +319,7 @@ WIDE_UPDATE_FEW_WEIGHT_ROWS = 3072   # weight measured (hidden sizes 2560, 4096,
                                      # hidden sizes 4096 and 5120 are the library's by a tenth
 WIDE_STORE_MAX_ROWS = 256      # ... and a product that stores bfloat16
 WIDE_MAX_WEIGHT_ROWS = 8192    # weights with more rows fill the chip in the library's large tiles
+WIDE_GATE_MAX_K = 4096         # the gate/up product for 17 to 64 rows: beyond this K the matrix library is faster
 WIDE_CUS = 256                 # the product's blocks run one a CU, round after round: the parts of K are chosen to fill the rounds
 
 
@@ -429,7 +430,8 @@ def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
         return None
     if _skinny_fits(x, weight):
         return gemm_skinny(x, weight, "f32", tiles=1, waves=4, splits=IN_PARTS_FEW_ROWS)
-    if _mid_fits(x, weight):
+    if _mid_fits(x, weight) and weight.shape[0] <= WIDE_MAX_WEIGHT_ROWS:
+        # (a weight of 10240 rows, K = 5120: 30 us at 32 rows against the library's 26; 7168 rows: 18 against 20)
         return gemm_mid_parts(x, weight, _mid_parts(steps, -(-weight.shape[0] // 64), most=4))
     return None
 
@@ -452,9 +454,12 @@ def linear_swiglu(x: Tensor, gate_up_weight: Tensor) -> Tensor:
         return gemm_skinny(x, gate_up_weight, "swiglu")
     if (SKINNY_MAX_ROWS < x.shape[0] <= MID_ROWS and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16
             and x.is_contiguous() and gate_up_weight.is_contiguous() and x.shape[1] % 64 == 0
+            and x.shape[1] <= WIDE_GATE_MAX_K
             and gate_up_weight.shape[0] % 2 == 0 and x.data_ptr() % 16 == 0 and gate_up_weight.data_ptr() % 16 == 0):
-        # 17 to 64 rows (many requests decoding): measured at 9728 columns, 24 and 28 us at 32 and 64 rows against
-        # 31 and 33 for the matrix library with the gate kernel behind it; from 96 rows on the library wins
+        # 17 to 64 rows (many requests decoding): measured at 32 rows against the matrix library with the gate
+        # kernel behind it: 24 against 28 us at 9728 columns of K = 2560, 46 against 50 at 12288 of K = 4096;
+        # at K = 5120 the library wins (17408 columns: 85 against 82 us, 25600 columns: 111 against 96), and
+        # from 96 rows on at every size
         return gemm_wide(x, gate_up_weight, "swiglu_half", block_rows=_gate_block_columns(gate_up_weight.shape[0] // 2))
     gate_up = linear(x, gate_up_weight)
     out = torch.empty((x.shape[0], gate_up_weight.shape[0] // 2), dtype=gate_up.dtype, device=x.device)

@@ -765,6 +765,14 @@ def test_linear_swiglu_routes_by_rows(ops, monkeypatch):
         gate, up = y[:, :328], y[:, 328:]
         torch.testing.assert_close(got, gate / (1 + torch.exp(-gate)) * up, atol=2e-2, rtol=2e-2)
     assert ops._gate_block_columns(9728) == 40 and ops._gate_block_columns(12288) == 48
+    # a K beyond the one up to which that product wins: the library and the gate kernel at 17 to 64 rows too
+    long_k = rand(g, 2 * 40, 5120, dtype=torch.bfloat16, scale=0.02)
+    x = rand(g, 32, 5120, dtype=torch.bfloat16)
+    taken.clear()
+    got = ops.linear_swiglu(x.to(DEV), long_k.to(DEV)).cpu().float()
+    assert taken[-1] == "fe_swiglu", taken
+    y = x.float() @ long_k.float().t()
+    torch.testing.assert_close(got, y[:, :40] / (1 + torch.exp(-y[:, :40])) * y[:, 40:], atol=2e-2, rtol=2e-2)
 
 
 def test_gemm_wide_refuses_and_routes(ops, monkeypatch):
