@@ -227,6 +227,31 @@ def gemm_skinny(x: Tensor, weight: Tensor, epilogue: str = "bf16", tiles: int = 
     return out
 
 
+# Which kernel takes a product of up to 16 rows, measured in the decode step at the sizes of Qwen3-4B, 8B and 32B
+# (hidden 2560 / 4096 / 5120; milliseconds a step before -> after at the batch named):
+# * updates of the stream (output and down projections): the K-split kernel for up to 16 rows is the fastest only
+#   where few rows meet a narrow weight; from 9 rows (4B, batch 16: 3.35 -> 3.22), and from 4 rows where the weight
+#   has more than 3072 rows (8B, batch 8: 4.15 -> 3.96; 32B, batch 16: 18.2 -> 16.3), the product for portions
+#   (one tile of 64 rows of x in LDS, K in the parts that fill the CUs) is faster, and faster than the library
+#   (8B, batch 16: 4.39 against 4.45);
+# * q/k/v: from 9 rows the product for 17 to 64 rows in parts (4B, batch 16: 3.35 -> 3.32; 8B: 4.84 -> 4.75); a weight
+#   of more than 8192 rows goes to the library from 9 rows (32B, batch 16: 15.85 -> 15.00 with the other two in place);
+# * gate/up: K up to 3072: from 9 rows the product that pairs gate and up rows in a wave (4B, batch 16: 3.35 -> 3.28;
+#   at K = 4096 it loses: 8B, batch 16: 4.84 -> 4.96); a weight of more than 40,000 rows goes to the library from
+#   2 rows (32B: 13.86 -> 13.50 at batch 2, 14.75 -> 14.27 at batch 8, 16.35 -> 15.85 at batch 16; a weight of 34,816
+#   rows at the same K does not: 72 against 78 us at 8 rows).
+FEW_ROWS = 8                        # up to here the kernels for up to 16 rows win wherever they fit
+FEW_ROWS_TALL_UPDATE = 3            # ... for updates through a weight of more than WIDE_UPDATE_FEW_WEIGHT_ROWS rows: up to here
+GATE_HALF_FEW_ROWS_MAX_K = 3072     # gate/up from FEW_ROWS + 1 rows in the product for 17 to 64 rows: K up to here
+GATE_LIBRARY_WEIGHT_ROWS = 40000    # gate/up through a weight of more rows than this: the library from 2 rows
+
+
+def _few_rows_to_library(x: Tensor, weight: Tensor) -> bool:
+    """A product that stores bfloat16 (q/k/v), 9 to 16 rows, a weight of more rows than the products
+    for portions take: the matrix library."""
+    return FEW_ROWS < x.shape[0] <= SKINNY_MAX_ROWS and weight.shape[0] > WIDE_MAX_WEIGHT_ROWS
+
+
 def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None) -> Tensor:
     """y = x @ weight^T (+ bias) for a weight in [out, in] layout; float32
     accumulation; y in ``out_dtype`` (default: x's dtype).
@@ -245,7 +270,8 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
         return y if out_dtype == torch.float32 else y.to(out_dtype)
     if x.dtype != weight.dtype:
         raise KernelError(f"activation {x.dtype} does not match weight {weight.dtype}")
-    if bias is None and _skinny_fits(x, weight) and out_dtype in (torch.float32, torch.bfloat16):
+    if (bias is None and _skinny_fits(x, weight) and out_dtype in (torch.float32, torch.bfloat16)
+            and not (out_dtype == torch.bfloat16 and _few_rows_to_library(x, weight))):
         return gemm_skinny(x, weight, "f32" if out_dtype == torch.float32 else "bf16")
     if bias is None and out_dtype == torch.bfloat16 and _wide_fits(x, weight, WIDE_STORE_MAX_ROWS, SKINNY_MAX_ROWS + 1):
         rows = x.shape[0]        # up to 64 rows: blocks of 32 weight rows, so that the launch has twice the blocks
@@ -382,6 +408,9 @@ def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None, stream:
     _gpu(x, "x")
     _gpu(weight, "weight", contiguous=False)
     plain_bf16 = bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+    few = FEW_ROWS_TALL_UPDATE if weight.shape[0] > WIDE_UPDATE_FEW_WEIGHT_ROWS else FEW_ROWS
+    if plain_bf16 and few < x.shape[0] <= SKINNY_MAX_ROWS and _wide_fits(x, weight, SKINNY_MAX_ROWS, 1):
+        return gemm_wide(x, weight, "parts", _wide_parts(x.shape[0], weight.shape[0], weight.shape[1]), row_tile=64)
     if (plain_bf16 and _skinny_fits(x, weight)
             and -(-weight.shape[0] // 16) <= UPDATE_SPLIT_MAX_TILES
             and -(-weight.shape[1] // 128) >= UPDATE_SPLIT_MIN_STEPS):
@@ -428,7 +457,7 @@ def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
     steps = -(-weight.shape[1] // 128)
     if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and steps >= IN_PARTS_MIN_STEPS):
         return None
-    if _skinny_fits(x, weight):
+    if _skinny_fits(x, weight) and x.shape[0] <= FEW_ROWS:
         return gemm_skinny(x, weight, "f32", tiles=1, waves=4, splits=IN_PARTS_FEW_ROWS)
     if _mid_fits(x, weight) and weight.shape[0] <= WIDE_MAX_WEIGHT_ROWS:
         # (a weight of 10240 rows, K = 5120: 30 us at 32 rows against the library's 26; 7168 rows: 18 against 20)
@@ -450,9 +479,13 @@ def linear_swiglu(x: Tensor, gate_up_weight: Tensor) -> Tensor:
     """silu(x Wg^T) * (x Wu^T) for the fused weight [2I, K] (gate rows first)."""
     _gpu(x, "x")
     _gpu(gate_up_weight, "gate_up_weight")
-    if _skinny_fits(x, gate_up_weight):
+    rows = x.shape[0]
+    to_library = (2 <= rows <= SKINNY_MAX_ROWS and gate_up_weight.shape[0] > GATE_LIBRARY_WEIGHT_ROWS
+                  and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16)
+    paired_from = FEW_ROWS if x.shape[1] <= GATE_HALF_FEW_ROWS_MAX_K else SKINNY_MAX_ROWS
+    if _skinny_fits(x, gate_up_weight) and rows <= paired_from and not to_library:
         return gemm_skinny(x, gate_up_weight, "swiglu")
-    if (SKINNY_MAX_ROWS < x.shape[0] <= MID_ROWS and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16
+    if (paired_from < rows <= MID_ROWS and not to_library and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16
             and x.is_contiguous() and gate_up_weight.is_contiguous() and x.shape[1] % 64 == 0
             and x.shape[1] <= WIDE_GATE_MAX_K
             and gate_up_weight.shape[0] % 2 == 0 and x.data_ptr() % 16 == 0 and gate_up_weight.data_ptr() % 16 == 0):
@@ -461,7 +494,7 @@ def linear_swiglu(x: Tensor, gate_up_weight: Tensor) -> Tensor:
         # at K = 5120 the library wins (17408 columns: 85 against 82 us, 25600 columns: 111 against 96), and
         # from 96 rows on at every size
         return gemm_wide(x, gate_up_weight, "swiglu_half", block_rows=_gate_block_columns(gate_up_weight.shape[0] // 2))
-    gate_up = linear(x, gate_up_weight)
+    gate_up = torch.matmul(x, gate_up_weight.t()) if to_library else linear(x, gate_up_weight)
     out = torch.empty((x.shape[0], gate_up_weight.shape[0] // 2), dtype=gate_up.dtype, device=x.device)
     return swiglu(gate_up, out)
 

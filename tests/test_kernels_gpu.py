@@ -666,7 +666,12 @@ def test_linear_update_routes(ops):
     few_rows = rand(g, 320, 4096, dtype=torch.bfloat16, scale=0.05).to(DEV)
     many_rows = rand(g, 8192, 4096, dtype=torch.bfloat16, scale=0.05).to(DEV)
     assert ops.linear_update(x, few_rows).dim() == 3              # few row tiles, long K: parts
-    assert ops.linear_update(x, many_rows).dim() == 2
+    assert ops.linear_update(x[:3].contiguous(), many_rows).dim() == 2     # many row tiles, up to three rows: K whole
+    tall = ops.linear_update(x, many_rows)                        # four to 16 rows through a weight of many rows: the product for portions
+    assert tall.dim() == 3
+    torch.testing.assert_close(tall.sum(0).cpu(), x.float().cpu() @ many_rows.float().cpu().T, atol=2e-3, rtol=2e-3)
+    x12 = rand(g, 12, 4096, dtype=torch.bfloat16).to(DEV)         # nine to 16 rows: the same whatever the weight
+    torch.testing.assert_close(ops.linear_update(x12, few_rows).sum(0).cpu(), x12.float().cpu() @ few_rows.float().cpu().T, atol=2e-3, rtol=2e-3)
     assert ops.linear_update(x[:, :1024].contiguous(), few_rows[:, :1024]).dim() == 2
     big = rand(g, 70, 4096, dtype=torch.bfloat16).to(DEV)
     assert ops.linear_update(big, few_rows).shape[1:] == (70, 320)     # 65 to 384 rows: the product for portions, in parts
