@@ -182,8 +182,9 @@ __global__ __launch_bounds__(64 * WPB, 2) void gemm_wide_kernel(
 //   of a result tile meet by a lane exchange), so that a block takes 8 columns a wave: block_rows = 32 to 64
 //   in steps of 8 (four to eight waves) is then the block's columns, chosen so that the blocks fill rounds of
 //   one a CU.
-// Any M: rows are taken in tiles of row_tile = 64 or 128 (smaller tiles: more blocks, and the weight
-// read again, from L2, once per tile).  block_rows = 64 or 32: the weight rows (gate/up ending: output
+// Any M: rows are taken in tiles of row_tile = 16, 32, 64 or 128 (smaller tiles: more blocks, and the weight
+// read again, from L2, once per tile; a tile's rows beyond M are fetched and multiplied all the same, so
+// few rows want a small tile; ending 2 takes tiles of 64 and 128 only).  block_rows = 64 or 32: the weight rows (gate/up ending: output
 // columns) a block of four or two waves takes; 32 gives a launch of few blocks twice as many; 128 (eight
 // waves, plain endings) halves how often x is read.
 extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int N, int K, long long ldw,
@@ -197,7 +198,7 @@ extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int 
   if (parts > 1 && part_stride < (long long)M * ldo) return FE_BAD_ARGUMENT;
   const int steps = K / WSTEP;
   const int per_part = (steps + parts - 1) / parts;
-  if (row_tile != 64 && row_tile != 128) return FE_BAD_ARGUMENT;
+  if (row_tile != 16 && row_tile != 32 && row_tile != 64 && row_tile != 128) return FE_BAD_ARGUMENT;
   const int mt = row_tile / 16;
   const long long m_tiles = (M + mt * 16 - 1) / (mt * 16);
   if (m_tiles > 65535) return FE_BAD_ARGUMENT;
@@ -221,7 +222,13 @@ extern "C" int fe_gemm_wide(const void* x, const void* w, void* out, int M, int 
     else if (waves == 6) FE_LAUNCH(MT, EPI_SWIGLU_HALF, 6); else if (waves == 7) FE_LAUNCH(MT, EPI_SWIGLU_HALF, 7); \
     else FE_LAUNCH(MT, EPI_SWIGLU_HALF, 8);                                                                      \
   } while (0)
-  if (mt == 4) {
+  if (mt == 1) {         // up to 16 rows a tile: the plain endings and the half-tile gate/up ending
+    if (ending == EPI_PARTS) FE_GO(1, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(1, EPI_BF16);
+    else if (ending == EPI_SWIGLU) return FE_BAD_ARGUMENT; else FE_HALF(1);
+  } else if (mt == 2) {
+    if (ending == EPI_PARTS) FE_GO(2, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(2, EPI_BF16);
+    else if (ending == EPI_SWIGLU) return FE_BAD_ARGUMENT; else FE_HALF(2);
+  } else if (mt == 4) {
     if (ending == EPI_PARTS) FE_GO(4, EPI_PARTS); else if (ending == EPI_BF16) FE_GO(4, EPI_BF16);
     else if (ending == EPI_SWIGLU) FE_GO(4, EPI_SWIGLU); else FE_HALF(4);
   } else {

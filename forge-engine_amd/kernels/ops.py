@@ -228,21 +228,22 @@ def gemm_skinny(x: Tensor, weight: Tensor, epilogue: str = "bf16", tiles: int = 
 
 
 # Which kernel takes a product of up to 16 rows, measured in the decode step at the sizes of Qwen3-4B, 8B and 32B
-# (hidden 2560 / 4096 / 5120; milliseconds a step before -> after at the batch named):
-# * updates of the stream (output and down projections): the K-split kernel for up to 16 rows is the fastest only
-#   where few rows meet a narrow weight; from 9 rows (4B, batch 16: 3.35 -> 3.22), and from 4 rows where the weight
-#   has more than 3072 rows (8B, batch 8: 4.15 -> 3.96; 32B, batch 16: 18.2 -> 16.3), the product for portions
-#   (one tile of 64 rows of x in LDS, K in the parts that fill the CUs) is faster, and faster than the library
-#   (8B, batch 16: 4.39 against 4.45);
+# (hidden 2560 / 4096 / 5120; milliseconds a step before -> after at the batch named).  The kernels for up to 16
+# rows (`fe_gemm_skinny`) were shaped at 8 rows of the 4B sizes; the product for portions (`fe_gemm_wide`: a tile
+# of 16 rows of x in LDS, 64 weight rows a block, K in the parts that fill the CUs) turned out faster for:
+# * updates of the stream (output and down projections) from 4 rows (4B, batch 8: 2.83 -> 2.79, batch 16: 3.35 ->
+#   3.17; 8B, batch 8: 4.15 -> 3.96; 32B, batch 16: 18.2 -> 16.3), and faster than the library there (8B, batch 16:
+#   4.39 against 4.45); with up to 3 rows the K-split kernel stays (4B, batch 1: 2.50 against 2.51);
+# * gate/up at K up to 3072, with gate and up rows paired in a wave, at every row count (4B: 2.50 -> 2.48 at batch 1,
+#   2.83 -> 2.79 at batch 8, 3.35 -> 3.28 at batch 16); at K = 4096 the kernel whose blocks keep x in registers wins
+#   (8B, batch 8: 3.94 against 4.15); a weight of more than 40,000 rows goes to the library from 2 rows (32B: 13.86
+#   -> 13.50 at batch 2, 14.75 -> 14.27 at batch 8, 16.35 -> 15.85 at batch 16; a weight of 34,816 rows at the same
+#   K does not: 72 against 78 us at 8 rows);
 # * q/k/v: from 9 rows the product for 17 to 64 rows in parts (4B, batch 16: 3.35 -> 3.32; 8B: 4.84 -> 4.75); a weight
-#   of more than 8192 rows goes to the library from 9 rows (32B, batch 16: 15.85 -> 15.00 with the other two in place);
-# * gate/up: K up to 3072: from 9 rows the product that pairs gate and up rows in a wave (4B, batch 16: 3.35 -> 3.28;
-#   at K = 4096 it loses: 8B, batch 16: 4.84 -> 4.96); a weight of more than 40,000 rows goes to the library from
-#   2 rows (32B: 13.86 -> 13.50 at batch 2, 14.75 -> 14.27 at batch 8, 16.35 -> 15.85 at batch 16; a weight of 34,816
-#   rows at the same K does not: 72 against 78 us at 8 rows).
-FEW_ROWS = 8                        # up to here the kernels for up to 16 rows win wherever they fit
-FEW_ROWS_TALL_UPDATE = 3            # ... for updates through a weight of more than WIDE_UPDATE_FEW_WEIGHT_ROWS rows: up to here
-GATE_HALF_FEW_ROWS_MAX_K = 3072     # gate/up from FEW_ROWS + 1 rows in the product for 17 to 64 rows: K up to here
+#   of more than 8192 rows goes to the library from 9 rows (32B, batch 16: 15.85 -> 15.00 with the other two in place).
+FEW_ROWS = 8                        # q/k/v: up to here the kernel for up to 16 rows
+FEW_ROWS_UPDATE = 3                 # updates of the stream: up to here
+GATE_HALF_FEW_ROWS_MAX_K = 3072     # gate/up in the product that pairs gate and up rows at every row count: K up to here
 GATE_LIBRARY_WEIGHT_ROWS = 40000    # gate/up through a weight of more rows than this: the library from 2 rows
 
 
@@ -379,7 +380,7 @@ def gemm_wide(x: Tensor, weight: Tensor, ending: str = "bf16", parts: int = 1, r
         raise KernelError(f"no ending {ending!r} with {parts} parts")
     _call("gemm_wide", "fe_gemm_wide", _ptr(x), _ptr(weight), _ptr(out), c_int(m), c_int(cols), c_int(k),
           c_longlong(weight.stride(0)), c_longlong(cols), c_int(code), c_int(parts), c_longlong(m * cols),
-          c_int(row_tile or (64 if m <= 64 else 128)), c_int(block_rows), _stream())
+          c_int(row_tile or (16 if m <= 16 else 64 if m <= 64 else 128)), c_int(block_rows), _stream())
     return out
 
 
@@ -408,9 +409,10 @@ def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None, stream:
     _gpu(x, "x")
     _gpu(weight, "weight", contiguous=False)
     plain_bf16 = bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
-    few = FEW_ROWS_TALL_UPDATE if weight.shape[0] > WIDE_UPDATE_FEW_WEIGHT_ROWS else FEW_ROWS
-    if plain_bf16 and few < x.shape[0] <= SKINNY_MAX_ROWS and _wide_fits(x, weight, SKINNY_MAX_ROWS, 1):
-        return gemm_wide(x, weight, "parts", _wide_parts(x.shape[0], weight.shape[0], weight.shape[1]), row_tile=64)
+    if plain_bf16 and FEW_ROWS_UPDATE < x.shape[0] <= SKINNY_MAX_ROWS and _wide_fits(x, weight, SKINNY_MAX_ROWS, 1):
+        # a tile of 16 rows of x: a tile's rows beyond M are fetched and multiplied like the others (with tiles of
+        # 64 rows: 4B, batch 16: 3.05 -> 3.00 ms; 32B: 15.4 -> 14.9; tiles of 32 rows for 17 to 32 rows lose 2 to 6 %)
+        return gemm_wide(x, weight, "parts", _wide_parts(x.shape[0], weight.shape[0], weight.shape[1]), row_tile=16)
     if (plain_bf16 and _skinny_fits(x, weight)
             and -(-weight.shape[0] // 16) <= UPDATE_SPLIT_MAX_TILES
             and -(-weight.shape[1] // 128) >= UPDATE_SPLIT_MIN_STEPS):
@@ -482,18 +484,18 @@ def linear_swiglu(x: Tensor, gate_up_weight: Tensor) -> Tensor:
     rows = x.shape[0]
     to_library = (2 <= rows <= SKINNY_MAX_ROWS and gate_up_weight.shape[0] > GATE_LIBRARY_WEIGHT_ROWS
                   and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16)
-    paired_from = FEW_ROWS if x.shape[1] <= GATE_HALF_FEW_ROWS_MAX_K else SKINNY_MAX_ROWS
-    if _skinny_fits(x, gate_up_weight) and rows <= paired_from and not to_library:
-        return gemm_skinny(x, gate_up_weight, "swiglu")
-    if (paired_from < rows <= MID_ROWS and not to_library and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16
-            and x.is_contiguous() and gate_up_weight.is_contiguous() and x.shape[1] % 64 == 0
-            and x.shape[1] <= WIDE_GATE_MAX_K
-            and gate_up_weight.shape[0] % 2 == 0 and x.data_ptr() % 16 == 0 and gate_up_weight.data_ptr() % 16 == 0):
-        # 17 to 64 rows (many requests decoding): measured at 32 rows against the matrix library with the gate
-        # kernel behind it: 24 against 28 us at 9728 columns of K = 2560, 46 against 50 at 12288 of K = 4096;
-        # at K = 5120 the library wins (17408 columns: 85 against 82 us, 25600 columns: 111 against 96), and
-        # from 96 rows on at every size
+    paired_fits = (rows <= MID_ROWS and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16
+                   and x.is_contiguous() and gate_up_weight.is_contiguous() and x.shape[1] % 64 == 0
+                   and x.shape[1] <= WIDE_GATE_MAX_K and gate_up_weight.shape[0] % 2 == 0
+                   and x.data_ptr() % 16 == 0 and gate_up_weight.data_ptr() % 16 == 0)
+    if paired_fits and not to_library and (rows > SKINNY_MAX_ROWS or x.shape[1] <= GATE_HALF_FEW_ROWS_MAX_K):
+        # gate and up rows paired in a wave.  17 to 64 rows (many requests decoding), measured at 32 rows against the
+        # matrix library with the gate kernel behind it: 24 against 28 us at 9728 columns of K = 2560, 46 against 50 at
+        # 12288 of K = 4096; at K = 5120 the library wins (17408 columns: 85 against 82 us, 25600 columns: 111 against
+        # 96), and from 96 rows on at every size.  Up to 16 rows: see FEW_ROWS above.
         return gemm_wide(x, gate_up_weight, "swiglu_half", block_rows=_gate_block_columns(gate_up_weight.shape[0] // 2))
+    if _skinny_fits(x, gate_up_weight) and not to_library:
+        return gemm_skinny(x, gate_up_weight, "swiglu")
     gate_up = torch.matmul(x, gate_up_weight.t()) if to_library else linear(x, gate_up_weight)
     out = torch.empty((x.shape[0], gate_up_weight.shape[0] // 2), dtype=gate_up.dtype, device=x.device)
     return swiglu(gate_up, out)

@@ -587,8 +587,8 @@ def test_gemm_skinny_swiglu(ops, m, inter, k):
     want = refs.linear_swiglu(x, w).float()
     got = ops.gemm_skinny(x.to(DEV), w.to(DEV), "swiglu").cpu().float()
     torch.testing.assert_close(got, want, atol=1e-2 * float(want.abs().max()) + 1e-6, rtol=1e-2)
-    routed = ops.linear_swiglu(x.to(DEV), w.to(DEV)).cpu().float()   # up to 16 rows: this kernel; more: library + SwiGLU kernel
-    if m <= 16:
+    routed = ops.linear_swiglu(x.to(DEV), w.to(DEV)).cpu().float()
+    if m <= 16 and k % 64:       # up to 16 rows where the product that pairs gate and up rows does not fit: this kernel
         assert torch.equal(routed, got)
     torch.testing.assert_close(routed, want, atol=1e-2 * float(want.abs().max()) + 1e-6, rtol=1e-2)
 
@@ -672,7 +672,10 @@ def test_linear_update_routes(ops):
     torch.testing.assert_close(tall.sum(0).cpu(), x.float().cpu() @ many_rows.float().cpu().T, atol=2e-3, rtol=2e-3)
     x12 = rand(g, 12, 4096, dtype=torch.bfloat16).to(DEV)         # nine to 16 rows: the same whatever the weight
     torch.testing.assert_close(ops.linear_update(x12, few_rows).sum(0).cpu(), x12.float().cpu() @ few_rows.float().cpu().T, atol=2e-3, rtol=2e-3)
-    assert ops.linear_update(x[:, :1024].contiguous(), few_rows[:, :1024]).dim() == 2
+    assert ops.linear_update(x[:3, :1024].contiguous(), few_rows[:, :1024]).dim() == 2      # a short K, up to three rows: K whole
+    short = ops.linear_update(x[:, :1024].contiguous(), few_rows[:, :1024])
+    torch.testing.assert_close((short.sum(0) if short.dim() == 3 else short).cpu(),
+                               x[:, :1024].float().cpu() @ few_rows[:, :1024].float().cpu().T, atol=1e-3, rtol=1e-3)
     big = rand(g, 70, 4096, dtype=torch.bfloat16).to(DEV)
     assert ops.linear_update(big, few_rows).shape[1:] == (70, 320)     # 65 to 384 rows: the product for portions, in parts
     huge = rand(g, 500, 4096, dtype=torch.bfloat16).to(DEV)
@@ -712,7 +715,7 @@ def test_gemm_mid_parts(ops, m, n, k, parts):
 
 @pytest.mark.parametrize("m", [17, 33, 64, 65, 100, 128, 130, 300])
 @pytest.mark.parametrize("n,k,parts", [(2560, 4096, 8), (200, 256, 2), (1003, 1024, 3), (64, 64, 1), (70, 640, 5), (330, 9728, 16)])
-@pytest.mark.parametrize("row_tile", [64, 128])
+@pytest.mark.parametrize("row_tile", [16, 32, 64, 128])
 def test_gemm_wide_parts(ops, m, n, k, parts, row_tile):
     """The product for portions of prompts: partial sums over parts of K (parts without steps are
     zeros), any number of rows in tiles of 64 or 128, weight rows that are no multiple of the
@@ -733,7 +736,7 @@ def test_gemm_wide_parts(ops, m, n, k, parts, row_tile):
         torch.testing.assert_close(got[part].cpu(), want_part, atol=1e-3 * (k / 256) ** 0.5, rtol=1e-3)
 
 
-@pytest.mark.parametrize("m", [20, 64, 77, 256, 260])
+@pytest.mark.parametrize("m", [9, 16, 20, 64, 77, 256, 260])
 @pytest.mark.parametrize("n,k", [(6144, 2560), (200, 192), (1002, 320)])
 def test_gemm_wide_stores_and_gates(ops, m, n, k):
     g = torch.Generator().manual_seed(m * 3 + n + k)
@@ -751,17 +754,26 @@ def test_gemm_wide_stores_and_gates(ops, m, n, k):
     for width in (32, 40, 48, 56, 64):
         gated = ops.gemm_wide(x.to(DEV), w.to(DEV), "swiglu_half", 1, 64 if width != 48 else 128, width)
         torch.testing.assert_close(gated.cpu().float(), (gate / (1 + torch.exp(-gate)) * up), atol=2e-2, rtol=2e-2)
+    # tiles of 16 and 32 rows (what few rows take): the plain stores and the half-tile gate ending
+    for row_tile, width in ((16, 40), (32, 64), (16, 32)):
+        got = ops.gemm_wide(x.to(DEV), w.to(DEV), "bf16", 1, row_tile, 64 if width != 32 else 32)
+        torch.testing.assert_close(got.cpu().float(), want.to(torch.bfloat16).float(), atol=2e-2, rtol=2e-2)
+        gated = ops.gemm_wide(x.to(DEV), w.to(DEV), "swiglu_half", 1, row_tile, width)
+        torch.testing.assert_close(gated.cpu().float(), (gate / (1 + torch.exp(-gate)) * up), atol=2e-2, rtol=2e-2)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_wide(x.to(DEV), w.to(DEV), "swiglu", 1, 16, 64)        # the two-tile gate ending takes tiles of 64 and 128 rows
 
 
 def test_linear_swiglu_routes_by_rows(ops, monkeypatch):
-    """Up to 16 rows: the streaming kernel; 17 to 64: the product that pairs gate and up rows within a
-    wave; more: the matrix library and the gate kernel.  All give the plain result."""
+    """Up to 64 rows at a K of up to 3072: the product that pairs gate and up rows within a wave (at a
+    longer K from 17 rows, the streaming kernel below); more: the matrix library and the gate kernel.
+    All give the plain result."""
     g = torch.Generator().manual_seed(33)
     w = rand(g, 2 * 328, 256, dtype=torch.bfloat16, scale=0.05)
     taken = []
     real_call = ops._call
     monkeypatch.setattr(ops, "_call", lambda lib, name, *a: taken.append(name) or real_call(lib, name, *a))
-    for rows, name in ((8, "fe_gemm_skinny"), (17, "fe_gemm_wide"), (64, "fe_gemm_wide"), (65, "fe_swiglu")):
+    for rows, name in ((1, "fe_gemm_wide"), (8, "fe_gemm_wide"), (17, "fe_gemm_wide"), (64, "fe_gemm_wide"), (65, "fe_swiglu")):
         x = rand(g, rows, 256, dtype=torch.bfloat16)
         taken.clear()
         got = ops.linear_swiglu(x.to(DEV), w.to(DEV)).cpu().float()
@@ -770,6 +782,15 @@ def test_linear_swiglu_routes_by_rows(ops, monkeypatch):
         gate, up = y[:, :328], y[:, 328:]
         torch.testing.assert_close(got, gate / (1 + torch.exp(-gate)) * up, atol=2e-2, rtol=2e-2)
     assert ops._gate_block_columns(9728) == 40 and ops._gate_block_columns(12288) == 48
+    # a K of 4096: the streaming kernel up to 16 rows, the paired product from 17
+    mid_k = rand(g, 2 * 40, 4096, dtype=torch.bfloat16, scale=0.02)
+    for rows, name in ((8, "fe_gemm_skinny"), (16, "fe_gemm_skinny"), (17, "fe_gemm_wide")):
+        x = rand(g, rows, 4096, dtype=torch.bfloat16)
+        taken.clear()
+        got = ops.linear_swiglu(x.to(DEV), mid_k.to(DEV)).cpu().float()
+        assert taken[-1] == name, (rows, taken)
+        y = x.float() @ mid_k.float().t()
+        torch.testing.assert_close(got, y[:, :40] / (1 + torch.exp(-y[:, :40])) * y[:, 40:], atol=2e-2, rtol=2e-2)
     # a K beyond the one up to which that product wins: the library and the gate kernel at 17 to 64 rows too
     long_k = rand(g, 2 * 40, 5120, dtype=torch.bfloat16, scale=0.02)
     x = rand(g, 32, 5120, dtype=torch.bfloat16)
