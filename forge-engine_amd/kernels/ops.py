@@ -239,9 +239,11 @@ def gemm_skinny(x: Tensor, weight: Tensor, epilogue: str = "bf16", tiles: int = 
 #   (8B, batch 8: 3.94 against 4.15); a weight of more than 40,000 rows goes to the library from 2 rows (32B: 13.86
 #   -> 13.50 at batch 2, 14.75 -> 14.27 at batch 8, 16.35 -> 15.85 at batch 16; a weight of 34,816 rows at the same
 #   K does not: 72 against 78 us at 8 rows);
-# * q/k/v: from 9 rows the product for 17 to 64 rows in parts (4B, batch 16: 3.35 -> 3.32; 8B: 4.84 -> 4.75); a weight
-#   of more than 8192 rows goes to the library from 9 rows (32B, batch 16: 15.85 -> 15.00 with the other two in place).
-FEW_ROWS = 8                        # q/k/v: up to here the kernel for up to 16 rows
+# * q/k/v: from 5 rows, in up to four parts that the attention launch adds up (4B, batch 8: 2.74 -> 2.71, batch 16:
+#   3.35 -> 3.31; 8B, batch 16: 4.84 -> 4.70); a weight of more than 8192 rows stays with the kernel for up to 16
+#   rows to 8 rows and goes to the library from 9 (32B, batch 16: 15.85 -> 15.00 with the other two in place).
+FEW_ROWS = 8                        # q/k/v where the product for portions does not fit: up to here the kernel for up to 16 rows
+FEW_ROWS_IN_PARTS = 4               # q/k/v: up to here the kernel for up to 16 rows, then the product for portions in parts
 FEW_ROWS_UPDATE = 3                 # updates of the stream: up to here
 GATE_HALF_FEW_ROWS_MAX_K = 3072     # gate/up in the product that pairs gate and up rows at every row count: K up to here
 GATE_LIBRARY_WEIGHT_ROWS = 40000    # gate/up through a weight of more rows than this: the library from 2 rows
@@ -384,7 +386,7 @@ def gemm_wide(x: Tensor, weight: Tensor, ending: str = "bf16", parts: int = 1, r
     return out
 
 
-def _wide_parts(m: int, n: int, k: int, block_rows: int = 64) -> int:
+def _wide_parts(m: int, n: int, k: int, block_rows: int = 64, most: int = 16) -> int:
     """Parts of K for the product above.  Its blocks run one a CU in rounds, so the count of parts is
     the one whose blocks fill their rounds best (measured at 40 to 160 blocks a part: 240 blocks beat
     280 and 320, 480 beat 160 and 320), the smaller of near equals (every part writes and the consumer
@@ -392,7 +394,7 @@ def _wide_parts(m: int, n: int, k: int, block_rows: int = 64) -> int:
     steps = k // 64
     base = -(-n // block_rows) * -(-m // (64 if m <= 64 else 128))
     best, best_fill = 1, 0.0
-    for parts in range(1, max(1, min(16, steps // 8)) + 1):
+    for parts in range(1, max(1, min(most, steps // 8)) + 1):
         blocks = base * parts
         fill = blocks / (-(-blocks // WIDE_CUS) * WIDE_CUS) - 0.02 * parts
         if fill > best_fill + 1e-9:
@@ -459,7 +461,13 @@ def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
     steps = -(-weight.shape[1] // 128)
     if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and steps >= IN_PARTS_MIN_STEPS):
         return None
-    if _skinny_fits(x, weight) and x.shape[0] <= FEW_ROWS:
+    rows = x.shape[0]
+    if FEW_ROWS_IN_PARTS < rows <= SKINNY_MAX_ROWS and _wide_fits(x, weight, SKINNY_MAX_ROWS, 1):
+        # blocks of 32 weight rows in up to four parts of K (768 blocks for 6144 weight rows): 1 % of the step
+        # at 6 to 16 rows against the kernels below (4B, batch 8: 2.74 -> 2.71 ms; 8B: 3.93 -> 3.89)
+        parts = _wide_parts(rows, weight.shape[0], weight.shape[1], 32, most=4)
+        return gemm_wide(x, weight, "parts", parts, row_tile=16, block_rows=32)
+    if _skinny_fits(x, weight) and rows <= FEW_ROWS:
         return gemm_skinny(x, weight, "f32", tiles=1, waves=4, splits=IN_PARTS_FEW_ROWS)
     if _mid_fits(x, weight) and weight.shape[0] <= WIDE_MAX_WEIGHT_ROWS:
         # (a weight of 10240 rows, K = 5120: 30 us at 32 rows against the library's 26; 7168 rows: 18 against 20)
