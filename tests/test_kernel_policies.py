@@ -26,6 +26,31 @@ def test_parts_of_k_for_the_large_model():
     assert ops._mid_parts(76, 40) == 6
 
 
+@pytest.mark.parametrize("m", [1, 8, 16, 40, 64, 100, 256, 384])
+@pytest.mark.parametrize("n", [64, 320, 2560, 4096, 5120, 6144])
+@pytest.mark.parametrize("k", [64, 512, 2560, 4096, 9728, 25600])
+@pytest.mark.parametrize("block_rows,most", [(64, 16), (32, 4), (128, 16)])
+def test_parts_of_the_product_for_portions(m, n, k, block_rows, most):
+    parts = ops._wide_parts(m, n, k, block_rows, most)
+    steps = k // 64
+    assert 1 <= parts <= most
+    per_part = -(-steps // parts)
+    assert (parts - 1) * per_part < steps                    # no part without steps
+    assert parts == 1 or per_part >= 8                       # a part is at least eight 64-steps long
+
+
+def test_blocks_of_the_products_for_few_rows_fill_the_chip():
+    # Qwen3-4B at up to 16 rows: output and down projections in six parts of 40 blocks (240 of 256 CUs)
+    assert ops._wide_parts(8, 2560, 4096) == 6 and ops._wide_parts(8, 2560, 9728) == 6
+    # q/k/v in blocks of 32 weight rows: 192 blocks a part, four parts (768 = three rounds of 256), never more than
+    # the four that the attention launch adds up
+    assert ops._wide_parts(8, 6144, 2560, 32, most=4) == 4 and ops._wide_parts(8, 6144, 4096, 32, most=4) == 4
+    # Qwen3-8B: 64 blocks a part, four parts fill 256 CUs
+    assert ops._wide_parts(8, 4096, 4096) == 4 and ops._wide_parts(8, 4096, 12288) == 4
+    # gate/up: columns a block so that the blocks fill rounds of one a CU (9728 / 40 = 244, 12288 / 48 = 256)
+    assert ops._gate_block_columns(9728) == 40 and ops._gate_block_columns(12288) == 48
+
+
 @pytest.mark.parametrize("num_decode,kv_heads,max_ctx,expect", [
     (8, 8, 1040, 4), (1, 8, 2048, 16), (64, 8, 1040, 1), (1, 8, 64, 1), (1, 1, 100000, 64),
 ])
