@@ -1,5 +1,5 @@
-// bfloat16 matrix product for a few dozen to a few hundred rows of x (a step that holds a
-// portion of a prompt, or many decoding requests):
+// bfloat16 matrix product for a few to a few hundred rows of x (a step of decoding requests, or
+// one that holds a portion of a prompt):
 //   out[M, N] = x[M, K] * W[N, K]^T
 // with one of three endings: float32 partial sums over parts of K ([parts][M, N]; the consumer, the
 // next norm, adds them in order), bfloat16, or silu(gate) * up as bfloat16 for a fused gate/up
