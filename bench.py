@@ -50,7 +50,7 @@ def _qwen3(**sizes) -> dict:
     return base
 
 
-# Sizes and workloads of the three models the benchmark names; the first is the default.
+# Sizes and workloads of the three models the benchmark names (and one between them); the first is the default.
 MODELS = {
     "qwen3-4b": {
         "label": "Qwen3-4B",
@@ -61,6 +61,13 @@ MODELS = {
     "qwen3-8b": {
         "label": "Qwen3-8B",
         "config": _qwen3(hidden_size=4096, intermediate_size=12288, num_hidden_layers=36, num_attention_heads=32,
+                         rope_theta=1000000.0, tie_word_embeddings=False),
+        "batch": 8, "points": "1,64", "prompt_len": 1024, "context": 8192,
+    },
+    # beside the three: the sizes between them, so that choices measured at those are checked at one more width
+    "qwen3-14b": {
+        "label": "Qwen3-14B",
+        "config": _qwen3(hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40,
                          rope_theta=1000000.0, tie_word_embeddings=False),
         "batch": 8, "points": "1,64", "prompt_len": 1024, "context": 8192,
     },

@@ -240,8 +240,8 @@ def gemm_skinny(x: Tensor, weight: Tensor, epilogue: str = "bf16", tiles: int = 
 #   -> 13.50 at batch 2, 14.75 -> 14.27 at batch 8, 16.35 -> 15.85 at batch 16; a weight of 34,816 rows at the same
 #   K does not: 72 against 78 us at 8 rows);
 # * q/k/v: from 5 rows, in up to four parts that the attention launch adds up (4B, batch 8: 2.74 -> 2.71, batch 16:
-#   3.35 -> 3.31; 8B, batch 16: 4.84 -> 4.70); a weight of more than 8192 rows stays with the kernel for up to 16
-#   rows to 8 rows and goes to the library from 9 (32B, batch 16: 15.85 -> 15.00 with the other two in place).
+#   3.35 -> 3.31; 8B, batch 16: 4.84 -> 4.70); a weight of more than 64 MB goes to the library from 5 rows (14B,
+#   batch 8: 6.70 -> 6.61; 32B, batch 16: 15.85 -> 15.00 with the other two in place).
 FEW_ROWS = 8                        # q/k/v where the product for portions does not fit: up to here the kernel for up to 16 rows
 FEW_ROWS_IN_PARTS = 4               # q/k/v: up to here the kernel for up to 16 rows, then the product for portions in parts
 FEW_ROWS_UPDATE = 3                 # updates of the stream: up to here
@@ -249,10 +249,16 @@ GATE_HALF_FEW_ROWS_MAX_K = 3072     # gate/up in the product that pairs gate and
 GATE_LIBRARY_WEIGHT_ROWS = 40000    # gate/up through a weight of more rows than this: the library from 2 rows
 
 
+IN_PARTS_MAX_WEIGHT_BYTES = 64 << 20   # q/k/v from 5 rows: a larger weight than this goes to the library (the 14B sizes'
+                                       # 7168 x 5120, 73 MB: 6.70 -> 6.61 ms a step at batch 8, 7.15 -> 7.05 at 16; the 8B
+                                       # sizes' 6144 x 4096, 50 MB, stays: 3.89 against 3.93)
+
+
 def _few_rows_to_library(x: Tensor, weight: Tensor) -> bool:
-    """A product that stores bfloat16 (q/k/v), 9 to 16 rows, a weight of more rows than the products
-    for portions take: the matrix library."""
-    return FEW_ROWS < x.shape[0] <= SKINNY_MAX_ROWS and weight.shape[0] > WIDE_MAX_WEIGHT_ROWS
+    """A product that stores bfloat16 (q/k/v), 5 to 16 rows, a weight too large for the kernels of
+    few rows to win: the matrix library."""
+    return (FEW_ROWS_IN_PARTS < x.shape[0] <= SKINNY_MAX_ROWS
+            and weight.shape[0] * weight.shape[1] * weight.element_size() > IN_PARTS_MAX_WEIGHT_BYTES)
 
 
 def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None) -> Tensor:
@@ -462,6 +468,8 @@ def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
     if not (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and steps >= IN_PARTS_MIN_STEPS):
         return None
     rows = x.shape[0]
+    if _few_rows_to_library(x, weight):
+        return None
     if FEW_ROWS_IN_PARTS < rows <= SKINNY_MAX_ROWS and _wide_fits(x, weight, SKINNY_MAX_ROWS, 1):
         # blocks of 32 weight rows in up to four parts of K (768 blocks for 6144 weight rows): 1 % of the step
         # at 6 to 16 rows against the kernels below (4B, batch 8: 2.74 -> 2.71 ms; 8B: 3.93 -> 3.89)
