@@ -267,9 +267,10 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
 
     float32 weights go through the true float32 kernel (a weight stored in
     32-bit stays 32-bit even in a bfloat16 model; the activation is widened).
-    bfloat16: up to 64 rows take the weight-streaming kernel; more rows use the
-    platform's matrix library, as the reference does for every projection (its
-    nn.Linear calls, qwen3.py:115-122,215-223).
+    bfloat16: up to 16 rows take the weight-streaming kernel and up to 256 rows the
+    product for portions, where the measurements above and below say they win; the
+    rest is the platform's matrix library's, which the reference uses for every
+    projection (its nn.Linear calls, qwen3.py:115-122,215-223).
     """
     _gpu(x, "x")
     _gpu(weight, "weight", contiguous=False)
