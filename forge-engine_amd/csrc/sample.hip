@@ -1,11 +1,10 @@
 // Sampling over float32 logits rows: argmax, and a draw from softmax(logits / temperature)
-// after top-k, top-p and min-p by inverse CDF with a counter-based generator, one block of
-// 1024 threads per row.  Each row also gets a status word:
+// after top-k, top-p and min-p by inverse CDF with a counter-based generator; a row is shared
+// by several blocks.  Each row also gets a status word:
 //   bit 0: a NaN was seen, bit 1: +inf was seen, bit 2: no finite entry.
 #include "common.h"
 #include "sample_api.h"
 #include <mutex>
-
 
 // tokens[row] = index of the largest entry; the lowest index wins ties.  Two
 // stages so that a few long rows still fill the chip: ARGMAX_PARTS blocks per
@@ -162,7 +161,7 @@ struct RowHeader {                 // what the launch before did for the row, an
   int shift;                       // a refinement's bins are (key - lo) >> shift
   unsigned int lo, hi;             // the keys [lo, hi) that the histogram of that launch splits
   unsigned int key_limit;          // keys up to this one stay (from the searches that are finished)
-  int owner;                       // the pick: the slice in which the running sum passes the target
+  int owner;                       // the pick: the slice in which the running sum passes the target (a row that ends at its maximum: its status)
   unsigned long long target;       // the count or mass to reach within [lo, hi); the pick's target
   unsigned long long before;       // the pick: the sum of the slices before the owner
   float mx;
