@@ -275,6 +275,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_rows_resident_f32_kernel(
 }
 
 #define FE_ROWS_F32_MAX 16     // most rows of A that the weight-streaming variant takes
+#define FE_ROWS_F32_RESIDENT_MAX 64   // most rows of A that go through the variant with A in registers, eight at a time
 
 extern "C" int fe_gemm_nt_f32(const float* A, const float* B, const float* bias, float* C,
                               int M, int N, int K, long long lda, long long ldb, long long ldc,
@@ -283,13 +284,23 @@ extern "C" int fe_gemm_nt_f32(const float* A, const float* B, const float* bias,
   if (K <= 0 || lda < K || ldb < K || ldc < N) return FE_BAD_ARGUMENT;
   const bool rows_ok = M <= FE_ROWS_F32_MAX && K % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 &&
                        ((((uintptr_t)A) | ((uintptr_t)B)) & 15) == 0;
-  if (rows_ok && M <= 8 && K >= 1024) {
-    // persistent blocks, two a CU with four waves (K up to 3,072 a pass), one with eight
+  const bool aligned = K % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 && ((((uintptr_t)A) | ((uintptr_t)B)) & 15) == 0;
+  if (aligned && M <= FE_ROWS_F32_RESIDENT_MAX && K >= 1024) {
+    // persistent blocks, two a CU with four waves (K up to 3,072 a pass), one with eight; more than
+    // eight rows in groups of eight, a launch each: the weight is streamed once a group, which up to
+    // 64 rows still beats the tiles below (measured at the 4B sizes, a decode step: 9 rows 11.7 ->
+    // 8.2 ms, 17 rows 50.4 -> 11.8 ms, 32 rows 51.5 -> 16.2 ms; 64 rows 31.2 ms), and a row's sums
+    // are those of the row alone
     const int tiles = (N + 1) / 2;
-    if (K <= 2048) gemm_rows_resident_f32_kernel<2, 4><<<std::min(tiles, 512), 256, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
-    else if (K <= 3072) gemm_rows_resident_f32_kernel<3, 4><<<std::min(tiles, 512), 256, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
-    else if (K <= 4096) gemm_rows_resident_f32_kernel<2, 8><<<std::min(tiles, 256), 512, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
-    else gemm_rows_resident_f32_kernel<3, 8><<<std::min(tiles, 256), 512, 0, stream>>>(A, B, bias, C, M, N, K, lda, ldb, ldc);
+    for (int m0 = 0; m0 < M; m0 += 8) {
+      const float* a = A + (size_t)m0 * lda;
+      float* c = C + (size_t)m0 * ldc;
+      const int rows = std::min(8, M - m0);
+      if (K <= 2048) gemm_rows_resident_f32_kernel<2, 4><<<std::min(tiles, 512), 256, 0, stream>>>(a, B, bias, c, rows, N, K, lda, ldb, ldc);
+      else if (K <= 3072) gemm_rows_resident_f32_kernel<3, 4><<<std::min(tiles, 512), 256, 0, stream>>>(a, B, bias, c, rows, N, K, lda, ldb, ldc);
+      else if (K <= 4096) gemm_rows_resident_f32_kernel<2, 8><<<std::min(tiles, 256), 512, 0, stream>>>(a, B, bias, c, rows, N, K, lda, ldb, ldc);
+      else gemm_rows_resident_f32_kernel<3, 8><<<std::min(tiles, 256), 512, 0, stream>>>(a, B, bias, c, rows, N, K, lda, ldb, ldc);
+    }
     return fe_check_launch();
   }
   if (rows_ok) {

@@ -131,7 +131,9 @@ def test_add_rows_and_swiglu(ops, dtype):
                                    (1, 9003, 2560), (3, 70, 52), (4, 2560, 4096), (8, 2560, 9728), (7, 1003, 200), (16, 330, 1028),
                                    (13, 6, 4), (9, 5, 1024),
                                    # up to 8 rows and K from 1,024: the rows of A stay in registers (K in one, two or three passes)
-                                   (8, 1003, 2560), (5, 7, 1024), (8, 2561, 3072), (2, 600, 4096), (8, 300, 6148), (6, 131, 12292), (1, 70, 1500)])
+                                   (8, 1003, 2560), (5, 7, 1024), (8, 2561, 3072), (2, 600, 4096), (8, 300, 6148), (6, 131, 12292), (1, 70, 1500),
+                                   # 9 to 64 rows and K from 1,024: the same kernel, eight rows a launch; more rows: tiles
+                                   (9, 300, 2560), (40, 301, 2560), (64, 129, 1024), (17, 2561, 4096), (33, 70, 6148), (65, 70, 1024)])
 def test_gemm_f32(ops, m, n, k):
     g = torch.Generator().manual_seed(4)
     a, b, bias = rand(g, m, k), rand(g, n, k), rand(g, n)
@@ -140,13 +142,14 @@ def test_gemm_f32(ops, m, n, k):
     torch.testing.assert_close(got, want, atol=1e-4 * math.sqrt(k), rtol=1e-5)
     # a row's result does not depend on the rows beside it
     alone = ops.gemm_nt_f32(a[:1].to(DEV).contiguous(), b.to(DEV), bias.to(DEV)).cpu()
-    if (m <= 8 or k < 1024 or k % 4) and (m <= 16 or k % 4):
+    def variant(rows):       # A in registers (eight rows a launch), the weight streamed past up to 16 rows, or tiles
+        return "resident" if rows <= 64 and k >= 1024 and k % 4 == 0 else "rows" if rows <= 16 and k % 4 == 0 else "tiles"
+    if variant(m) == variant(1):
         assert torch.equal(alone[0], got[0])        # the same variant, whose order of sums depends on K alone
-    else:                                           # few rows stream the weight, many rows take tiles: another order of the same sums
+    else:                                           # another order of the same sums
         torch.testing.assert_close(alone[0], got[0], atol=1e-5 * math.sqrt(k), rtol=1e-5)
-    resident = lambda rows: rows <= 8 and k >= 1024 and k % 4 == 0      # the variant that keeps A in registers
-    for rows in (2, 5, 9, 16):                      # the variants for few rows give the same bits within their kind
-        if rows < m <= 16 and resident(rows) == resident(m):
+    for rows in (2, 5, 9, 16, 40):                  # the variants for few rows give the same bits within their kind
+        if rows < m and variant(m) != "tiles" and variant(rows) == variant(m):
             part = ops.gemm_nt_f32(a[:rows].to(DEV).contiguous(), b.to(DEV), bias.to(DEV)).cpu()
             assert torch.equal(part, got[:rows])
 
