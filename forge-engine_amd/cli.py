@@ -118,11 +118,9 @@ def run_generate(args) -> int:
         engine = engine_from_random(load_model_config(args.random_config), args.weights_seed,
                                     engine_config=engine_config, scheduler_config=scheduler_config,
                                     dtype=args.dtype, device=args.device)
-    ids = [engine.submit(prompt) for prompt in prompts]
-    engine.run_until_idle()
+    # more prompts than --max-requests or than the pages hold at once wait their turn
     failed = False
-    for index, request_id in enumerate(ids):
-        view = engine.request(request_id)
+    for index, view in enumerate(engine.run(prompts)):
         record = {"prompt": index, "status": view.status.value, "finish_reason": view.finish_reason,
                   "token_ids": list(view.output_token_ids)}
         if view.text:

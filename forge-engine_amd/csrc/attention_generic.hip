@@ -412,7 +412,11 @@ __global__ __launch_bounds__(256) void paged_attention_rows_kernel(
   constexpr int KPP = 256 / LPK;    // keys the block covers with one fetch a thread: a thread's keys lie KPP apart
   constexpr int LPD = TK / 4;       // lanes that share an output dim
   constexpr int DPP = 256 / LPD;    // dims the block covers with one fetch a thread: a thread's dims lie DPP apart
-  __shared__ __align__(16) float Ps[GMAX][TK];   // a tile's scores, then its probabilities
+  // A tile's scores, then its probabilities.  Two buffers that the tiles take in turn: a wave that has
+  // used a tile's probabilities goes on to write the next tile's scores before the block's next barrier,
+  // while a slower wave may still be reading the probabilities; in the other buffer it disturbs nobody,
+  // and that buffer's last readers passed two barriers ago.
+  __shared__ __align__(16) float Ps2[2][GMAX][TK];
   __shared__ float ml_s[GMAX][2];                // running maximum and sum of a row
   __shared__ float corr_s[GMAX];                 // what the tile scales a row's earlier sums by
 
@@ -490,8 +494,10 @@ __global__ __launch_bounds__(256) void paged_attention_rows_kernel(
     fetch_values(my_first * TK, pv);
     if (my_first * TK + TK < kt_end) lookup(my_first * TK + TK, pkn, pvn);
   }
-  for (int kt = my_first * TK; kt < kt_end; kt += TK) {
+  int buffer = 0;
+  for (int kt = my_first * TK; kt < kt_end; kt += TK, buffer ^= 1) {
     const bool more = kt + TK < kt_end;
+    float (*Ps)[TK] = Ps2[buffer];
     float s[GMAX][4];
 #pragma unroll
     for (int g = 0; g < GMAX; ++g)

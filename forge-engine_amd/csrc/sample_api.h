@@ -29,7 +29,9 @@ int fe_argmax_rows(const float* logits, long long row_stride, int rows, int voca
 // allocator.  The partial maxima live in an array inside the library's device image
 // (FE_ARGMAX_STATIC_MAX_ROWS * 32 * 3 words = 384 KiB on each GPU the library runs on, until the
 // process ends); its address on a device is looked up once, at the first call with that device
-// current.  The call allocates nothing and frees nothing.  rows > FE_ARGMAX_STATIC_MAX_ROWS is
+// current.  That first call on a device is set-up: the lookup may make the runtime load the
+// library's device image, so it must be made outside any graph capture (one row suffices); every
+// later call on that device may be captured.  The call allocates nothing and frees nothing.  rows > FE_ARGMAX_STATIC_MAX_ROWS is
 // refused with FE_BAD_ARGUMENT.  Nothing in the array has to start at zero: every word that the
 // merge reads is written by the same call first.  All calls on one GPU share the array, so two
 // calls that overlap on one GPU (different streams, or threads) race; calls on one stream do not.

@@ -339,17 +339,24 @@ class ConcurrentGenerationEngine:
             feed = None
         try:
             logits = self._runner.step(entries, device_tokens=feed) if feed is not None else self._runner.step(entries)
+        except CacheCapacityError:
+            return None                             # nothing was changed: pages are reserved all or none
+        except Exception as error:
+            return self._land() + self._fail_batch(requests, error)
+        # from here on the step has run: the cache holds one token more for every request
+        for request in requests:
+            request.fed += 1
+        try:
             # a request with a token in flight has drawn one more than it has consumed
             launched = self._sampler.sample_on_device(
                 logits, [r.params for r in requests], [r.seed for r in requests],
                 [r.sampled_tokens + (1 if r.in_flight else 0) for r in requests])
-        except Exception:
-            return None                             # nothing was changed: pages are reserved all or none
+        except Exception as error:
+            return self._land() + self._fail_batch(requests, error)
         self._last_batch = tuple(r.request_id for r in requests)
         self._last_tokens = tuple(1 for _ in requests)
         events = self._land()                       # the step before, read while this one runs
         for request in requests:
-            request.fed += 1
             request.in_flight = True
         self._flight = (requests, launched)
         self.overlapped_steps += 1
@@ -357,6 +364,7 @@ class ConcurrentGenerationEngine:
 
     def step(self) -> list[StreamEvent]:
         """One model step over a fresh batch; returns what it produced."""
+        order_before = deque(self._order)
         selected = self._select_batch()
         self._iteration += 1
         events: list[StreamEvent] = []
@@ -365,8 +373,11 @@ class ConcurrentGenerationEngine:
             if produced is not None:
                 return produced
         if self._flight is not None:
-            # another kind of step follows: first learn what the step in flight sampled, then choose again
+            # another kind of step follows: first learn what the step in flight sampled, then choose again,
+            # from the queue as it stood (a selection that did not run must not cost anyone a turn)
             events.extend(self._land())
+            self._order = order_before
+            self._drop_terminal()
             selected = self._select_batch()
         while True:
             self._last_batch = tuple(r.request_id for r, _ in selected)
@@ -417,14 +428,18 @@ class ConcurrentGenerationEngine:
         events: list[StreamEvent] = []
         while not self.idle:
             produced = self.step()
-            if not self._last_batch and not produced:
-                raise RuntimeError("scheduler made no progress")
             events.extend(produced)
+            # a step that only read the tokens in flight (the last request ended on one of them) ran
+            # no batch and may emit nothing: that is the end of the work, not a lack of progress
+            if not self._last_batch and not produced and not self.idle:
+                raise RuntimeError("scheduler made no progress")
         return events
 
-    def generate(self, prompts: Sequence, sampling_params: SamplingParams | None = None) -> list[list[int]]:
-        """Run the prompts to completion (admitting them as room allows) and
-        return each one's generated token ids."""
+    def run(self, prompts: Sequence, sampling_params: SamplingParams | None = None) -> list[RequestView]:
+        """Run the prompts to completion, admitting each as the request limit and the pages allow
+        (a prompt that can never be admitted raises ``OverloadedError`` once nothing else is
+        running), and return every request's last view, in the order of the prompts.  The requests
+        are forgotten."""
         pending = deque(enumerate(prompts))
         ids: dict[int, str] = {}
         while pending or not self.idle:
@@ -440,14 +455,19 @@ class ConcurrentGenerationEngine:
             produced = self.step()
             if not self._last_batch and not produced and not self.idle:
                 raise RuntimeError("scheduler made no progress")
-        results = []
+        views = [self.request(ids[index]) for index in range(len(prompts))]
         for index in range(len(prompts)):
-            view = self.request(ids[index])
+            self.forget(ids[index])
+        return views
+
+    def generate(self, prompts: Sequence, sampling_params: SamplingParams | None = None) -> list[list[int]]:
+        """Run the prompts to completion (admitting them as room allows) and
+        return each one's generated token ids."""
+        views = self.run(prompts, sampling_params)
+        for view in views:
             if view.status is RequestStatus.FAILED:
                 raise RuntimeError(f"request {view.request_id} failed: {view.error}")
-            results.append(list(view.output_token_ids))
-            self.forget(ids[index])
-        return results
+        return [list(view.output_token_ids) for view in views]
 
     # -------------------------------------------------------------- results
     def _consume(self, request: _Request, token: int) -> list[StreamEvent]:
@@ -495,6 +515,14 @@ class ConcurrentGenerationEngine:
             request.error = f"{type(error).__name__}: {error}"
             self._cleanup(request)
             events.append(StreamEvent(request.request_id, "", request.status))
+        return events
+
+    def _fail_batch(self, requests: list[_Request], error: Exception) -> list[StreamEvent]:
+        """A model call or a sampling call failed: every live request of its batch fails."""
+        for request in requests:
+            request.in_flight = False
+        events = self._fail([r for r in requests if not r.status.terminal], error)
+        self._drop_terminal()
         return events
 
     def _cleanup(self, request: _Request) -> None:

@@ -13,7 +13,12 @@ entry's tokens whose logits are written; ``end`` lists requests that are
 finished after the step (their pages and state slot go back to the pools).
 For a step with wanted places the file ``<out>/<step>.f32`` gets the logits as
 little-endian float32 [wanted, vocab], in the order of the entries and of each
-``want``.  After every step the line ``done <step>`` is printed and flushed.
+``want``.  Beside it ``<out>/<step>.json`` says what the step looked like from the
+cache's side, for debugging: ``rows`` names the (request, absolute position) of every
+logits row of ``<step>.f32``, and ``tables`` gives, for every request of the step, its
+length after the step and the pages of its block table in every cache group (-1: a page
+that a window has passed and given back).  After every step the line ``done <step>`` is
+printed and flushed.
 """
 
 from __future__ import annotations
@@ -39,7 +44,9 @@ def build_parser() -> argparse.ArgumentParser:
     return parser
 
 
-def run(args, stdin=None, stdout=None) -> int:
+def run(args, stdin=None, stdout=None, device=None) -> int:
+    """``device``: where the model runs; the default is ``args.device``, which must be a GPU (a
+    caller that has put plain implementations in place of the kernels passes a CPU device here)."""
     import torch
 
     from .engine import ModelRunner, StepEntry, load_model
@@ -51,7 +58,7 @@ def run(args, stdin=None, stdout=None) -> int:
         raise ValueError("--block-size must divide 64")
     if args.max_tokens < 1:
         raise ValueError("--max-tokens must be positive")
-    device = require_gpu(args.device) if not getattr(args, "allow_cpu", False) else torch.device(args.device)
+    device = require_gpu(args.device) if device is None else torch.device(device)
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
     _, model = load_model(args.model, dtype=args.dtype, device=device)
@@ -72,7 +79,16 @@ def run(args, stdin=None, stdout=None) -> int:
             entries.append(StepEntry(request_id, [int(t) for t in item["tokens"]],
                                      [int(w) for w in item.get("want", [])]))
         if entries:
+            before = {entry.request_id: runner.length(entry.request_id) for entry in entries}
             logits = runner.step(entries)
+            records = {entry.request_id: runner.cache.request(entry.request_id) for entry in entries}
+            layout = {
+                "step": step,
+                "rows": [[entry.request_id, before[entry.request_id] + place] for entry in entries for place in entry.want],
+                "tables": {name: {"length": record.length, "pages": [list(map(int, table)) for table in record.tables]}
+                           for name, record in records.items()},
+            }
+            (out_dir / f"{step}.json").write_text(json.dumps(layout))
             if logits.shape[0]:
                 data = logits.to(torch.float32).cpu().contiguous().numpy().astype("<f4", copy=False)
                 data.tofile(str(out_dir / f"{step}.f32"))

@@ -8,8 +8,7 @@ generator, so the n-th token of a request depends only on (seed, n) and the
 logits, not on what else was in the batch or on how often the request was
 preempted.  NaN, +inf or a row without a finite entry raise, as in
 sampling.py:62-70; the check runs inside the kernels and comes back with the
-tokens in one transfer.  ``filter_logits`` is the same filter on whole tensors
-(what the kernel keeps, for callers that want the filtered logits themselves).
+tokens in one transfer.
 """
 
 from __future__ import annotations
@@ -19,32 +18,6 @@ from torch import Tensor
 
 from ..kernels import ops
 from .params import SamplingParams
-
-NEG_INF = float("-inf")
-
-
-def filter_logits(logits: Tensor, params: SamplingParams) -> Tensor:
-    """Rows after temperature, top-k, top-p and min-p; removed entries are -inf."""
-    if params.greedy:
-        raise ValueError("greedy sampling does not filter logits")
-    x = logits.float()
-    x = (x - x.amax(dim=-1, keepdim=True)) / params.temperature
-    if params.top_k is not None and params.top_k < x.shape[-1]:
-        values, indices = torch.topk(x, params.top_k, dim=-1)
-        x = torch.full_like(x, NEG_INF).scatter_(-1, indices, values)
-    if params.top_p < 1.0:
-        ordered, order = torch.sort(x, dim=-1, descending=True)
-        mass = torch.softmax(ordered, dim=-1, dtype=torch.float32).cumsum(dim=-1)
-        # a token goes if the mass of the tokens before it already exceeds top_p;
-        # the first token always stays
-        before = torch.zeros_like(mass)
-        before[..., 1:] = mass[..., :-1]
-        ordered = ordered.masked_fill(before > params.top_p, NEG_INF)
-        x = torch.full_like(x, NEG_INF).scatter_(-1, order, ordered)
-    if params.min_p > 0.0:
-        probs = torch.softmax(x, dim=-1, dtype=torch.float32)
-        x = x.masked_fill(probs < probs.amax(dim=-1, keepdim=True) * params.min_p, NEG_INF)
-    return x
 
 
 def _raise_on_status(status: list[int]) -> None:

@@ -120,18 +120,18 @@ def trace_mixed(requests, seed: int, max_live: int = 4, prompt_fraction: float =
 
 
 def run_trace(model_dir, dtype: str, trace: TraceBuilder, out_dir, *, block_size: int,
-              max_tokens: int | None = None, device: str = "cuda:0", allow_cpu: bool = False):
+              max_tokens: int | None = None, device: str = "cuda:0", on_cpu: bool = False):
     """Replay in-process through the replay module; returns
-    {(request, position): logits row}."""
+    {(request, position): logits row}.  ``on_cpu``: the caller has patched the kernels' plain
+    references in and the model runs on the CPU."""
     from forge_engine_amd import replay
 
     out_dir = Path(out_dir)
     stdin = io.StringIO("".join(json.dumps(step) + "\n" for step in trace.steps))
     stdout = io.StringIO()
     args = Namespace(model=str(model_dir), dtype=dtype, out=str(out_dir), block_size=block_size,
-                     max_tokens=trace.peak_tokens if max_tokens is None else max_tokens, device=device,
-                     allow_cpu=allow_cpu)
-    assert replay.run(args, stdin=stdin, stdout=stdout) == 0
+                     max_tokens=trace.peak_tokens if max_tokens is None else max_tokens, device=device)
+    assert replay.run(args, stdin=stdin, stdout=stdout, device="cpu" if on_cpu else None) == 0
     assert stdout.getvalue().split() == [w for s in trace.steps for w in ("done", str(s["step"]))]
     return collect(trace, out_dir, json.loads((Path(model_dir) / "config.json").read_text())["vocab_size"])
 
@@ -142,6 +142,8 @@ def collect(trace: TraceBuilder, out_dir, vocab: int):
         if not rows:
             continue
         data = np.fromfile(str(Path(out_dir) / f"{index}.f32"), dtype="<f4").reshape(len(rows), vocab)
+        layout = json.loads((Path(out_dir) / f"{index}.json").read_text())
+        assert [tuple(row) for row in layout["rows"]] == rows, "the step's own account of its rows differs"
         for row, key in zip(data, rows):
             got[key] = torch.from_numpy(row.copy())
     return got

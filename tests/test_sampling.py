@@ -1,4 +1,4 @@
-"""Sampling parameters and the logits filters (CPU).  The draw kernels are
+"""Sampling parameters and the sampler's routing (CPU); the filters' thresholds against the plain filters.  The draw kernels are
 covered by the GPU tests."""
 
 from __future__ import annotations
@@ -10,7 +10,7 @@ import kernel_refs
 import plain_qwen3 as plain
 from forge_engine_amd.config import EngineConfig
 from forge_engine_amd.sampling import SamplingParams
-from forge_engine_amd.sampling.sampler import Sampler, filter_logits
+from forge_engine_amd.sampling.sampler import Sampler
 
 
 @pytest.mark.parametrize("kwargs", [
@@ -34,27 +34,6 @@ def test_defaults_follow_the_reference():
 
 def kept(x):
     return torch.isfinite(x).nonzero()[:, 1].tolist()
-
-
-def test_filter_vectors_of_the_reference():
-    # tests/test_sampling.py:47-81 of the reference
-    assert kept(filter_logits(torch.tensor([[0.0, 3.0, 2.0, 1.0]]), SamplingParams(temperature=1.0, top_k=2))) == [1, 2]
-    assert kept(filter_logits(torch.tensor([[5.0, 4.0, 0.0]]), SamplingParams(temperature=1.0, top_p=0.7))) == [0]
-    assert kept(filter_logits(torch.tensor([[0.0, -1.0, -3.0]]), SamplingParams(temperature=1.0, min_p=0.2))) == [0, 1]
-    with pytest.raises(ValueError, match="greedy"):
-        filter_logits(torch.zeros(1, 3), SamplingParams())
-
-
-@pytest.mark.parametrize("seed", range(5))
-def test_filters_equal_the_plain_implementation(seed):
-    g = torch.Generator().manual_seed(seed)
-    logits = torch.randn(4, 50, generator=g) * 3
-    for p in (SamplingParams(temperature=0.7, top_k=5), SamplingParams(temperature=1.3, top_p=0.6),
-              SamplingParams(temperature=0.9, min_p=0.1), SamplingParams(temperature=0.5, top_k=20, top_p=0.8, min_p=0.05)):
-        got = filter_logits(logits, p)
-        want = plain.filter_logits(logits, p.temperature, p.top_k, p.top_p, p.min_p)
-        assert torch.equal(torch.isfinite(got), torch.isfinite(want))
-        torch.testing.assert_close(got, want)
 
 
 @pytest.mark.parametrize("seed", range(5))

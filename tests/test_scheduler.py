@@ -12,9 +12,10 @@ import kernel_refs
 import plain_qwen3 as plain
 from conftest import TINY
 from forge_engine_amd.config import SchedulerConfig, load_model_config
-from forge_engine_amd.engine import (ConcurrentGenerationEngine, GenerationEngine, IncrementalDetokenizer,
-                                     OverloadedError, RequestStatus, build_engine, load_model)
+from forge_engine_amd.engine import (ConcurrentGenerationEngine, GenerationEngine, IncrementalDetokenizer, ModelRunner,
+                                     OverloadedError, RequestStatus, StepEntry, build_engine, load_model)
 from forge_engine_amd.sampling import SamplingParams
+from forge_engine_amd.sampling.sampler import Sampler
 from forge_engine_amd.weights import write_random_model
 from safetensors.torch import load_file
 
@@ -267,6 +268,110 @@ def test_single_request_engine_streams_and_cleans_up(make, folder):
     next(stream)
     stream.close()                       # the consumer stops early: pages go back
     assert engine.engine.cache_pool.allocated_pages == 0 and engine.engine.idle
+
+
+class DeviceFeedRunner:
+    """The CPU runner with the two things that overlapped decoding asks of a runner: it says that
+    it can feed a step of single tokens from a device tensor, and does so (here by reading it)."""
+
+    def __init__(self, runner) -> None:
+        self._runner = runner
+        self.fail_next_step = None
+
+    def __getattr__(self, name):
+        return getattr(self._runner, name)
+
+    def feeds_from_device(self, entries) -> bool:
+        return all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+
+    def step(self, entries, device_tokens=None):
+        if self.fail_next_step is not None:
+            error, self.fail_next_step = self.fail_next_step, None
+            raise error
+        if device_tokens is not None:
+            entries = [StepEntry(e.request_id, [int(device_tokens[i])], e.want) for i, e in enumerate(entries)]
+        return self._runner.step(entries)
+
+
+@pytest.fixture()
+def make_overlapped(folder, monkeypatch):
+    kernel_refs.install(monkeypatch)
+
+    def build(**limits) -> ConcurrentGenerationEngine:
+        _, model = load_model(folder, dtype="float32", device="cpu")
+        eos = limits.pop("eos", ())
+        config = SchedulerConfig(**{"block_size": 2, "block_capacity": 64, **limits})
+        runner = DeviceFeedRunner(ModelRunner(model, block_size=config.block_size, block_capacity=config.block_capacity,
+                                              num_state_slots=config.max_requests))
+        return ConcurrentGenerationEngine(runner, Sampler(model.ctx.device), SamplingParams(), config, eos_token_ids=eos)
+    return build
+
+
+def test_overlapped_decoding_ends_cleanly_when_the_last_request_stops_on_its_end_token(make_overlapped, folder):
+    # the request's end token is read a step late, while the request rides in a step already launched:
+    # the step after that only reads that step's tokens, runs no batch and emits nothing, and is the end
+    sampled = params(12, temperature=1.0, seed=5)
+    probe = make_overlapped(overlap_decode=False)
+    tokens = probe.generate([[5, 17, 3]], sampled)[0]
+    at = next(i for i in range(2, 12) if tokens[i] not in tokens[:i])   # first token not seen before
+    engine = make_overlapped(eos=(tokens[at],))
+    engine.submit([5, 17, 3], request_id="e", sampling_params=sampled)
+    events = engine.run_until_idle()
+    view = engine.request("e")
+    assert engine.overlapped_steps >= at - 1 and engine.idle
+    assert view.status is RequestStatus.FINISHED and view.finish_reason == "stop"
+    assert list(view.output_token_ids) == tokens[:at] and view.sampled_tokens == at + 1
+    assert [e.token_ids for e in events] == [(t,) for t in tokens[:at]] + [()]
+    assert engine.cache_pool.allocated_pages == 0 and engine.snapshot().reserved_blocks == 0
+    assert engine.generate([[5, 17, 3]], sampled) == [tokens[:at]]     # and through generate
+
+
+def test_overlapped_decoding_serves_requests_in_the_same_order(make_overlapped, make, folder):
+    # more live requests than a step takes: a selection that could not be overlapped is made again
+    # from the queue as it stood, so nobody loses a turn and the batches are those of the plain scheduler
+    prompts = {name: [3 + i, 40 + i, 9] for i, name in enumerate("abcde")}
+    batches = {}
+    for overlap, build in ((True, make_overlapped), (False, make)):
+        engine = build(max_batch_size=2, overlap_decode=overlap)
+        for name, prompt in prompts.items():
+            engine.submit(prompt, request_id=name, sampling_params=params(4))
+        seen = []
+        while not engine.idle:
+            engine.step()
+            seen.append(engine.snapshot().last_batch)
+        batches[overlap] = [b for b in seen if b]
+        for name, prompt in prompts.items():
+            assert list(engine.request(name).output_token_ids) == plain_greedy(folder, prompt, 4)
+    assert batches[True] == batches[False]
+
+
+def test_a_failure_after_an_overlapped_step_has_run_fails_the_batch(make_overlapped, monkeypatch):
+    # the step ran and moved the cache on; if sampling then fails, feeding the same tokens again would
+    # put them one position late: the batch fails instead, and everything is given back
+    engine = make_overlapped()
+    engine.submit([1, 2, 3], request_id="a", sampling_params=params(8))
+    engine.submit([4, 5], request_id="b", sampling_params=params(8))
+    engine.step()
+    engine.step()
+    assert engine.overlapped_steps == 1
+
+    def broken(*args, **kwargs):
+        raise RuntimeError("sampling kernel failed")
+    monkeypatch.setattr(engine._sampler, "sample_on_device", broken)
+    events = engine.step()
+    assert all(engine.request(n).status is RequestStatus.FAILED for n in "ab")
+    assert engine.request("a").error == "RuntimeError: sampling kernel failed"
+    assert [e.status for e in events if e.status is RequestStatus.FAILED] == [RequestStatus.FAILED] * 2
+    assert engine.cache_pool.allocated_pages == 0 and engine.snapshot().reserved_blocks == 0 and engine.idle
+    # a model call that fails is not retried on the plain path either
+    engine = make_overlapped()
+    engine.submit([1, 2, 3], request_id="a", sampling_params=params(8))
+    engine.step()
+    engine.step()
+    engine._runner.fail_next_step = RuntimeError("device lost")
+    engine.step()
+    assert engine.request("a").error == "RuntimeError: device lost" and engine.idle
+    assert engine._runner.steps_run == 2 and engine.cache_pool.allocated_pages == 0
 
 
 class WordTokenizer:
