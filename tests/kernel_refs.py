@@ -154,6 +154,36 @@ def paged_attention(q, key_pages, value_pages, out, cu_q, ctx_len, block_table, 
     return out
 
 
+def paged_attention_by_matrices(q, key_pages, value_pages, cu_q, ctx_len, block_table, *, q_heads, kv_heads,
+                                head_dim, scale, window=None):
+    """``paged_attention`` for long sequences: a whole (sequence, head) at a time as two float32
+    matrix products with the causal (and window) mask between them, instead of a token at a time.
+    The same formula; ``tests/test_kernel_policies.py`` holds the two against each other.  Returns float32."""
+    block_size = key_pages.shape[2]
+    groups = q_heads // kv_heads
+    result = torch.zeros((q.shape[0], q_heads * head_dim), dtype=torch.float32)
+    for s in range(ctx_len.numel()):
+        q0, q1 = int(cu_q[s]), int(cu_q[s + 1])
+        q_len, ctx = q1 - q0, int(ctx_len[s])
+        if q_len == 0:
+            continue
+        before = ctx - q_len
+        keys = gather_pages(key_pages, block_table[s], ctx, block_size)
+        values = gather_pages(value_pages.transpose(2, 3), block_table[s], ctx, block_size)
+        position = before + torch.arange(q_len).view(-1, 1)
+        key_index = torch.arange(ctx).view(1, -1)
+        seen = key_index <= position
+        if window:
+            seen &= key_index > position - window
+        keys, values = torch.nan_to_num(keys), torch.nan_to_num(values)   # pages given back lie outside every window
+        for h in range(q_heads):
+            queries = q[q0:q1, h * head_dim:(h + 1) * head_dim].float()
+            scores = (queries @ keys[h // groups].T) * scale
+            probs = torch.softmax(scores.masked_fill(~seen, float("-inf")), dim=-1)
+            result[q0:q1, h * head_dim:(h + 1) * head_dim] = probs @ values[h // groups]
+    return result
+
+
 def argmax_rows(logits, tokens, status):
     for r in range(logits.shape[0]):
         row = logits[r]
@@ -256,6 +286,11 @@ def decode_prepare_supported(*args, **kwargs):
 
 def linear_in_parts(x, weight):
     return None
+
+
+# Key splits of the bfloat16 decode attention that the GPU tests launch (every count the kernel takes:
+# 1 to 4, 5 to 8 and 9 to 16 merge with all loads in one round, 17 to 64 in a loop)
+DECODE_SPLITS_TESTED = tuple(range(1, 65))
 
 
 NAMES = ("decode_prepare_supported", "linear_in_parts", "embed_rows", "add_rmsnorm", "add_rows", "swiglu", "gemm_nt_f32", "linear", "linear_update", "linear_swiglu", "gemm_skinny",

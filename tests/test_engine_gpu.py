@@ -160,6 +160,39 @@ def test_command_line_generates(folders, capsys):
     check_choice(folder_weights(folders["A"]), TINY["A"], prompt, records[0]["token_ids"], "float32")
 
 
+def test_a_lone_request_that_ends_on_its_end_token_while_decoding_overlapped(folders, tmp_path, capsys):
+    """The last running request samples its end-of-sequence token during overlapped decoding: it
+    still rides in the step already launched, the step after that only reads that step's tokens,
+    and the run ends there, through ``run_until_idle`` and through the command line (whose model
+    folder names the end token in config.json; more prompts than ``--max-requests`` wait their turn)."""
+    from forge_engine_amd.cli import main
+    name = "B"
+    prompt = ru.make_requests(TINY[name], 87, (12, 30))["r1"]
+    scheduler = SchedulerConfig(block_size=8, block_capacity=64)
+    probe = engine_from_folder(folders[name], scheduler_config=scheduler, dtype="float32", eos_token_ids=[])
+    tokens = probe.generate([prompt], SamplingParams(max_new_tokens=24))[0]
+    at = next(j for j in range(3, len(tokens)) if tokens[j] not in tokens[:j])
+    engine = engine_from_folder(folders[name], scheduler_config=scheduler, dtype="float32", eos_token_ids=[tokens[at]])
+    request_id = engine.submit(prompt, sampling_params=SamplingParams(max_new_tokens=24))
+    engine.run_until_idle()
+    view = engine.request(request_id)
+    assert engine.overlapped_steps >= at - 1 and engine.idle and engine.cache_pool.allocated_pages == 0
+    assert view.finish_reason == "stop" and list(view.output_token_ids) == tokens[:at]
+    # the command line: a folder whose config.json names that end token, three prompts through two request places
+    folder = tmp_path / "with_eos"
+    folder.mkdir()
+    (folder / "model.safetensors").symlink_to(folders[name] / "model.safetensors")
+    (folder / "config.json").write_text(json.dumps({**TINY[name], "eos_token_id": tokens[at]}))
+    ids = ",".join(map(str, prompt))
+    code = main(["generate", "--model", str(folder), "--dtype", "float32", "--prompt-ids", ids, "--prompt-ids", "7,7,9",
+                 "--prompt-ids", ids, "--max-new-tokens", "24", "--block-size", "8", "--max-requests", "2"])
+    assert code == 0
+    records = [json.loads(line) for line in capsys.readouterr().out.strip().splitlines()]
+    assert [r["prompt"] for r in records] == [0, 1, 2]
+    assert records[0]["finish_reason"] == "stop" and records[0]["token_ids"] == tokens[:at]
+    assert records[2] == {**records[0], "prompt": 2}
+
+
 def test_temperature_sampling_is_seeded_and_batch_independent(folders):
     scheduler = SchedulerConfig(block_size=8, block_capacity=64)
     engine = engine_from_folder(folders["B"], scheduler_config=scheduler, dtype="float32")

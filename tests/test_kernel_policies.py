@@ -96,3 +96,51 @@ def test_workspaces_are_per_owner():
             assert ops._split_counters(cpu, 8) is not mine
         assert ops._split_counters(cpu, 8) is mine
     assert ops._split_counters(cpu, 8) is not mine                # outside: the default of (device, stream)
+
+
+def test_every_count_of_key_splits_that_a_decode_step_can_take_is_one_that_the_gpu_tests_launch():
+    import kernel_refs
+    seen = set()
+    for batch in list(range(1, 66)) + [96, 128, 255, 256]:
+        for kv_heads in (1, 2, 3, 4, 5, 8, 16, 40, 64):
+            for ctx in [1, 31, 32, 33, 127, 128, 129] + [64 * n for n in range(1, 1025)]:
+                seen.add(ops.decode_splits(batch, kv_heads, ctx))
+    assert seen <= set(kernel_refs.DECODE_SPLITS_TESTED)
+    assert {1, 16, 17, 64} <= seen and max(seen) == 64 and min(seen) == 1
+    # the table-width bound of a captured decode step (a multiple of 64 pages of 16 tokens) at batch 1 and 2 past
+    # 1,024 tokens, and at batch 1 past 4,096: the merges of 9 to 16 splits and of 17 to 64
+    assert ops.decode_splits(1, 8, 2048) == 16 and ops.decode_splits(2, 8, 2048) == 16
+    assert ops.decode_splits(1, 8, 8192) == 32 and ops.decode_splits(1, 1, 16384) == 64
+
+
+@pytest.mark.parametrize("window", [None, 1, 9, 40])
+def test_the_two_references_of_paged_attention_agree(window):
+    """The reference by whole matrices (used where sequences are thousands of tokens long) against
+    the one that goes token by token: mixed batch, shuffled pages, a window whose passed pages were
+    given back."""
+    import kernel_refs
+    import torch
+    g = torch.Generator().manual_seed(5)
+    q_heads, kv_heads, head_dim, block_size = 6, 2, 8, 4
+    seqs = [(0, 7), (13, 1), (5, 9), (30, 0), (0, 1)]
+    total = sum(n for _, n in seqs)
+    pages = [-(-(b + n) // block_size) for b, n in seqs]
+    order = torch.randperm(sum(pages) + 2, generator=g).tolist()
+    table = torch.full((len(seqs), max(pages)), -1, dtype=torch.int32)
+    at = 0
+    for s, count in enumerate(pages):
+        table[s, :count] = torch.tensor(order[at:at + count], dtype=torch.int32)
+        at += count
+    if window:   # pages that every query's window has passed
+        for s, (before, n) in enumerate(seqs):
+            table[s, :max(0, before - window + 1) // block_size] = -1
+    kp = torch.randn(sum(pages) + 2, kv_heads, block_size, head_dim, generator=g)
+    vp = torch.randn(sum(pages) + 2, kv_heads, head_dim, block_size, generator=g)
+    q = torch.randn(total, q_heads * head_dim + 5, generator=g)
+    cu = torch.tensor([0] + torch.tensor([n for _, n in seqs]).cumsum(0).tolist(), dtype=torch.int32)
+    ctx = torch.tensor([b + n for b, n in seqs], dtype=torch.int32)
+    kw = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=0.3, window=window)
+    slow = kernel_refs.paged_attention(q, kp, vp, torch.empty(total, q_heads * head_dim), cu, ctx, table,
+                                       num_seqs=len(seqs), max_q_len=9, **kw)
+    fast = kernel_refs.paged_attention_by_matrices(q, kp, vp, cu, ctx, table, **kw)
+    torch.testing.assert_close(fast, slow, atol=1e-5, rtol=1e-5)

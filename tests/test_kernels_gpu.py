@@ -929,6 +929,86 @@ def test_decode_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size, s
             torch.testing.assert_close(again, expect, atol=2e-2, rtol=2e-2)
 
 
+LONG_CONTEXTS = [2046, 4095, 19999, 33, 0, 700, 8191]     # tokens each sequence holds before its one new token
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [(4, 2, 128, 16), (5, 1, 64, 32)])
+def test_decode_attention_kernel_every_count_of_key_splits(ops, q_heads, kv_heads, head_dim, block_size):
+    """Every count of key splits that the kernel takes (1 to 64: the merges with all loads in one
+    round for up to 4, 8 and 16 splits, and the loop beyond), over contexts from one key to 20,000:
+    splits without any key, splits of one 32-key block, a context one short of a block's and a
+    page's edge.  Each count is launched twice on the same arrival counters, with other queries."""
+    g = torch.Generator().manual_seed(61)
+    seqs = [(before, 1) for before in LONG_CONTEXTS]
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
+                                                extra_width=2 * kv_heads * head_dim)
+    kw = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=head_dim ** -0.5)
+    queries = [q, (q.float() * -1.5).to(torch.bfloat16)]
+    wants = [refs.paged_attention_by_matrices(x, kp, vp, cu, ctx, table, **kw) for x in queries]
+    dev = [t.to(DEV) for t in (kp, vp, cu, ctx, table)]
+    queries_dev = [x.to(DEV) for x in queries]
+    assert set(refs.DECODE_SPLITS_TESTED) == set(range(1, 65))
+    for splits in refs.DECODE_SPLITS_TESTED:
+        for x, want in zip(queries_dev, wants):
+            out = torch.full((len(seqs), q_heads * head_dim), float("nan"), dtype=torch.bfloat16, device=DEV)
+            ops.paged_attention(x, dev[0], dev[1], out, dev[2], dev[3], dev[4], num_seqs=len(seqs), max_q_len=1,
+                                num_decode=len(seqs), max_ctx=20000, splits=splits, **kw)
+            torch.testing.assert_close(out.cpu().float(), want, atol=2e-2, rtol=2e-2, msg=lambda m: f"{splits} splits: {m}")
+
+
+@pytest.mark.parametrize("splits", [9, 12, 16, 17, 32, 64])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [(4, 2, 128, 16), (8, 1, 64, 32)])
+def test_decode_attention_that_prepares_with_many_key_splits(ops, q_heads, kv_heads, head_dim, block_size, splits):
+    """The kernel that makes its own queries and keys with 9 to 64 key splits over long contexts,
+    against the plain reference of the two steps; twice on the same pages and counters."""
+    g = torch.Generator().manual_seed(62)
+    qkv, kp, vp, cu, ctx, table, qw, kw, inv_freq, positions, token_seq = _prepare_case(
+        g, q_heads, kv_heads, head_dim, block_size, LONG_CONTEXTS)
+    n = len(LONG_CONTEXTS)
+    sizes = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim)
+    qkv_ref, kp_ref, vp_ref = qkv.clone(), kp.clone(), vp.clone()
+    refs.qk_norm_rope_write(qkv_ref, qw, kw, inv_freq, positions, token_seq, table, kp_ref, vp_ref,
+                            rotary_dim=head_dim, eps=1e-6, **sizes)
+    want = refs.paged_attention_by_matrices(qkv_ref, kp_ref, vp_ref, cu, ctx, table, scale=head_dim ** -0.5, **sizes)
+    kp_dev, vp_dev = kp.to(DEV), vp.to(DEV)
+    for _ in range(2):
+        out = torch.full((n, q_heads * head_dim), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.decode_attention_prepare(qkv.to(DEV), qw.to(DEV), kw.to(DEV), inv_freq.to(DEV), kp_dev, vp_dev, out, cu.to(DEV),
+                                     ctx.to(DEV), table.to(DEV), eps=1e-6, scale=head_dim ** -0.5, max_ctx=20000,
+                                     splits=splits, **sizes)
+        torch.testing.assert_close(out.cpu().float(), want, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(kp_dev.cpu().float(), kp_ref.float(), **tol(torch.bfloat16))
+    assert torch.equal(vp_dev.cpu(), vp_ref)
+
+
+@pytest.mark.parametrize("batch,kv_heads,context,chosen", [(1, 8, 2048, 16), (1, 8, 8192, 32), (1, 1, 16384, 64), (2, 8, 2048, 16)])
+def test_decode_attention_with_the_key_splits_that_the_step_chooses(ops, batch, kv_heads, context, chosen):
+    """What a decode step at batch 1 or 2 launches once its block tables are wider than 64 pages:
+    the count of key splits is left to ``ops.decode_splits`` (given the table-width bound as the
+    step gives it), both for finished queries and for the kernel that prepares its own."""
+    assert ops.decode_splits(batch, kv_heads, context) == chosen
+    g = torch.Generator().manual_seed(63)
+    q_heads, head_dim, block_size = 2 * kv_heads, 64, 16
+    contexts = [context - 1 - 37 * i for i in range(batch)]     # the longest fills the bound to its last key
+    qkv, kp, vp, cu, ctx, table, qw, kw, inv_freq, positions, token_seq = _prepare_case(
+        g, q_heads, kv_heads, head_dim, block_size, contexts)
+    sizes = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim)
+    qkv_ref, kp_ref, vp_ref = qkv.clone(), kp.clone(), vp.clone()
+    refs.qk_norm_rope_write(qkv_ref, qw, kw, inv_freq, positions, token_seq, table, kp_ref, vp_ref,
+                            rotary_dim=head_dim, eps=1e-6, **sizes)
+    want = refs.paged_attention_by_matrices(qkv_ref, kp_ref, vp_ref, cu, ctx, table, scale=head_dim ** -0.5, **sizes)
+    out = torch.full((batch, q_heads * head_dim), float("nan"), dtype=torch.bfloat16, device=DEV)
+    kp_dev, vp_dev = kp.to(DEV), vp.to(DEV)
+    ops.decode_attention_prepare(qkv.to(DEV), qw.to(DEV), kw.to(DEV), inv_freq.to(DEV), kp_dev, vp_dev, out, cu.to(DEV),
+                                 ctx.to(DEV), table.to(DEV), eps=1e-6, scale=head_dim ** -0.5, max_ctx=context, **sizes)
+    torch.testing.assert_close(out.cpu().float(), want, atol=2e-2, rtol=2e-2)
+    # finished queries over the pages that the launch above completed
+    out = torch.full((batch, q_heads * head_dim), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.paged_attention(qkv_ref.to(DEV), kp_dev, vp_dev, out, cu.to(DEV), ctx.to(DEV), table.to(DEV), num_seqs=batch,
+                        max_q_len=1, num_decode=batch, max_ctx=context, scale=head_dim ** -0.5, **sizes)
+    torch.testing.assert_close(out.cpu().float(), want, atol=2e-2, rtol=2e-2)
+
+
 def test_attention_kernels_on_random_mixed_batches(ops):
     """Random head counts, groups, page sizes, windows and mixtures of single tokens and portions
     (with and without context before them): the fast kernels that a bfloat16 batch is routed to
@@ -1319,6 +1399,28 @@ def test_prefill_attention_kernel_long_walks(ops, q_heads, kv_heads, head_dim, b
     got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV),
                               torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
                               cu.to(DEV), ctx.to(DEV), table.to(DEV), num_decode=1, max_ctx=2048, **kw).cpu().float()
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("key_groups", [1, 2])
+@pytest.mark.parametrize("seqs,q_heads,kv_heads,head_dim", [
+    ([(0, 2048)], 4, 2, 128), ([(0, 8192)], 2, 1, 128), ([(0, 1024)] * 8, 4, 2, 64), ([(6000, 2048), (0, 1)], 2, 1, 64),
+])
+def test_prefill_attention_kernel_at_the_lengths_of_the_benchmarks(ops, seqs, q_heads, kv_heads, head_dim, key_groups, monkeypatch):
+    """Whole prompts of 2,048 and 8,192 tokens, eight of 1,024, and a portion of 2,048 behind 6,000
+    cached tokens: walks of up to 128 key tiles, with blocks of one and of two key groups."""
+    monkeypatch.setattr(ops, "PREFILL_KEY_GROUPS", key_groups)
+    g = torch.Generator().manual_seed(46)
+    q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, 16,
+                                                extra_width=2 * kv_heads * head_dim)
+    kw = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=head_dim ** -0.5)
+    want = refs.paged_attention_by_matrices(q, kp, vp, cu, ctx, table, **kw)
+    longest = max(n for _, n in seqs)
+    got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV),
+                              torch.full((q.shape[0], q_heads * head_dim), float("nan"), dtype=q.dtype, device=DEV),
+                              cu.to(DEV), ctx.to(DEV), table.to(DEV), num_seqs=len(seqs), max_q_len=longest,
+                              num_decode=sum(1 for _, n in seqs if n == 1), max_ctx=max(b + n for b, n in seqs), **kw).cpu().float()
     assert torch.isfinite(got).all()
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
 

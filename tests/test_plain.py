@@ -284,3 +284,133 @@ def test_attention_block_is_library_attention_with_its_default_scale():
     want = want.transpose(0, 1).reshape(7, heads * d) @ w[f"{prefix}.o_proj.weight"].T
     got = plain.attention_block(x, w, prefix, config, torch.arange(7))
     torch.testing.assert_close(got, want, atol=1e-6, rtol=1e-5)
+
+
+def _one_layer_attention_only(seed: int, **overrides):
+    """A one-layer model of configuration A whose feed-forward is silenced: the layer's update of
+    the stream is the attention block's output alone."""
+    config = dict(TINY["A"], num_hidden_layers=1, **overrides)
+    w = plain.random_weights(config, seed)
+    w["model.layers.0.mlp.down_proj.weight"].zero_()
+    return config, w
+
+
+def test_input_norm_weight_scales_what_the_projections_read():
+    # x = w_in * normalised(h) feeds q, k and v (qwen3.py:248-253): zeroing element j of the input
+    # norm's weight is zeroing column j of W_q, W_k and W_v; a unit weight, or the post-attention
+    # norm's weight in its place, breaks the first equality.  Scaling the weight by c scales v by c
+    # and leaves q and k to their own norms: the update scales by c (the eps is made tiny for that).
+    config, w = _one_layer_attention_only(21, rms_norm_eps=1e-12)
+    p = "model.layers.0"
+    ids = torch.tensor([9, 8, 100, 7, 33])
+    e = w["model.embed_tokens.weight"][ids]
+    _, hidden = plain.forward(w, config, ids, return_hidden=True)
+    update = hidden[0] - e
+    assert update.abs().max() > 1e-4
+    for j in (0, 17, 63):
+        gated = dict(w)
+        gated[f"{p}.input_layernorm.weight"] = w[f"{p}.input_layernorm.weight"].clone()
+        gated[f"{p}.input_layernorm.weight"][j] = 0.0
+        cut = dict(w)
+        for name in ("q_proj", "k_proj", "v_proj"):
+            cut[f"{p}.self_attn.{name}.weight"] = w[f"{p}.self_attn.{name}.weight"].clone()
+            cut[f"{p}.self_attn.{name}.weight"][:, j] = 0.0
+        _, a = plain.forward(gated, config, ids, return_hidden=True)
+        _, b = plain.forward(cut, config, ids, return_hidden=True)
+        torch.testing.assert_close(a[0], b[0], atol=1e-7, rtol=1e-5)
+        assert (a[0] - hidden[0]).abs().max() > 1e-5             # and element j did matter
+    scaled = dict(w)
+    scaled[f"{p}.input_layernorm.weight"] = w[f"{p}.input_layernorm.weight"] * 3.0
+    _, c = plain.forward(scaled, config, ids, return_hidden=True)
+    torch.testing.assert_close(c[0] - e, 3.0 * update, atol=1e-7, rtol=1e-4)
+    # the post-attention norm's weight does not reach the attention at all (the feed-forward is silent)
+    other = dict(w)
+    other[f"{p}.post_attention_layernorm.weight"] = w[f"{p}.post_attention_layernorm.weight"] * 5.0
+    _, d = plain.forward(other, config, ids, return_hidden=True)
+    torch.testing.assert_close(d[0], hidden[0], atol=0, rtol=0)
+
+
+def test_input_norm_uses_the_configurations_eps():
+    # One token: its attention output is its own value whatever q and k are, so the layer's update
+    # is W_o expand(W_v x) with x = w_in * e / sqrt(mean(e^2) + eps) (qwen3.py:99-105,237,248).
+    # The embedding row is scaled so that mean(e^2) equals eps exactly: the norm then divides by
+    # sqrt(2) times the row's RMS, a factor that another eps (1e-6, say) would not give.
+    eps = 1e-3
+    config, w = _one_layer_attention_only(22, rms_norm_eps=eps)
+    p = "model.layers.0"
+    token = 41
+    row = w["model.embed_tokens.weight"][token]
+    row *= math.sqrt(eps) / row.square().mean().sqrt()
+    e = w["model.embed_tokens.weight"][token]
+    assert abs(float(e.square().mean()) - eps) < 1e-9
+    x = w[f"{p}.input_layernorm.weight"] * e / (math.sqrt(2.0) * e.square().mean().sqrt())
+    groups = config["num_attention_heads"] // config["num_key_value_heads"]
+    v = (w[f"{p}.self_attn.v_proj.weight"] @ x).view(config["num_key_value_heads"], config["head_dim"])
+    want = w[f"{p}.self_attn.o_proj.weight"] @ v.repeat_interleave(groups, dim=0).reshape(-1)
+    _, hidden = plain.forward(w, config, [token], return_hidden=True)
+    torch.testing.assert_close(hidden[0][0] - e, want, atol=1e-8, rtol=1e-5)
+    wrong = w[f"{p}.self_attn.o_proj.weight"] @ (v * math.sqrt(2.0)).repeat_interleave(groups, dim=0).reshape(-1)   # what eps -> 0 gives
+    assert (hidden[0][0] - e - wrong).abs().max() > 1e-4 * wrong.abs().max()
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_layers_run_in_the_order_of_their_numbers(name):
+    # the stream after layer i of an L-layer model is the output of the (i + 1)-layer model made
+    # of the first i + 1 layers' tensors alone (qwen3.py:328-331)
+    config = TINY[name]
+    w = plain.random_weights(config, 23)
+    ids = torch.randint(0, config["vocab_size"], (9,), generator=torch.Generator().manual_seed(2))
+    _, hidden = plain.forward(w, config, ids, return_hidden=True)
+    assert len(hidden) == config["num_hidden_layers"]
+    for count in range(1, config["num_hidden_layers"]):
+        shorter = dict(config, num_hidden_layers=count)
+        first = {k: v for k, v in w.items() if not k.startswith("model.layers.")
+                 or int(k.split(".")[2]) < count}
+        _, partial = plain.forward(first, shorter, ids, return_hidden=True)
+        torch.testing.assert_close(hidden[count - 1], partial[-1], atol=0, rtol=0)
+        assert (hidden[count - 1] - hidden[count]).abs().max() > 1e-4
+
+
+def test_attention_biases_are_added_to_the_projections_before_the_head_norms():
+    # attention_bias (qwen3.py:115-122): with W_q = W_k = 0 every query is norm(b_q) and every key
+    # norm(b_k), each turned by its position; v = W_v x + b_v; the output gets b_o.  The biases'
+    # RMS is far from one, so a bias added after the per-head norm, like a bias that is dropped,
+    # gives other scores; values differ from token to token, so the scores matter.
+    config = dict(TINY["B"], attention_bias=True)
+    heads, kv_heads, d = config["num_attention_heads"], config["num_key_value_heads"], config["head_dim"]
+    w = plain.random_weights(config, 24)
+    prefix = "model.layers.0.self_attn"
+    g = torch.Generator().manual_seed(25)
+    w[f"{prefix}.q_proj.weight"].zero_()
+    w[f"{prefix}.k_proj.weight"].zero_()
+    w[f"{prefix}.v_proj.weight"] *= 20.0
+    biases = {"q_proj": torch.randn(heads * d, generator=g) * 3.0, "k_proj": torch.randn(kv_heads * d, generator=g) * 3.0,
+              "v_proj": torch.randn(kv_heads * d, generator=g), "o_proj": torch.randn(config["hidden_size"], generator=g)}
+    for name, bias in biases.items():
+        w[f"{prefix}.{name}.bias"] = bias
+    length = 6
+    x = torch.randn(length, config["hidden_size"], generator=g)
+    eps = config["rms_norm_eps"]
+    q = F.rms_norm(biases["q_proj"].view(heads, d), (d,), w[f"{prefix}.q_norm.weight"], eps)
+    k = F.rms_norm(biases["k_proj"].view(kv_heads, d), (d,), w[f"{prefix}.k_norm.weight"], eps)
+    q = q.unsqueeze(1).expand(heads, length, d)
+    k = k.unsqueeze(1).expand(kv_heads, length, d)
+    v = (x @ w[f"{prefix}.v_proj.weight"].T + biases["v_proj"]).view(length, kv_heads, d).transpose(0, 1)
+    cos, sin = plain.rotary_tables(torch.arange(length), d, config["rope_theta"])
+    q, k = plain.apply_rotary(q, cos, sin), plain.apply_rotary(k, cos, sin)
+    groups = heads // kv_heads
+    want = F.scaled_dot_product_attention(q.unsqueeze(0), k.repeat_interleave(groups, 0).unsqueeze(0),
+                                          v.repeat_interleave(groups, 0).unsqueeze(0), is_causal=True)[0]
+    want = want.transpose(0, 1).reshape(length, heads * d) @ w[f"{prefix}.o_proj.weight"].T + biases["o_proj"]
+    got = plain.attention_block(x, w, prefix, config, torch.arange(length))
+    torch.testing.assert_close(got, want, atol=1e-5, rtol=1e-5)
+    # each of the four biases matters here
+    for name in biases:
+        without = {key: value for key, value in w.items() if key != f"{prefix}.{name}.bias"}
+        assert (plain.attention_block(x, without, prefix, config, torch.arange(length)) - want).abs().max() > 1e-3, name
+    # and a bias added after the norm would give other scores: the unnormalised biases are three times as long
+    unnormalised = plain.apply_rotary(biases["q_proj"].view(heads, d).unsqueeze(1).expand(heads, length, d), cos, sin)
+    other = F.scaled_dot_product_attention(unnormalised.unsqueeze(0), k.repeat_interleave(groups, 0).unsqueeze(0),
+                                           v.repeat_interleave(groups, 0).unsqueeze(0), is_causal=True)[0]
+    other = other.transpose(0, 1).reshape(length, heads * d) @ w[f"{prefix}.o_proj.weight"].T + biases["o_proj"]
+    assert (other - want).abs().max() > 1e-3

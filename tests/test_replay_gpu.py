@@ -66,6 +66,35 @@ def test_replay_matches_plain(name, mode, dtype, folders, plain_cache, tmp_path)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_of_long_requests_whose_block_tables_cross_64_and_128_pages(dtype, folders, tmp_path):
+    """The lengths at which benchmarks run and no tiny trace arrives: a request of 2,608 tokens fed
+    as 2,048 + 500 and then token by token, beside one of 1,100 tokens fed as 1,000 and then token by
+    token.  The block tables pass 64 pages (the second of the captured decode steps' table widths),
+    128 and 160; the decode attention takes 16 key splits and then 24 (the merge in one round, and
+    the merge in a loop); the prefill attention walks 32 key tiles.  Every position's logits are
+    compared with the plain implementation."""
+    name = "C"
+    requests = ru.make_requests(TINY[name], 17, (2608, 1100))
+    long, grow = requests["r0"], requests["r1"]
+    trace = ru.TraceBuilder()
+    trace.step([("r0", long[:2048])])
+    trace.step([("r1", grow[:1000])])
+    trace.step([("r0", long[2048:2548])])
+    for i in range(100):                       # both decode; the shorter one ends after 100 tokens, the longer after 60
+        parts = [("r1", grow[1000 + i:1001 + i])]
+        if i < 60:
+            parts.append(("r0", long[2548 + i:2549 + i]))
+        trace.step(parts, end=[r for r, last in (("r0", 59), ("r1", 99)) if i == last])
+    print(f"long replay {dtype}: {len(trace.steps)} steps, pool for {trace.peak_tokens} tokens", flush=True)
+    got = ru.run_trace(folders[name], dtype, trace, tmp_path, block_size=BLOCK_SIZE[name])
+    tables = [json.loads((tmp_path / f"{i}.json").read_text())["tables"] for i in range(len(trace.steps))]
+    assert len(tables[3]["r1"]["pages"][0]) == 63 and len(tables[30]["r1"]["pages"][0]) == 65     # crosses 64 pages while decoding
+    assert len(tables[3]["r0"]["pages"][0]) == 160 and len(tables[62]["r0"]["pages"][0]) == 163
+    worst = ru.compare(got, ru.plain_logits(folders[name], requests), dtype)
+    print(f"  worst difference {worst:.3e}", flush=True)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("mode", list(TRACES))
 def test_replay_of_the_reference_tiny_configuration(mode, dtype, tmp_path):
     """The configuration of the reference's own model tests: two query heads of four elements over
