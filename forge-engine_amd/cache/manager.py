@@ -30,6 +30,11 @@ class CacheGroup:
     head_dim: int
     window: int | None
     slots: tuple[int, ...]  # cache slots (schedule indices that write) in this group
+    value_dim: int = -1     # width of a value row (-1: head_dim; 0: the group holds keys only)
+
+    @property
+    def value_width(self) -> int:
+        return self.head_dim if self.value_dim < 0 else self.value_dim
 
 
 @dataclass
@@ -53,11 +58,11 @@ def plan_groups(needs: list[CacheNeeds], schedule) -> tuple[list[CacheGroup], di
         paged = needs[index].paged
         if paged is None or call.cache != index:
             continue
-        by_key.setdefault((paged.kv_heads, paged.head_dim, paged.window), []).append(index)
+        by_key.setdefault((paged.kv_heads, paged.head_dim, paged.window, paged.value_width), []).append(index)
     groups = []
     where: dict[int, tuple[int, int]] = {}
     for g, (key, slots) in enumerate(by_key.items()):
-        groups.append(CacheGroup(g, key[0], key[1], key[2], tuple(slots)))
+        groups.append(CacheGroup(g, key[0], key[1], key[2], tuple(slots), key[3]))
         for j, slot in enumerate(slots):
             where[slot] = (g, j)
     for index, call in enumerate(schedule):
@@ -66,7 +71,7 @@ def plan_groups(needs: list[CacheNeeds], schedule) -> tuple[list[CacheGroup], di
             if call.cache not in where:
                 raise ValueError(f"schedule entry {index} reads cache slot {call.cache}, which holds no pages")
             owner = needs[call.cache].paged
-            if (owner.kv_heads, owner.head_dim) != (paged.kv_heads, paged.head_dim):
+            if (owner.kv_heads, owner.head_dim, owner.value_width) != (paged.kv_heads, paged.head_dim, paged.value_width):
                 raise ValueError(f"schedule entry {index} reads a cache of another geometry")
             # the owner's window decides which pages go back: a reader that looks further back
             # would read pages that are no longer the request's

@@ -2,8 +2,8 @@
 
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import Any
+from dataclasses import dataclass, field
+from typing import Any, Mapping
 
 
 @dataclass(frozen=True)
@@ -15,6 +15,11 @@ class PagedKV:
     kv_heads: int
     head_dim: int
     window: int | None = None
+    value_dim: int | None = None   # width of a value row: None, as wide as a key; 0: keys only, no value pages at all
+
+    @property
+    def value_width(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)
@@ -27,8 +32,19 @@ class FixedState:
 
 @dataclass(frozen=True)
 class CacheNeeds:
+    """``state``: one ``FixedState``, or several by name, each with a shape and a dtype of its own
+    (a recurrent state in float32 beside the tail of a short convolution in bfloat16, say)."""
+
     paged: PagedKV | None = None
-    state: FixedState | None = None
+    state: FixedState | Mapping[str, FixedState] | None = None
+
+    def states(self) -> dict[str, FixedState]:
+        """The states by name; a single unnamed one is called ``state``."""
+        if self.state is None:
+            return {}
+        if isinstance(self.state, FixedState):
+            return {"state": self.state}
+        return dict(self.state)
 
 
 @dataclass
@@ -36,9 +52,11 @@ class CacheView:
     """What one layer call sees of the cache in one step.
 
     ``key_pages`` [blocks, kv_heads, block_size, head_dim] and ``value_pages``
-    (transposed) [blocks, kv_heads, head_dim, block_size] of this call's cache slot; ``block_table``: int32 [sequences, max_blocks] of the
-    slot's group (entry -1: no page); ``state``: [slots, *shape] of this call's
-    fixed-size state, indexed by ``StepBatch.state_slots``.
+    (transposed) [blocks, kv_heads, value width, block_size] of this call's cache slot (None for a
+    mixer that keeps keys only); ``block_table``: int32 [sequences, max_blocks] of the
+    slot's group (entry -1: no page); ``states``: by name, [slots, *shape] of each of this call's
+    fixed-size states, indexed by ``StepBatch.state_slots``; ``state``: the only one, for a mixer
+    that has one.
     """
 
     key_pages: Any = None
@@ -46,4 +64,10 @@ class CacheView:
     block_table: Any = None
     block_size: int = 0
     window: int | None = None
-    state: Any = None
+    states: dict = field(default_factory=dict)
+
+    @property
+    def state(self) -> Any:
+        if len(self.states) != 1:
+            raise AttributeError(f"this call has {len(self.states)} fixed-size states: name one in ``states``")
+        return next(iter(self.states.values()))

@@ -154,9 +154,10 @@ class _PortionGraph:
 
 
 class ModelRunner:
-    def __init__(self, model: DecoderModel, *, block_size: int, block_capacity: int,
+    def __init__(self, model: DecoderModel, *, block_size: int, block_capacity: int | list[int] | tuple[int, ...],
                  num_state_slots: int, use_graphs: bool = True, eager_sightings: int | None = None) -> None:
-        """``eager_sightings``: how often a shape of a step with prompt portions runs eagerly before
+        """``block_capacity``: pages of every cache group's pool, or one count per group (a group
+        whose window bounds what a request holds needs fewer).  ``eager_sightings``: how often a shape of a step with prompt portions runs eagerly before
         it is captured (None: by the step's size, see ``PORTION_GRAPH_SIGHTINGS``; a loop that repeats
         one shape, a benchmark for instance, passes 1)."""
         self.model = model
@@ -179,22 +180,22 @@ class ModelRunner:
         if self.device.type == "cuda":
             library.ensure_built(sorted(model.kernel_libraries()))
         # pages of a group, per cache slot: keys [page, kv head, position in page, head dim],
-        # values transposed [page, kv head, head dim, position in page]
+        # values transposed [page, kv head, value width, position in page]; a group that keeps keys
+        # only has no value pages
+        capacities = [pool.capacity for pool in self.cache.pools]
         self.key_pages = [
-            torch.zeros((len(g.slots), block_capacity, g.kv_heads, block_size, g.head_dim),
-                        dtype=self.dtype, device=self.device) for g in groups]
+            torch.zeros((len(g.slots), capacity, g.kv_heads, block_size, g.head_dim),
+                        dtype=self.dtype, device=self.device) for g, capacity in zip(groups, capacities)]
         self.value_pages = [
-            torch.zeros((len(g.slots), block_capacity, g.kv_heads, g.head_dim, block_size),
-                        dtype=self.dtype, device=self.device) for g in groups]
-        self.states: list[Tensor | None] = []
-        for need in needs:
-            if need.state is None:
-                self.states.append(None)
-            else:
-                # one row more than there are slots: the empty sequences that pad a captured step
-                # point there, so that a mixer that writes its state back never touches a live slot
-                self.states.append(torch.zeros((num_state_slots + 1, *need.state.shape),
-                                               dtype=need.state.dtype or torch.float32, device=self.device))
+            torch.zeros((len(g.slots), capacity, g.kv_heads, g.value_width, block_size),
+                        dtype=self.dtype, device=self.device) if g.value_width else None
+            for g, capacity in zip(groups, capacities)]
+        # fixed-size states of every schedule call, by name, each with its own shape and dtype; one row
+        # more than there are slots: the empty sequences that pad a captured step point there, so that
+        # a mixer that writes its state back never touches a live slot
+        self.states: list[dict[str, Tensor]] = [
+            {name: torch.zeros((num_state_slots + 1, *state.shape), dtype=state.dtype or torch.float32, device=self.device)
+             for name, state in need.states().items()} for need in needs]
         self.pad_state_slot = num_state_slots
         self.steps_run = 0
         self.workspace = ops.Workspace()    # scratch that this runner's launches (and its captured graphs) share
@@ -204,8 +205,8 @@ class ModelRunner:
         """Lease a state slot and empty tables for the request.  The slot's fixed-size state starts
         at zero: the runner clears it here, so a mixer never has to know a request's first step."""
         record = self.cache.begin(request_id)
-        for state in self.states:
-            if state is not None:
+        for states in self.states:
+            for state in states.values():
                 state[record.state_slot].zero_()
 
     def end(self, request_id: str) -> None:
@@ -249,16 +250,17 @@ class ModelRunner:
         state is handed out as a copy, for a run whose effects on it must not stay."""
         views: list[CacheView | None] = []
         for index, call in enumerate(self.model.schedule):
-            state = self.states[index]
-            if scratch_state and state is not None:
-                state = state.clone()
+            states = self.states[index]
+            if scratch_state:
+                states = {name: state.clone() for name, state in states.items()}
             if call.cache in self._where:
                 g, j = self._where[call.cache]
                 group = self.cache.groups[g]
-                views.append(CacheView(self.key_pages[g][j], self.value_pages[g][j], batch.block_tables[g],
-                                       self.block_size, group.window, state))
-            elif state is not None:
-                views.append(CacheView(state=state))
+                values = self.value_pages[g]
+                views.append(CacheView(self.key_pages[g][j], None if values is None else values[j], batch.block_tables[g],
+                                       self.block_size, group.window, states))
+            elif states:
+                views.append(CacheView(states=states))
             else:
                 views.append(None)
         return views

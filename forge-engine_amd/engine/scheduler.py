@@ -106,7 +106,7 @@ class _Request:
     seed: int
     eos_ids: frozenset
     detokenizer: IncrementalDetokenizer | None
-    reserved_blocks: int
+    reserved_blocks: list[int]                         # per cache group
     admitted: int
     status: RequestStatus = RequestStatus.WAITING
     outputs: list[int] = field(default_factory=list)   # sampled tokens that go back into the model
@@ -151,12 +151,12 @@ class ConcurrentGenerationEngine:
             eos_token_ids = getattr(runner.model.plan, "eos_token_ids", frozenset())
         self._eos_ids = frozenset(eos_token_ids)
         cache = runner.cache
-        if cache.block_size != self._config.block_size or any(
-                pool.capacity != self._config.block_capacity for pool in cache.pools):
+        self._capacities = self._config.capacities(len(cache.pools))     # pages of each cache group's pool
+        if cache.block_size != self._config.block_size or [pool.capacity for pool in cache.pools] != self._capacities:
             raise ValueError("the runner's cache pool does not match the scheduler configuration")
         self._requests: dict[str, _Request] = {}
         self._order: deque[str] = deque()
-        self._reserved_blocks = 0
+        self._reserved = [0] * len(self._capacities)                     # pages reserved in each group
         self._next_number = 1
         self._admitted = 0
         self._iteration = 0
@@ -215,16 +215,18 @@ class ConcurrentGenerationEngine:
         if config.max_context is not None and total > config.max_context:
             raise OverloadedError(f"request needs {total} positions but max_context is {config.max_context}")
         portion = min(config.token_budget, config.prefill_chunk or config.token_budget)
-        needed = max(self._runner.cache.worst_case_pages(total, step_tokens=portion), default=0)
-        if needed > config.block_capacity:
-            raise OverloadedError(
-                f"request needs {needed} KV blocks but pool capacity is {config.block_capacity}")
-        reserved = 0
+        # every cache group has a pool of its own: a group whose window bounds what a request holds
+        # needs, and reserves, less than one that keeps every key
+        needed = self._runner.cache.worst_case_pages(total, step_tokens=portion)
+        for need, capacity in zip(needed, self._capacities):
+            if need > capacity:
+                raise OverloadedError(f"request needs {need} KV blocks but pool capacity is {capacity}")
+        reserved = [0] * len(needed)
         if config.admission == "reserve":
-            available = config.block_capacity - self._reserved_blocks
-            if needed > available:
-                raise OverloadedError(
-                    f"request needs {needed} KV blocks but only {available} are unreserved")
+            for need, capacity, taken in zip(needed, self._capacities, self._reserved):
+                if need > capacity - taken:
+                    raise OverloadedError(
+                        f"request needs {need} KV blocks but only {capacity - taken} are unreserved")
             reserved = needed
         detokenizer = None
         if self._tokenizer is not None:
@@ -237,7 +239,7 @@ class ConcurrentGenerationEngine:
         self._requests[assigned] = _Request(assigned, tokens, params, seed, self._eos_ids, detokenizer,
                                             reserved, self._admitted, holds_cache=True)
         self._order.append(assigned)
-        self._reserved_blocks += reserved
+        self._reserved = [taken + more for taken, more in zip(self._reserved, reserved)]
         return assigned
 
     def cancel(self, request_id: str) -> bool:
@@ -531,7 +533,7 @@ class ConcurrentGenerationEngine:
             self._runner.end(request.request_id)
             request.holds_cache = False
         if not request.reservation_released:
-            self._reserved_blocks -= request.reserved_blocks
+            self._reserved = [taken - held for taken, held in zip(self._reserved, request.reserved_blocks)]
             request.reservation_released = True
 
     def _drop_terminal(self) -> None:
@@ -541,7 +543,7 @@ class ConcurrentGenerationEngine:
     def request(self, request_id: str) -> RequestView:
         r = self._request(request_id)
         return RequestView(r.request_id, r.status, len(r.prompt), r.sampled_tokens,
-                           0 if r.reservation_released else r.reserved_blocks, r.finish_reason, r.error,
+                           0 if r.reservation_released else max(r.reserved_blocks, default=0), r.finish_reason, r.error,
                            tuple(r.outputs), r.text)
 
     def forget(self, request_id: str) -> None:
@@ -558,7 +560,7 @@ class ConcurrentGenerationEngine:
             waiting=sum(r.status is RequestStatus.WAITING for r in requests),
             running=sum(r.status is RequestStatus.RUNNING for r in requests),
             terminal=sum(r.status.terminal for r in requests),
-            reserved_blocks=self._reserved_blocks,
+            reserved_blocks=max(self._reserved, default=0),
             allocated_blocks=self._runner.cache.allocated_pages,
             last_batch=self._last_batch,
             model_batches=(self._last_batch,) if self._last_batch else (),

@@ -499,9 +499,10 @@ def test_attention_mixer_and_block_alone(dtype):
 # ------------------------------------------------- a toy architecture, defined here
 
 class EmaMixer(Mixer):
-    """A toy mixer with state of its own: s_t = decay * s_{t-1} + x_t (per
-    request, reset at its first token), update = W s_t.  Plain torch ops: it is
-    test code, not a kernel."""
+    """A toy mixer with two states of its own, of different shape and precision: a float32
+    s_t = decay * s_{t-1} + x_t (per request, zero before its first token) and a bfloat16 pair
+    (n_t, -n_t) that counts the request's tokens (small integers: exact in bfloat16);
+    update = W s_t + (n_t / 8) W[:, 0].  Plain torch ops: it is test code, not a kernel."""
 
     graph_safe = False      # it loops over the step's requests on the host
 
@@ -517,19 +518,23 @@ class EmaMixer(Mixer):
         self.weight = tensor
 
     def cache_needs(self):
-        return CacheNeeds(state=FixedState((self.hidden_size,), torch.float32))
+        return CacheNeeds(state={"ema": FixedState((self.hidden_size,), torch.float32),
+                                 "seen": FixedState((2,), torch.bfloat16)})
 
     def forward(self, x, batch, cache, writes_cache=True):
+        assert cache.states["ema"].dtype == torch.float32 and cache.states["seen"].dtype == torch.bfloat16
         out = torch.empty((x.shape[0], self.hidden_size), dtype=torch.float32, device=x.device)
         slots = batch.state_slots_host
+        weight = self.weight.float()
         at = 0
         for i, count in enumerate(batch.q_lens):
-            state = cache.state[slots[i]]
-            if batch.ctx_before_host[i] == 0:
-                state.zero_()                      # a slot is reused: a request's first portion starts from zero
+            # both states are zero when a request begins, also in a slot that another request used: the runner clears them
+            state, seen = cache.states["ema"][slots[i]], cache.states["seen"][slots[i]]
             for t in range(at, at + count):
                 state.mul_(self.decay).add_(x[t].float())
-                out[t] = self.weight.float() @ state
+                seen += torch.tensor([1.0, -1.0], dtype=seen.dtype, device=seen.device)
+                assert float(seen[0]) == batch.ctx_before_host[i] + t - at + 1 and float(seen[1]) == -float(seen[0])
+                out[t] = weight @ state + seen[0].float() / 8.0 * weight[:, 0]
             at += count
         return out
 
@@ -539,8 +544,9 @@ class DeviceEmaMixer(EmaMixer):
     device tensors of the batch (``cu_q``, ``token_seq``, ``state_slots``), so its steps may be
     captured and replayed.  Within a step, token t of a sequence that starts at token a gets
     s_t = decay^(t-a+1) * s_before + sum_{a <= u <= t} decay^(t-u) x_u; the state after the
-    sequence's last token goes back to its slot, and an empty sequence leaves its slot alone.
-    The slot starts at zero because the runner clears it when the request begins."""
+    sequence's last token goes back to its slot, and an empty sequence leaves its slot alone; the
+    count of tokens seen goes on from the slot's likewise.  The slot starts at zero because the
+    runner clears it when the request begins."""
 
     graph_safe = True
 
@@ -553,14 +559,19 @@ class DeviceEmaMixer(EmaMixer):
         distance = t[:, None] - t[None, :]
         visible = (seq[:, None] == seq[None, :]) & (distance >= 0)
         mix = torch.where(visible, torch.pow(self.decay, distance.clamp(min=0).float()), torch.zeros((), device=x.device))
-        before = cache.state.index_select(0, slots)
+        ema, seen = cache.states["ema"], cache.states["seen"]
+        before = ema.index_select(0, slots)
         carried = torch.pow(self.decay, (t - start + 1).float())[:, None] * before.index_select(0, seq)
         states = mix @ xf + carried
         lengths = cu[1:] - cu[:-1]
         last = (cu[1:] - 1).clamp(min=0)
         after = torch.where((lengths > 0)[:, None], states.index_select(0, last), before)
-        cache.state.index_copy_(0, slots, after)
-        return states @ self.weight.float().T
+        ema.index_copy_(0, slots, after)
+        seen_before = seen.index_select(0, slots).float()                       # [sequences, 2]: (n, -n)
+        count = seen_before[:, 0].index_select(0, seq) + (t - start + 1).float()
+        seen.index_copy_(0, slots, (seen_before + torch.stack((lengths, -lengths), dim=1).float()).to(seen.dtype))
+        weight = self.weight.float()
+        return states @ weight.T + (count / 8.0)[:, None] * weight[:, 0][None, :]
 
 
 @dataclass(frozen=True)
@@ -639,7 +650,7 @@ def toy_plain_forward(weights, config: ToyConfig, tokens):
         rows = []
         for t in range(len(tokens)):
             state = config.decay * state + x[t]
-            rows.append(weights[f"{prefix}.mix.weight"] @ state)
+            rows.append(weights[f"{prefix}.mix.weight"] @ state + (t + 1) / 8.0 * weights[f"{prefix}.mix.weight"][:, 0])
         return torch.stack(rows)
 
     for call, (index, mode) in enumerate([(0, "own"), (1, "ema"), (2, "window"), (0, "own"), (1, "ema"), (0, "shared")]):
@@ -672,9 +683,13 @@ def test_toy_architecture_registered_from_a_test(dtype, ema):
     assert isinstance(config, ToyConfig)
     model = build_model(config, dtype=dtype, device=DEV)
     fill_random_weights(model, 7, device=DEV, dtype=model.ctx.dtype)
-    runner = ModelRunner(model, block_size=4, block_capacity=24, num_state_slots=2)
+    # the windowed group has a smaller pool: two requests hold at most its window's keys and a step's (4 pages each)
+    runner = ModelRunner(model, block_size=4, block_capacity=[24, 8], num_state_slots=2)
     groups = runner.cache.groups
-    assert sorted((g.window or 0, len(g.slots)) for g in groups) == [(0, 2), (6, 1)]   # windowed pages apart from full ones
+    assert [(g.window or 0, len(g.slots)) for g in groups] == [(0, 2), (6, 1)]   # windowed pages apart from full ones
+    assert [p.shape[1] for p in runner.key_pages] == [24, 8] and [pool.capacity for pool in runner.cache.pools] == [24, 8]
+    assert {name: (tuple(t.shape[1:]), t.dtype) for name, t in runner.states[1].items()} == {
+        "ema": ((40,), torch.float32), "seen": ((2,), torch.bfloat16)}
     weights = {}
     for name in model.param_specs():
         owner = model._owners[name]
