@@ -421,19 +421,21 @@ def main() -> int:
         return 0
     prefill_times, _ = timed(prefill_once, 2, max(3, min(10, args.steps)))
     prefill_ms = spread(prefill_times)["median"]
-    if args.phase == "prefill":
-        print(json.dumps({"phase": "prefill", "model": chosen["label"], "tokens": args.prefill_tokens, "ms": prefill_ms,
-                          "step_ms": spread(prefill_times),
-                          "value": round(args.prefill_tokens / prefill_ms * 1e3, 1), "unit": "tokens/s",
-                          "layers_run": layers, "layers_model": full_layers}))
-        return 0
-
     matrix_params = layers * (config.hidden_size * (config.q_size + 2 * config.kv_size)
                               + config.q_size * config.hidden_size
                               + 3 * config.hidden_size * config.intermediate_size)
     t = args.prefill_tokens
     prefill_flops = 2.0 * t * matrix_params + 2.0 * t * t * config.q_size * layers \
         + 2.0 * config.vocab_size * config.hidden_size
+    if args.phase == "prefill":
+        print(json.dumps({"phase": "prefill", "model": chosen["label"], "dtype": args.dtype, "tokens": t, "ms": prefill_ms,
+                          "step_ms": spread(prefill_times),
+                          "value": round(t / prefill_ms * 1e3, 1), "unit": "tokens/s",
+                          "frac": round(prefill_flops / (prefill_ms * 1e-3) / PEAK_FLOPS[args.dtype], 4),
+                          "peak_tflops": PEAK_FLOPS[args.dtype] / 1e12,
+                          "layers_run": layers, "layers_model": full_layers}))
+        return 0
+
     times, wall, mean_ctx = results[args.batch]
     median = spread(times)["median"]
     record = {

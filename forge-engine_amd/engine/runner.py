@@ -16,7 +16,7 @@ from ..kernels import library, ops
 from ..models.decoder import DecoderModel
 from .batch import StepBatch, StepEntry, build_batch, static_batch, static_batch_size
 
-GRAPH_MAX_REQUESTS = 64      # decode steps of up to this many requests replay a captured graph
+GRAPH_MAX_REQUESTS = 256     # steps of up to this many requests replay a captured graph
 GRAPH_TABLE_STEP = 64        # block-table widths of graphs are multiples of this many pages
 GRAPH_LIMIT = 24             # captured graphs kept (least recently used goes first)
 PORTION_GRAPH_MAX_TOKENS = 4096   # steps with prompt portions of up to this many tokens may be captured

@@ -982,6 +982,45 @@ def test_batched_decode_through_graphs_matches_eager(dtype, folders):
     assert float((rows[True] - want).abs().max()) <= bound
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("count", [65, 130, 256])
+def test_decode_steps_of_many_requests_replay_graphs(count, dtype, folders):
+    """Decode steps of 65 to 256 requests are captured and replayed like smaller ones: every
+    request's last six tokens one by one, all requests in one step, against the plain
+    implementation; a 257th request makes the step run eagerly."""
+    name = "C"
+    config, weights = TINY[name], folder_weights(folders[name])
+    lengths = tuple(7 + (5 * i) % 23 for i in range(count))
+    requests = ru.make_requests(config, 41, lengths)
+    _, model = load_model(folders[name], dtype=dtype, device=DEV)
+    runner = ModelRunner(model, block_size=16, block_capacity=2 * count + 8, num_state_slots=count + 1)
+    names = list(requests)
+    for at in range(0, count, 40):                                  # prompts, forty requests a step
+        for k in names[at:at + 40]:
+            runner.begin(k)
+        runner.step([StepEntry(k, requests[k][:-6], []) for k in names[at:at + 40]])
+    collected = []
+    for step in range(6):
+        entries = [StepEntry(k, [requests[k][len(requests[k]) - 6 + step]], [0]) for k in names]
+        collected.append(runner.step(entries).clone())
+    assert runner.graph_replays == 6
+    got = torch.stack(collected).cpu()
+    want = torch.stack([plain.forward(weights, config, tokens)[-6:] for tokens in requests.values()], dim=1)
+    scale = float(want.abs().max())
+    bound = 1e-4 * scale + 1e-5 if dtype == "float32" else ru.BF16_FRACTION * scale
+    assert float((got - want).abs().max()) <= bound
+    if count == 256:
+        extra = ru.make_requests(config, 42, (9,))["r0"]
+        runner.begin("one more")
+        runner.step([StepEntry("one more", extra[:-1], [])])
+        replays = runner.graph_replays
+        entries = [StepEntry(k, [3], [0]) for k in names] + [StepEntry("one more", extra[-1:], [0])]
+        logits = runner.step(entries)
+        assert runner.graph_replays == replays and logits.shape[0] == 257
+        expect = plain.forward(weights, config, extra)[-1]
+        assert float((logits[-1].cpu() - expect).abs().max()) <= bound
+
+
 def test_steps_of_single_tokens_prepare_queries_and_keys_inside_attention(folders, monkeypatch):
     """A step in which every request brings one token runs norm, rotation, cache write and
     attention as one launch per layer; a mixed step runs them as two.  The same tokens fed
