@@ -484,6 +484,24 @@ def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
     return None
 
 
+def gemm_gated(x: Tensor, gate_up_weight: Tensor, shape: int = 0) -> Tensor:
+    """silu(x Wg^T) * (x Wu^T) for the fused weight [2I, K] (gate rows first) and any number of
+    bfloat16 rows: blocks keep a tile of rows of x in LDS and their accumulators in registers over
+    the whole of K; the intermediate [M, 2I] never exists.  ``shape``: the block's tile, see
+    ``fe_gemm_gated``."""
+    _gpu(x, "x", torch.bfloat16)
+    _gpu(gate_up_weight, "gate_up_weight", torch.bfloat16, contiguous=False)
+    m, k = x.shape
+    rows = gate_up_weight.shape[0]
+    if (gate_up_weight.dim() != 2 or gate_up_weight.shape[1] != k or k % 64 or rows % 2 or gate_up_weight.stride(1) != 1
+            or gate_up_weight.stride(0) % 8 or x.data_ptr() % 16 or gate_up_weight.data_ptr() % 16):
+        raise KernelError("the gated product takes contiguous bfloat16 rows, K a multiple of 64, an even number of weight rows")
+    out = torch.empty((m, rows // 2), dtype=torch.bfloat16, device=x.device)
+    _call("gemm_tile", "fe_gemm_gated", _ptr(x), _ptr(gate_up_weight), _ptr(out), c_int(m), c_int(rows // 2), c_int(k),
+          c_longlong(gate_up_weight.stride(0)), c_longlong(rows // 2), c_int(shape), _stream())
+    return out
+
+
 def _gate_block_columns(columns: int) -> int:
     """Output columns a block of the gate/up product for 17 to 64 rows takes (8 a wave, four to eight
     waves): the count whose blocks fill rounds of one a CU best, the larger of equals (x is read once a
@@ -929,4 +947,4 @@ def sample_filtered_rows(logits: Tensor, params: Tensor, tokens: Tensor, status:
           _stream())
 
 
-LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")
+LIBRARIES = ("rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "gemm_tile", "qk_rope", "attention_generic", "attention_decode", "attention_prefill", "sample")

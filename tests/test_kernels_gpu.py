@@ -767,6 +767,42 @@ def test_gemm_wide_stores_and_gates(ops, m, n, k):
         ops.gemm_wide(x.to(DEV), w.to(DEV), "swiglu", 1, 16, 64)        # the two-tile gate ending takes tiles of 64 and 128 rows
 
 
+@pytest.mark.parametrize("shape", [0, 1, 2])
+@pytest.mark.parametrize("m", [1, 70, 256, 300, 513])
+@pytest.mark.parametrize("inter,k", [(9728, 2560), (200, 192), (1003, 320), (64, 64)])
+def test_gemm_gated_tile(ops, shape, m, inter, k):
+    """The gate/up product with its SwiGLU ending for any number of rows (tiles of 128 or 256 rows of x
+    in LDS, 64 or 128 output columns a block): row counts and widths that are no multiple of the tile,
+    a width that is odd (the rows of the result then leave element by element), one step of K."""
+    g = torch.Generator().manual_seed(70 + shape)
+    x = rand(g, m, k, dtype=torch.bfloat16)
+    w = rand(g, 2 * inter, k, dtype=torch.bfloat16, scale=0.05)
+    want = refs.linear_swiglu(x, w).float()
+    got = ops.gemm_gated(x.to(DEV), w.to(DEV), shape).cpu()
+    assert got.shape == (m, inter) and got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), want, atol=2e-2 * float(want.abs().max()), rtol=2e-2)
+    # a weight whose rows lie further apart than they are long (a slice of a wider matrix)
+    wide = rand(g, 2 * inter, k + 64, dtype=torch.bfloat16, scale=0.05).to(DEV)
+    view = wide[:, :k]
+    want = refs.linear_swiglu(x, view.cpu()).float()
+    torch.testing.assert_close(ops.gemm_gated(x.to(DEV), view, shape).cpu().float(), want,
+                               atol=2e-2 * float(want.abs().max()), rtol=2e-2)
+
+
+def test_gemm_gated_tile_refuses(ops):
+    g = torch.Generator().manual_seed(71)
+    x = rand(g, 8, 96, dtype=torch.bfloat16).to(DEV)                 # K no multiple of 64
+    with pytest.raises(ops.KernelError):
+        ops.gemm_gated(x, rand(g, 64, 96, dtype=torch.bfloat16).to(DEV))
+    x = rand(g, 8, 128, dtype=torch.bfloat16).to(DEV)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_gated(x, rand(g, 63, 128, dtype=torch.bfloat16).to(DEV))      # an odd number of weight rows
+    with pytest.raises(ops.KernelError):
+        ops.gemm_gated(x, rand(g, 64, 128, dtype=torch.bfloat16).to(DEV), shape=7)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_gated(x.float(), rand(g, 64, 128, dtype=torch.bfloat16).to(DEV))
+
+
 def test_linear_swiglu_routes_by_rows(ops, monkeypatch):
     """Up to 64 rows at a K of up to 3072: the product that pairs gate and up rows within a wave (at a
     longer K from 17 rows, the streaming kernel below); more: the matrix library and the gate kernel.
