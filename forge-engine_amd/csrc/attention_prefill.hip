@@ -59,6 +59,7 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 
 #define BN 64        // keys per tile
 #define XCDS 8
+#define RESCALE_MARGIN 8.f   // base-2 units a row's maximum may exceed the exponents' reference point
 
 __device__ __forceinline__ unsigned int pack_bf16(float lo, float hi) {
   const bf16x2 v = {(__bf16)lo, (__bf16)hi};
@@ -190,7 +191,9 @@ __global__ __launch_bounds__(256 * KG, 4) void paged_prefill_kernel(   // four w
       qb[c] = __builtin_bit_cast(bf16x8, row < q_len ? v : uintx4{0u, 0u, 0u, 0u});
     }
   }
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = -INFINITY;
+  floatx4 l_sum = floatx4{0.f, 0.f, 0.f, 0.f};     // every entry: the row's sum of probabilities so far
+  const bf16x8 ones = __builtin_bit_cast(bf16x8, uintx4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
   floatx4 o[DT];
 #pragma unroll
   for (int t = 0; t < DT; ++t) o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -318,24 +321,25 @@ __global__ __launch_bounds__(256 * KG, 4) void paged_prefill_kernel(   // four w
           s[j] = visible ? s[j] : -INFINITY;
         }
       }
-      float mx = s[0];
-#pragma unroll
-      for (int j = 1; j < 16; ++j) mx = fmaxf(mx, s[j]);
+      // the largest of the lane's 16 scores as a tree (three-operand maxima), then across the four lanes of the row
+      float mx = fmaxf(fmaxf(fmaxf(fmaxf(s[0], s[1]), s[2]), fmaxf(fmaxf(s[3], s[4]), s[5])),
+                       fmaxf(fmaxf(fmaxf(s[6], s[7]), s[8]), fmaxf(fmaxf(s[9], s[10]), s[11])));
+      mx = fmaxf(fmaxf(mx, fmaxf(fmaxf(s[12], s[13]), s[14])), s[15]);
       mx = max_xor16(mx);
       mx = max_xor32(mx);
+      // The reference point of the exponents moves only when the row's maximum has outgrown it by more
+      // than RESCALE_MARGIN (base-2 units): until then the probabilities of this tile are at most
+      // 2^RESCALE_MARGIN instead of at most 1, which float32 sums and bfloat16 operands hold as well,
+      // and the 32 products that rescale the output, and the wave's vote on them, are left out.  The
+      // quotient at the end does not depend on the reference point.
       const float m_new = fmaxf(m_run, mx * scale_log2);   // the scale is positive
-      const float m_use = m_new > -INFINITY ? m_new : 0.f; // a row with nothing visible yet
-      const float corr = __builtin_amdgcn_exp2f(m_run - m_use);
-      float sum = 0.f;
+      const bool moved = m_new > m_run + RESCALE_MARGIN;   // (from -infinity: any finite maximum moves it)
+      const float m_next = moved ? m_new : m_run;
+      const float m_use = m_next > -INFINITY ? m_next : 0.f; // a row with nothing visible yet
+      const float corr = moved ? __builtin_amdgcn_exp2f(m_run - m_use) : 1.f;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        s[j] = __builtin_amdgcn_exp2f(fmaf(s[j], scale_log2, -m_use));
-        sum += s[j];
-      }
-      sum = sum_xor16(sum);
-      sum = sum_xor32(sum);
-      l_run = l_run * corr + sum;
-      m_run = m_new;
+      for (int j = 0; j < 16; ++j) s[j] = __builtin_amdgcn_exp2f(fmaf(s[j], scale_log2, -m_use));
+      m_run = m_next;
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk) {
         uintx4 pw;
@@ -343,11 +347,13 @@ __global__ __launch_bounds__(256 * KG, 4) void paged_prefill_kernel(   // four w
         pw.z = pack_bf16(s[8 * blk + 4], s[8 * blk + 5]); pw.w = pack_bf16(s[8 * blk + 6], s[8 * blk + 7]);
         pb[blk] = __builtin_bit_cast(bf16x8, pw);
       }
-      if (__any(corr != 1.f)) {
+      if (__any(moved)) {
 #pragma unroll
         for (int t = 0; t < DT; ++t)
 #pragma unroll
           for (int i = 0; i < 4; ++i) o[t][i] *= corr;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) l_sum[i] *= corr;
       }
     }
     FE_WAIT_VMEM(0);
@@ -382,9 +388,15 @@ __global__ __launch_bounds__(256 * KG, 4) void paged_prefill_kernel(   // four w
           const bf16x8 va = __builtin_bit_cast(bf16x8, Vs[(blk * 4 + lq) * D + t * 16 + lr]);
           o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[blk], o[t], 0, 0, 0);
         }
+      // the rows' sums of probabilities as one more output tile whose "values" are all one: the matrix
+      // pipe has room, the vector pipe (16 additions and two exchanges a tile) has not; and the sum is
+      // then of the probabilities as the product above sees them, rounded to bfloat16
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) l_sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[blk], l_sum, 0, 0, 0);
     }
   }
 
+  float l_run = l_sum[0];
   if constexpr (KG == 2) {
     // the second group hands its running maximum, sum and output to the first through LDS (the
     // tiles' buffers are free now), value by value with the lanes side by side
