@@ -363,6 +363,52 @@ def test_steps_with_portions_replay_captured_graphs(name, dtype, folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_of_a_hundred_requests_with_portions_replay_captured_graphs(dtype, folders):
+    """Steps of more than 64 requests that hold prompt portions beside decoded tokens are captured
+    too: 90 requests, ten of which bring portions of 5 tokens in every step while the others bring
+    one token each; the same shape comes six times.  The attention kernels then find their work
+    among more sequences than a wave has lanes."""
+    name = "C"
+    config, weights = TINY[name], folder_weights(folders[name])
+    count = 90
+    lengths = tuple(31 + (3 * i) % 11 if i < 10 else 12 + (7 * i) % 9 for i in range(count))
+    requests = ru.make_requests(config, 43, lengths)
+    names = list(requests)
+    want = {k: plain.forward(weights, config, v) for k, v in requests.items()}
+    _, model = load_model(folders[name], dtype=dtype, device=DEV)
+    runner = ModelRunner(model, block_size=16, block_capacity=3 * count + 8, num_state_slots=count)
+    at = {}
+    for first in range(0, count, 45):
+        chunk = names[first:first + 45]
+        for k in chunk:
+            runner.begin(k)
+        # everything but the part that the six steps below bring
+        runner.step([StepEntry(k, requests[k][:len(requests[k]) - (30 if names.index(k) < 10 else 6)], []) for k in chunk])
+        for k in chunk:
+            at[k] = len(requests[k]) - (30 if names.index(k) < 10 else 6)
+    worst = 0.0
+    scale = max(float(w.abs().max()) for w in want.values())
+    bound = 1e-4 * scale + 1e-5 if dtype == "float32" else ru.BF16_FRACTION * scale
+    for step in range(6):
+        entries = []
+        for i, k in enumerate(names):
+            size = 5 if i < 10 else 1
+            entries.append(StepEntry(k, requests[k][at[k]:at[k] + size], list(range(size))))
+        logits = runner.step(entries).cpu()
+        row = 0
+        for e in entries:
+            for j in range(len(e.tokens)):
+                worst = max(worst, float((logits[row + j] - want[e.request_id][at[e.request_id] + j]).abs().max()))
+            row += len(e.tokens)
+            at[e.request_id] += len(e.tokens)
+    assert runner.portion_graph_replays >= 3
+    assert worst <= bound, f"{worst:.3e} > {bound:.3e}"
+    for k in names:
+        runner.end(k)
+    assert runner.cache.allocated_pages == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_first_tokens_of_a_sequence(name, dtype, folders):
     """Position 0 alone, then 1, 2, 3: the shortest contexts, one page, first slots."""
