@@ -26,6 +26,7 @@
 //   and receives D[m = 4*(l / 16) + i][n = l % 16]: four neighbouring output columns of one row
 //   of x, which leave as one 8-byte store.
 #include "common.h"
+#include <algorithm>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
@@ -79,10 +80,14 @@ __device__ __forceinline__ float silu_times(float g, float u) { return g / (1.f 
 // the lanes that a 16-byte read serves in one cycle then hit different bank groups.  A wave's load
 // instruction fills 64 consecutive 16-byte units (8 rows); which chunk of memory a lane asks for is
 // what places the chunks.
-template <int MT, int NG, int RW, int CW, int STAGES, int R, int D, int OCC>
-__global__ __launch_bounds__(64 * RW * CW, OCC) void gemm_gated_kernel(
+//
+// One tile: block `block_id` of a region of `col_blocks` column blocks x `row_tiles` row tiles whose
+// first column is `first_col` (a launch is one region, or two with tiles of different widths).
+template <int MT, int NG, int RW, int CW, int STAGES, int R, int D>
+__device__ __forceinline__ void gated_tile(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ out, int M, int N,
-    int K, long long ldw, long long ldo, long long up_offset, int col_blocks, int row_tiles) {
+    int K, long long ldw, long long ldo, long long up_offset, int block_id, int col_blocks, int row_tiles,
+    int first_col) {
   constexpr int THREADS = 64 * RW * CW;
   constexpr int ROWS = MT * 16 * RW;                 // rows of x a block holds
   constexpr int NF = 2 * NG;                         // weight operands a wave holds: NG gate tiles, then their NG up tiles
@@ -103,11 +108,11 @@ __global__ __launch_bounds__(64 * RW * CW, OCC) void gemm_gated_kernel(
   const int wave_row = wave / CW, wave_col = wave % CW;
   // Block id b runs on XCD b % 8.  The row tiles of one column block read the same weight rows:
   // they get neighbouring ids on one XCD, so that the second tile finds the rows in that XCD's L2.
-  const int group = blockIdx.x / (8 * row_tiles), within = blockIdx.x % (8 * row_tiles);
+  const int group = block_id / (8 * row_tiles), within = block_id % (8 * row_tiles);
   const int col_block = group * 8 + within % 8;
   const int row_tile = within / 8;
   if (col_block >= col_blocks) return;
-  const int col0 = (col_block * CW + wave_col) * 16 * NG;
+  const int col0 = first_col + (col_block * CW + wave_col) * 16 * NG;
   const int m0 = row_tile * ROWS;
 
   // x: unit u = tid + THREADS * i of a stage is position u % 8 of row u / 8 and holds the row's chunk
@@ -251,7 +256,7 @@ __global__ __launch_bounds__(64 * RW * CW, OCC) void gemm_gated_kernel(
   asm volatile("" : "+v"(tid_again));
   const int lr_out = tid_again & 15, lq_out = (tid_again & 63) >> 4;
   const int wave_row_out = (tid_again >> 6) / CW, wave_col_out = (tid_again >> 6) % CW;
-  const int col0_out = (col_block * CW + wave_col_out) * 16 * NG;
+  const int col0_out = first_col + (col_block * CW + wave_col_out) * 16 * NG;
 #pragma unroll
   for (int g = 0; g < NG; ++g) {
     const int col = col0_out + g * 16 + lq_out * 4;
@@ -277,27 +282,54 @@ __global__ __launch_bounds__(64 * RW * CW, OCC) void gemm_gated_kernel(
   }
 }
 
-template <int MT, int NG, int RW, int CW, int STAGES, int R, int D, int OCC = 1>
+template <int MT, int NG, int RW, int CW, int STAGES, int R, int D>
+__global__ __launch_bounds__(64 * RW * CW, 1) void gemm_gated_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ out, int M, int N,
+    int K, long long ldw, long long ldo, long long up_offset, int col_blocks, int row_tiles) {
+  gated_tile<MT, NG, RW, CW, STAGES, R, D>(x, w, out, M, N, K, ldw, ldo, up_offset, blockIdx.x, col_blocks, row_tiles, 0);
+}
+
+// Tiles of 256 x 128 for as many columns as fill whole rounds of one block a CU, tiles of 256 x 64 for
+// the columns that are left: the last, partly filled round then takes two thirds of a round's time
+// instead of a whole one (2,048 rows x 9,728 columns: 608 wide tiles are 2.4 rounds of 256 CUs; 512
+// wide and 192 narrow ones are 2 + 0.66).  The blocks of the wide tiles come first.
+__global__ __launch_bounds__(256, 1) void gemm_gated_mixed_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ out, int M, int N,
+    int K, long long ldw, long long ldo, long long up_offset, int wide_blocks, int wide_col_blocks,
+    int narrow_col_blocks, int row_tiles) {
+  if ((int)blockIdx.x < wide_blocks)
+    gated_tile<16, 2, 1, 4, 4, 3, 4>(x, w, out, M, N, K, ldw, ldo, up_offset, blockIdx.x, wide_col_blocks, row_tiles, 0);
+  else
+    gated_tile<16, 1, 1, 4, 4, 4, 8>(x, w, out, M, N, K, ldw, ldo, up_offset, blockIdx.x - wide_blocks, narrow_col_blocks,
+                                     row_tiles, wide_col_blocks * 128);
+}
+
+// The kernels' loads are waited for by hand, on registers that the compiler must leave alone
+// meanwhile: a build that spills registers to scratch memory would move values that are still in
+// flight (and its scratch accesses would be loads that the waits do not count).  Such a build is
+// never launched.  Also raises the kernel's LDS limit.  0: not yet asked, 1: fit, -1: refused.
+static int fit_to_launch(const void* kernel, size_t lds_bytes, int* checked) {
+  if (*checked == 0) {
+    hipFuncAttributes attributes;
+    if (hipFuncGetAttributes(&attributes, kernel) != hipSuccess) return FE_LAUNCH_FAILED;
+    if (attributes.localSizeBytes != 0) { *checked = -1; return FE_BAD_ARGUMENT; }
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+      return FE_LAUNCH_FAILED;
+    *checked = 1;                 // (a race here only repeats the calls)
+  }
+  return *checked < 0 ? FE_BAD_ARGUMENT : FE_OK;
+}
+
+template <int MT, int NG, int RW, int CW, int STAGES, int R, int D>
 static int launch_gated(const void* x, const void* w, void* out, int M, int N, int K, long long ldw, long long ldo,
                         hipStream_t stream) {
   constexpr int rows = MT * 16 * RW;
   constexpr size_t lds_bytes = (size_t)STAGES * rows * 128;
-  static_assert(lds_bytes * OCC <= 160 * 1024, "LDS of a CU");
-  static int checked = 0;            // 0: not yet, 1: fit to launch, -1: refused (a race here only repeats the calls)
-  auto kernel = gemm_gated_kernel<MT, NG, RW, CW, STAGES, R, D, OCC>;
-  if (checked == 0) {
-    // The kernel's loads are waited for by hand, on registers that the compiler must leave alone
-    // meanwhile: a build that spills registers to scratch memory would move values that are still
-    // in flight (and its scratch accesses would be loads that the waits do not count).  Such a
-    // build is never launched.
-    hipFuncAttributes attributes;
-    if (hipFuncGetAttributes(&attributes, (const void*)kernel) != hipSuccess) return FE_LAUNCH_FAILED;
-    if (attributes.localSizeBytes != 0) { checked = -1; return FE_BAD_ARGUMENT; }
-    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-      return FE_LAUNCH_FAILED;
-    checked = 1;
-  }
-  if (checked < 0) return FE_BAD_ARGUMENT;
+  static_assert(lds_bytes <= 160 * 1024, "LDS of a CU");
+  static int checked = 0;
+  auto kernel = gemm_gated_kernel<MT, NG, RW, CW, STAGES, R, D>;
+  const int fit = fit_to_launch((const void*)kernel, lds_bytes, &checked);
+  if (fit != FE_OK) return fit;
   const int col_blocks = (N + CW * 16 * NG - 1) / (CW * 16 * NG);
   const int row_tiles = (M + rows - 1) / rows;
   const long long blocks = (long long)((col_blocks + 7) / 8) * 8 * row_tiles;
@@ -307,11 +339,40 @@ static int launch_gated(const void* x, const void* w, void* out, int M, int N, i
   return fe_check_launch();
 }
 
+#define FE_CUS 256
+// Wide tiles alone, or wide tiles for whole rounds and narrow ones for the rest, whichever takes fewer
+// rounds (a round of narrow tiles counted as two thirds of a round of wide ones: measured).
+static int launch_gated_rounds(const void* x, const void* w, void* out, int M, int N, int K, long long ldw, long long ldo,
+                               hipStream_t stream) {
+  const int row_tiles = (M + 255) / 256;
+  const int all_wide = (N + 127) / 128;
+  const long long tiles = (long long)row_tiles * all_wide;
+  const int wide_cols = (int)std::min<long long>(all_wide, (tiles / FE_CUS) * FE_CUS / row_tiles);   // column blocks of the whole rounds
+  const int narrow_cols = (N - wide_cols * 128 + 63) / 64;
+  const double plain = (double)((tiles + FE_CUS - 1) / FE_CUS);
+  const double mixed = (double)(((long long)wide_cols * row_tiles + FE_CUS - 1) / FE_CUS) +
+                       0.67 * (double)(((long long)narrow_cols * row_tiles + FE_CUS - 1) / FE_CUS);
+  if (wide_cols == 0 || narrow_cols <= 0 || mixed >= plain)
+    return launch_gated<16, 2, 1, 4, 4, 3, 4>(x, w, out, M, N, K, ldw, ldo, stream);
+  constexpr size_t lds_bytes = (size_t)4 * 256 * 128;
+  static int checked = 0;
+  const int fit = fit_to_launch((const void*)gemm_gated_mixed_kernel, lds_bytes, &checked);
+  if (fit != FE_OK) return fit;
+  const long long wide_blocks = (long long)((wide_cols + 7) / 8) * 8 * row_tiles;
+  const long long narrow_blocks = (long long)((narrow_cols + 7) / 8) * 8 * row_tiles;
+  if (wide_blocks + narrow_blocks > 0x7fffffffLL) return FE_BAD_ARGUMENT;
+  gemm_gated_mixed_kernel<<<(unsigned)(wide_blocks + narrow_blocks), 256, lds_bytes, stream>>>(
+      (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)out, M, N, K, ldw, ldo, (long long)N * ldw, (int)wide_blocks, wide_cols,
+      narrow_cols, row_tiles);
+  return fe_check_launch();
+}
+
 // x [M, K] bf16 contiguous, K a multiple of 64; w [2 N, K] bf16 with row stride ldw (a multiple of 8),
 // gate rows first; out [M, N] bf16 with row stride ldo: out = silu(x gate^T) * (x up^T), float32 sums.
 // shape: which tile a block of four waves takes (rows of x x output columns):
 //   0: 256 x 64, waves of 256 rows x 16 columns     1: 256 x 128, waves of 256 rows x 32 columns
 //   2: 128 x 64, waves of 128 rows x 16 columns
+//   3: tiles of 256 x 128 for the columns that fill whole rounds of one block a CU, 256 x 64 for the rest
 // The weight is read once per row tile.  Both operands must be smaller than 2^32 elements.
 // FE_BAD_ARGUMENT also if the library was built with registers spilled to scratch memory (see
 // launch_gated): the kernel then never runs.
@@ -325,6 +386,7 @@ extern "C" int fe_gemm_gated(const void* x, const void* w, void* out, int M, int
     case 0: return launch_gated<16, 1, 1, 4, 4, 4, 8>(x, w, out, M, N, K, ldw, ldo, stream);
     case 1: return launch_gated<16, 2, 1, 4, 4, 3, 4>(x, w, out, M, N, K, ldw, ldo, stream);
     case 2: return launch_gated<8, 1, 1, 4, 6, 4, 8>(x, w, out, M, N, K, ldw, ldo, stream);
+    case 3: return launch_gated_rounds(x, w, out, M, N, K, ldw, ldo, stream);
   }
   return FE_BAD_ARGUMENT;
 }

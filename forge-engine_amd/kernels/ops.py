@@ -512,11 +512,27 @@ def _gate_block_columns(columns: int) -> int:
     return max((32, 40, 48, 56, 64), key=lambda width: (round(fill(width), 3), width))
 
 
+# The gate/up product with its SwiGLU ending in one kernel (`fe_gemm_gated`, tiles of 256 rows of x in LDS)
+# against the matrix library followed by `fe_swiglu`, microseconds at Qwen3-4B's widths (K = 2560, 9728 columns):
+# 1,024 rows 134 / 126, 1,536: 157 / 148, 2,048: 199 / 224, 2,560: 264 / 310, 3,072: 297 / 272, 4,096: 377 / 438,
+# 8,192: 793 / 755; at K = 4096 (12,288 columns) the library wins at every row count but one (2,048: 329 / 306,
+# 4,096: 683 / 590).  So: a short K, and the row counts of a prompt portion of 2,048 to 4,096 tokens.
+GATED_TILE_MIN_ROWS = 2048
+GATED_TILE_MAX_ROWS = 4096
+GATED_TILE_MAX_K = 3072
+
+
 def linear_swiglu(x: Tensor, gate_up_weight: Tensor) -> Tensor:
     """silu(x Wg^T) * (x Wu^T) for the fused weight [2I, K] (gate rows first)."""
     _gpu(x, "x")
     _gpu(gate_up_weight, "gate_up_weight")
     rows = x.shape[0]
+    if (GATED_TILE_MIN_ROWS <= rows <= GATED_TILE_MAX_ROWS and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16
+            and x.is_contiguous() and x.shape[1] % 64 == 0 and x.shape[1] <= GATED_TILE_MAX_K and gate_up_weight.shape[0] % 2 == 0
+            and gate_up_weight.dim() == 2 and gate_up_weight.stride(1) == 1 and gate_up_weight.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and gate_up_weight.data_ptr() % 16 == 0
+            and gate_up_weight.shape[0] * gate_up_weight.stride(0) < 2 ** 32 and rows * x.shape[1] < 2 ** 32):
+        return gemm_gated(x, gate_up_weight, shape=3)
     to_library = (2 <= rows <= SKINNY_MAX_ROWS and gate_up_weight.shape[0] > GATE_LIBRARY_WEIGHT_ROWS
                   and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16)
     paired_fits = (rows <= MID_ROWS and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16

@@ -50,7 +50,7 @@ class SwiGLU(FeedForward):
         return ops.linear_update(act, self.down_weight, stream=stream)   # the update stays float32 for the residual sum
 
     def kernel_libraries(self):
-        return {"rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
+        return {"rowwise", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide", "gemm_tile"}
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

@@ -1240,6 +1240,23 @@ def test_long_portions_at_the_large_widths(dtype, wide_folder, tmp_path):
     ru.compare(got, want, dtype)
 
 
+def test_a_portion_of_two_thousand_tokens_at_the_large_widths(wide_folder, tmp_path):
+    """A prompt of 2,300 tokens fed as 2,100 + 200 at the widths of the large model, bfloat16: the row
+    count at which the gate/up product runs in the kernel that keeps tiles of x in LDS (wide tiles for
+    whole rounds, narrow ones for the rest, a last row tile that is partly empty), the prefill attention
+    walks 33 key tiles, and the second portion reads 2,100 cached keys.  Logits at four positions."""
+    folder, config, weights = wide_folder
+    tokens = ru.make_requests(config, 75, (2300,))["r0"]
+    trace = ru.TraceBuilder(False)
+    trace.step([("r0", tokens[:2100])], want_all=False)
+    trace.step([("r0", tokens[2100:])], end=["r0"], want_all=False)
+    got = ru.run_trace(folder, "bfloat16", trace, tmp_path, block_size=16)
+    positions = [2099, 2299]
+    want = {("r0", p): row for p, row in zip(positions, plain.forward(weights, config, tokens, rows=positions))}
+    assert set(got) == set(want)
+    ru.compare(got, want, "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_scheduler_with_sixty_four_rows_at_the_large_widths(dtype, wide_folder):
     """Forty requests through the scheduler at its largest batch (64 requests a step, 256 tokens):

@@ -767,7 +767,7 @@ def test_gemm_wide_stores_and_gates(ops, m, n, k):
         ops.gemm_wide(x.to(DEV), w.to(DEV), "swiglu", 1, 16, 64)        # the two-tile gate ending takes tiles of 64 and 128 rows
 
 
-@pytest.mark.parametrize("shape", [0, 1, 2])
+@pytest.mark.parametrize("shape", [0, 1, 2, 3])
 @pytest.mark.parametrize("m", [1, 70, 256, 300, 513])
 @pytest.mark.parametrize("inter,k", [(9728, 2560), (200, 192), (1003, 320), (64, 64)])
 def test_gemm_gated_tile(ops, shape, m, inter, k):
@@ -838,6 +838,15 @@ def test_linear_swiglu_routes_by_rows(ops, monkeypatch):
     assert taken[-1] == "fe_swiglu", taken
     y = x.float() @ long_k.float().t()
     torch.testing.assert_close(got, y[:, :40] / (1 + torch.exp(-y[:, :40])) * y[:, 40:], atol=2e-2, rtol=2e-2)
+    # 2,048 to 4,096 rows at a K of up to 3,072: the product that keeps tiles of x in LDS and forms the ending itself
+    for rows, k, name in ((2047, 256, "fe_swiglu"), (2048, 256, "fe_gemm_gated"), (4096, 256, "fe_gemm_gated"), (4097, 256, "fe_swiglu"),
+                          (2048, 4096, "fe_swiglu")):
+        weight = rand(g, 2 * 72, k, dtype=torch.bfloat16, scale=0.05)
+        x = rand(g, rows, k, dtype=torch.bfloat16)
+        taken.clear()
+        got = ops.linear_swiglu(x.to(DEV), weight.to(DEV)).cpu().float()
+        assert taken[-1] == name, (rows, k, taken)
+        torch.testing.assert_close(got, refs.linear_swiglu(x, weight).float(), atol=2e-2, rtol=2e-2)
 
 
 def test_gemm_wide_refuses_and_routes(ops, monkeypatch):
