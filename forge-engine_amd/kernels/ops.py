@@ -666,6 +666,7 @@ def decode_splits(num_decode: int, kv_heads: int, max_ctx: int) -> int:
 
 
 PREFILL_KEY_GROUPS = 0         # 0: the prefill attention launch chooses its blocks' key groups (1 or 2 force them)
+PREFILL_ROW_SETS = 0           # 0: ... and how many sets of 16 query rows a wave takes (1 or 2 force them)
 GENERIC_TARGET_BLOCKS = 512    # blocks the general attention kernel aims at before it stops cutting the keys into runs
 
 
@@ -775,7 +776,8 @@ def paged_attention(q: Tensor, key_pages: Tensor, value_pages: Tensor, out: Tens
               _ptr(key_pages), _ptr(value_pages), _ptr(out), c_longlong(out.stride(0)), _ptr(cu_q),
               _ptr(ctx_len), _ptr(block_table), c_int(block_table.stride(0)), c_int(num_seqs),
               c_int(max_q_len), c_int(kv_heads), c_int(groups), c_int(head_dim), c_int(block_size),
-              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(PREFILL_KEY_GROUPS), c_int(tokens), _stream())
+              c_int(num_blocks), c_int(window or 0), c_float(scale), c_int(PREFILL_KEY_GROUPS), c_int(PREFILL_ROW_SETS),
+              c_int(tokens), _stream())
     # whatever the two fast kernels did not take: single tokens go to the vector-ALU decode kernel where
     # it can read four elements at a time, the rest to the general kernel
     single_left = any_single and not fast_decode

@@ -1380,9 +1380,12 @@ def test_decode_attention_that_prepares_ignores_what_unowned_slots_hold(ops, win
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [
     (8, 2, 128, 16), (5, 5, 64, 16), (12, 1, 128, 32), (3, 3, 64, 64),
 ])
-def test_prefill_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size):
+@pytest.mark.parametrize("row_sets", [1, 2])
+def test_prefill_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size, row_sets, monkeypatch):
     """The matrix-core kernel for portions of prompts: whole prompts, portions with context already
-    cached, lengths that are no multiple of the tile, beside single tokens in the same batch."""
+    cached, lengths that are no multiple of the tile, beside single tokens in the same batch; with
+    blocks of 64 and of 128 query rows."""
+    monkeypatch.setattr(ops, "PREFILL_ROW_SETS", row_sets)
     g = torch.Generator().manual_seed(40)
     seqs = [(0, 130), (70, 1), (13, 9), (0, 2), (200, 65), (63, 64), (5, 1), (0, 64)]
     q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
@@ -1397,12 +1400,14 @@ def test_prefill_attention_kernel(ops, q_heads, kv_heads, head_dim, block_size):
 
 
 @pytest.mark.parametrize("num_seqs", [40, 64, 65, 130])
-def test_prefill_attention_kernel_places_every_tile(ops, num_seqs):
-    """The kernel's grid holds a place for every 64-row tile there may be (the host knows only the
+@pytest.mark.parametrize("row_sets", [1, 2])
+def test_prefill_attention_kernel_places_every_tile(ops, num_seqs, row_sets, monkeypatch):
+    """The kernel's grid holds a place for every 64-row (or 128-row) tile there may be (the host knows only the
     step's tokens and sequences) and every block finds its sequence and tile on the device: up to 64
     sequences by a search with a lane a sequence, more one after the other.  Sequences of every
     kind side by side: empty ones (a captured step pads with them), single tokens, one to four tiles,
     with and without cached context."""
+    monkeypatch.setattr(ops, "PREFILL_ROW_SETS", row_sets)
     g = torch.Generator().manual_seed(50 + num_seqs)
     lengths = torch.randint(0, 7, (num_seqs,), generator=g).tolist()
     seqs = []
@@ -1426,12 +1431,14 @@ def test_prefill_attention_kernel_places_every_tile(ops, num_seqs):
 @pytest.mark.parametrize("window", [None, 100, 700])
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size", [(8, 2, 128, 16), (6, 3, 64, 32)])
 @pytest.mark.parametrize("key_groups", [1, 2])
-def test_prefill_attention_kernel_long_walks(ops, q_heads, kv_heads, head_dim, block_size, window, key_groups, monkeypatch):
+@pytest.mark.parametrize("row_sets", [1, 2])
+def test_prefill_attention_kernel_long_walks(ops, q_heads, kv_heads, head_dim, block_size, window, key_groups, row_sets, monkeypatch):
     """Launches that leave the chip underfilled take blocks of two key groups that walk every
     other tile and merge at the end: walks of one tile (the second group idle), of an odd and an
     even number of tiles, behind a long context, beside single tokens; with unowned slots
-    poisoned.  Both kinds of block, forced in turn."""
+    poisoned.  Every kind of block (one or two key groups, 64 or 128 rows), forced in turn."""
     monkeypatch.setattr(ops, "PREFILL_KEY_GROUPS", key_groups)
+    monkeypatch.setattr(ops, "PREFILL_ROW_SETS", row_sets)
     g = torch.Generator().manual_seed(45)
     seqs = [(0, 300), (500, 257), (70, 1), (3, 2), (1000, 64), (0, 64), (61, 67)]
     q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, block_size,
@@ -1449,13 +1456,15 @@ def test_prefill_attention_kernel_long_walks(ops, q_heads, kv_heads, head_dim, b
 
 
 @pytest.mark.parametrize("key_groups", [1, 2])
+@pytest.mark.parametrize("row_sets", [1, 2])
 @pytest.mark.parametrize("seqs,q_heads,kv_heads,head_dim", [
     ([(0, 2048)], 4, 2, 128), ([(0, 8192)], 2, 1, 128), ([(0, 1024)] * 8, 4, 2, 64), ([(6000, 2048), (0, 1)], 2, 1, 64),
 ])
-def test_prefill_attention_kernel_at_the_lengths_of_the_benchmarks(ops, seqs, q_heads, kv_heads, head_dim, key_groups, monkeypatch):
+def test_prefill_attention_kernel_at_the_lengths_of_the_benchmarks(ops, seqs, q_heads, kv_heads, head_dim, key_groups, row_sets, monkeypatch):
     """Whole prompts of 2,048 and 8,192 tokens, eight of 1,024, and a portion of 2,048 behind 6,000
-    cached tokens: walks of up to 128 key tiles, with blocks of one and of two key groups."""
+    cached tokens: walks of up to 128 key tiles, with blocks of one and of two key groups, of 64 and of 128 rows."""
     monkeypatch.setattr(ops, "PREFILL_KEY_GROUPS", key_groups)
+    monkeypatch.setattr(ops, "PREFILL_ROW_SETS", row_sets)
     g = torch.Generator().manual_seed(46)
     q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, q_heads, kv_heads, head_dim, 16,
                                                 extra_width=2 * kv_heads * head_dim)
@@ -1471,7 +1480,9 @@ def test_prefill_attention_kernel_at_the_lengths_of_the_benchmarks(ops, seqs, q_
 
 
 @pytest.mark.parametrize("window", [1, 7, 64, 100])
-def test_prefill_attention_kernel_window(ops, window):
+@pytest.mark.parametrize("row_sets", [1, 2])
+def test_prefill_attention_kernel_window(ops, window, row_sets, monkeypatch):
+    monkeypatch.setattr(ops, "PREFILL_ROW_SETS", row_sets)
     g = torch.Generator().manual_seed(41)
     seqs = [(0, 150), (90, 40), (3, 2)]
     q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, seqs, 4, 2, 64, 16)
@@ -1482,9 +1493,11 @@ def test_prefill_attention_kernel_window(ops, window):
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
 
 
-def test_prefill_attention_far_key_and_tile_edges(ops):
+@pytest.mark.parametrize("row_sets", [1, 2])
+def test_prefill_attention_far_key_and_tile_edges(ops, row_sets, monkeypatch):
     """A query late in a long prompt whose score for one early key stands far out: the key is put at
     the first and last slot of a page and of a 64-key tile in turn."""
+    monkeypatch.setattr(ops, "PREFILL_ROW_SETS", row_sets)
     g = torch.Generator().manual_seed(42)
     head_dim, block_size, length = 128, 16, 600
     q, kp, vp, cu, ctx, table = _attention_case(g, torch.bfloat16, [(0, length)], 2, 1, head_dim, block_size)
