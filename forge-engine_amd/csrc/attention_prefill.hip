@@ -456,16 +456,17 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
   // compiler, left to itself, requests four fragments and waits for all that is under way).  A lane's
   // address is a part that the lane keeps (for the keys one for each step c: the swizzle mixes c in) plus
   // a multiple of 256 bytes that is a constant of the instruction.
-  constexpr int AHEAD = 3, RING = 4;
+  constexpr int AHEAD = 3, RING = AHEAD + 1;       // (five ahead in the blocks of 128 rows: no faster)
   unsigned int key_at[KC], value_at;
 #pragma unroll
   for (int c = 0; c < KC; ++c) key_at[c] = (unsigned int)((krow * CH + ((c * 4 + lq) ^ key_swizzle(krow, CH))) * 16);
   value_at = (unsigned int)((lq * D + lr) * 16);
   auto lds_address = [](const uintx4* p) { return (unsigned int)(size_t)(const __attribute__((address_space(3))) char*)p; };
   auto wait_ring = [&](uintx4& v, int pending) {
-    if (pending >= 3) lds_arrived<3>(v); else if (pending == 2) lds_arrived<2>(v); else if (pending == 1) lds_arrived<1>(v); else lds_arrived<0>(v);
+    if (pending >= 5) lds_arrived<5>(v); else if (pending == 4) lds_arrived<4>(v); else if (pending == 3) lds_arrived<3>(v);
+    else if (pending == 2) lds_arrived<2>(v); else if (pending == 1) lds_arrived<1>(v); else lds_arrived<0>(v);
   };
-  static_assert(AHEAD <= 3, "wait_ring");
+  static_assert(AHEAD <= 5, "wait_ring");
   auto scores_ahead = [&](const uintx4* Kt, floatx4 (&st)[RM][2][2]) {
     constexpr int FRAGMENTS = 4 * KC;                 // step c outermost
     const unsigned int base = lds_address(Kt);
