@@ -14,7 +14,7 @@ from torch import Tensor
 from ..cache import CacheCapacityError, CacheManager, CacheView, plan_groups
 from ..kernels import library, ops
 from ..models.decoder import DecoderModel
-from .batch import StepBatch, StepEntry, build_batch, static_batch, static_batch_size
+from .batch import StepBatch, StepEntry, build_batch, static_batch, static_batch_size, token_input_places, token_input_values
 
 GRAPH_MAX_REQUESTS = 256     # steps of up to this many requests replay a captured graph
 GRAPH_TABLE_STEP = 64        # block-table widths of graphs are multiples of this many pages
@@ -38,9 +38,10 @@ class _DecodeGraph:
     rows are rewritten only when a request's table changed (a request that ended and began again
     under the same name holds another lease and other pages)."""
 
-    def __init__(self, num_seqs: int, widths, device) -> None:
+    def __init__(self, num_seqs: int, widths, device, token_inputs=None) -> None:
         n = num_seqs
-        size = static_batch_size(n, widths)
+        size = static_batch_size(n, widths, token_inputs=token_inputs)
+        self.inputs_at = token_input_places(n, widths, n, n, token_inputs)
         self.host = torch.empty(size, dtype=torch.int32).pin_memory()
         self.dev = torch.zeros(size, dtype=torch.int32, device=device)
         self.np = self.host.numpy()
@@ -62,9 +63,17 @@ class _DecodeGraph:
         self.batch = None
         self.copied = torch.cuda.Event()   # the last upload of the host buffer
 
-    def fill(self, tokens, before, records) -> None:
+    def fill_inputs(self, entries, positions) -> None:
+        """The per-token inputs of a step of single tokens at ``positions``."""
+        n, buf = self.n, self.np
+        for name, (at, width) in self.inputs_at.items():
+            for i, entry in enumerate(entries):
+                buf[at + i * width:at + (i + 1) * width] = token_input_values(entry, name, width, int(positions[i]))
+
+    def fill(self, tokens, before, records, entries) -> None:
         n, buf = self.n, self.np
         before = np.asarray(before, dtype=np.int32)
+        self.fill_inputs(entries, before)
         buf[0:n] = tokens
         buf[n:2 * n] = before                            # positions
         buf[4 * n + 1:5 * n + 1] = before + 1            # ctx_len
@@ -97,9 +106,11 @@ class _PortionGraph:
     Sequences beyond the step's own are empty (no tokens, so every kernel skips them), wanted
     rows beyond the step's own repeat row 0 and are cut off the result."""
 
-    def __init__(self, num_tokens: int, num_seqs: int, num_wanted: int, widths, device, pad_state_slot: int = 0) -> None:
+    def __init__(self, num_tokens: int, num_seqs: int, num_wanted: int, widths, device, pad_state_slot: int = 0,
+                 token_inputs=None) -> None:
         self.pad_state_slot = pad_state_slot
-        size = static_batch_size(num_seqs, widths, num_tokens, num_wanted)
+        size = static_batch_size(num_seqs, widths, num_tokens, num_wanted, token_inputs)
+        self.inputs_at = token_input_places(num_seqs, widths, num_tokens, num_wanted, token_inputs)
         self.host = torch.empty(size, dtype=torch.int32).pin_memory()
         self.dev = torch.zeros(size, dtype=torch.int32, device=device)
         self.np = self.host.numpy()
@@ -131,6 +142,8 @@ class _PortionGraph:
             for place in entry.want:
                 want[rows] = at + place
                 rows += 1
+            for name, (first, width) in self.inputs_at.items():
+                buf[first + at * width:first + (at + count) * width] = token_input_values(entry, name, width, before[i])
             at += count
         cu[n:] = at                                                   # the other sequences are empty
         want[rows:] = 0
@@ -173,6 +186,7 @@ class ModelRunner:
         self.device = model.ctx.device
         self.dtype = model.ctx.dtype
         self.block_size = block_size
+        self.token_inputs = model.token_inputs()     # per-token integers beside the positions, name -> width
         needs = model.cache_needs()
         groups, self._where = plan_groups(needs, model.schedule)
         self.cache = CacheManager(groups, block_size=block_size, block_capacity=block_capacity,
@@ -243,7 +257,7 @@ class ModelRunner:
         self.cache.reserve({e.request_id: before[i] + len(e.tokens) for i, e in enumerate(entries)})
         records = [self.cache.request(e.request_id) for e in entries]
         tables = [[record.tables[g] for record in records] for g in range(len(self.cache.groups))]
-        return build_batch(entries, before, [r.state_slot for r in records], tables, self.device)
+        return build_batch(entries, before, [r.state_slot for r in records], tables, self.device, token_inputs=self.token_inputs)
 
     def cache_views(self, batch: StepBatch, scratch_state: bool = False) -> list[CacheView | None]:
         """What each schedule call sees of the cache in this step.  ``scratch_state``: fixed-size
@@ -297,6 +311,7 @@ class ModelRunner:
             buf[0:n] = tokens
             buf[n:2 * n] += 1                                # positions
             buf[4 * n + 1:6 * n + 1] += 1                    # ctx_len, ctx_before
+            slot.fill_inputs(entries, buf[n:2 * n])
             slot.dev.copy_(slot.host, non_blocking=True)
             slot.copied.record(torch.cuda.current_stream(self.device))
             if device_tokens is not None:
@@ -326,17 +341,17 @@ class ModelRunner:
         if slot is None:
             if len(self._graphs) >= GRAPH_LIMIT:
                 self._graphs.pop(next(iter(self._graphs)))
-            slot = _DecodeGraph(len(entries), widths, self.device)
+            slot = _DecodeGraph(len(entries), widths, self.device, self.token_inputs)
         self._graphs[key] = slot   # most recently used last
         slot.copied.synchronize()          # the pinned buffer is free to be rewritten
-        slot.fill(tokens, before, records)
+        slot.fill(tokens, before, records, entries)
         slot.dev.copy_(slot.host, non_blocking=True)
         slot.copied.record(torch.cuda.current_stream(self.device))
         if slot.graph is None:
             bound = max(widths, default=GRAPH_TABLE_STEP) * self.block_size
             tables = [[record.tables[g] for record in records] for g in groups]
             batch = build_batch(entries, before, [r.state_slot for r in records], tables, self.device,
-                                widths=widths, static=(slot.host, slot.dev), max_ctx=bound)
+                                widths=widths, static=(slot.host, slot.dev), max_ctx=bound, token_inputs=self.token_inputs)
             views = self.cache_views(batch)
             self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()
@@ -406,7 +421,7 @@ class ModelRunner:
                 return None
             if len(self._portion_graphs) >= GRAPH_LIMIT:
                 self._portion_graphs.pop(next(iter(self._portion_graphs)))
-            slot = _PortionGraph(shape[0], shape[1], shape[2], widths, self.device, self.pad_state_slot)
+            slot = _PortionGraph(shape[0], shape[1], shape[2], widths, self.device, self.pad_state_slot, self.token_inputs)
         self._portion_graphs[key] = slot
         cache.reserve({e.request_id: n for e, n in zip(entries, after)})
         records = [cache.request(e.request_id) for e in entries]
@@ -417,7 +432,7 @@ class ModelRunner:
         if slot.graph is None:
             batch = static_batch(slot.dev, num_tokens=shape[0], num_seqs=shape[1], num_wanted=shape[2],
                                  widths=widths, max_q_len=shape[0], max_ctx=widths[0] * self.block_size if widths else 0,
-                                 num_decode=None if shape[3] else 0)
+                                 num_decode=None if shape[3] else 0, token_inputs=self.token_inputs)
             views = self.cache_views(batch)
             self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()

@@ -118,6 +118,7 @@ class _Request:
     reservation_released: bool = False
     holds_cache: bool = False
     in_flight: bool = False                            # its last sampled token is still on the device, unread
+    inputs: dict | None = None                         # per-token integers of the prompt by name (``StepEntry.inputs``)
 
     def feed(self) -> list[int]:
         return self.prompt + self.outputs
@@ -131,6 +132,19 @@ class _Request:
         if start + count <= len(prompt):
             return prompt[start:start + count]
         return prompt[start:] + self.outputs[:start + count - len(prompt)]
+
+    def next_inputs(self, count: int) -> dict | None:
+        """The per-token inputs of the next ``count`` tokens: the prompt's rows as submitted; sampled
+        tokens bring none (they get their position on every axis)."""
+        if not self.inputs:
+            return None
+        start, found = self.fed, {}
+        for name, rows in self.inputs.items():
+            width = len(rows[0]) if isinstance(rows[0], (list, tuple)) else 1
+            part = list(rows[start:start + count])
+            part.extend([position] * width for position in range(start + len(part), start + count))
+            found[name] = part
+        return found
 
     def remaining(self) -> int:
         return len(self.prompt) + len(self.outputs) + (1 if self.in_flight else 0) - self.fed
@@ -198,10 +212,12 @@ class ConcurrentGenerationEngine:
         return tokens
 
     def submit(self, prompt, *, request_id: str | None = None,
-               sampling_params: SamplingParams | None = None) -> str:
+               sampling_params: SamplingParams | None = None, inputs: dict | None = None) -> str:
         """Admit a request (token ids, or text if a tokenizer is present).
         Raises ``OverloadedError`` if the request limit is reached or, under
-        ``admission="reserve"``, its worst-case pages are not unreserved."""
+        ``admission="reserve"``, its worst-case pages are not unreserved.
+        ``inputs``: per-token integers of the prompt by name, for a model whose parts ask for
+        them (a row for every prompt token)."""
         config = self._config
         active = sum(not r.status.terminal for r in self._requests.values())
         if active >= config.max_requests:
@@ -211,6 +227,13 @@ class ConcurrentGenerationEngine:
             raise ValueError(f"duplicate request_id: {assigned}")
         params = sampling_params or self._default_params
         tokens = self._tokens_of(prompt)
+        if inputs:
+            asked = getattr(self._runner, "token_inputs", {})
+            for name, rows in inputs.items():
+                if name not in asked:
+                    raise ValueError(f"the model asks for no token input '{name}' (it asks for {sorted(asked)})")
+                if len(rows) != len(tokens):
+                    raise ValueError(f"input '{name}' must hold a row for each of the {len(tokens)} prompt tokens")
         total = len(tokens) + params.max_new_tokens
         if config.max_context is not None and total > config.max_context:
             raise OverloadedError(f"request needs {total} positions but max_context is {config.max_context}")
@@ -237,7 +260,7 @@ class ConcurrentGenerationEngine:
         self._runner.begin(assigned)
         self._admitted += 1
         self._requests[assigned] = _Request(assigned, tokens, params, seed, self._eos_ids, detokenizer,
-                                            reserved, self._admitted, holds_cache=True)
+                                            reserved, self._admitted, holds_cache=True, inputs=inputs or None)
         self._order.append(assigned)
         self._reserved = [taken + more for taken, more in zip(self._reserved, reserved)]
         return assigned
@@ -390,7 +413,7 @@ class ConcurrentGenerationEngine:
             for request, count in selected:
                 tokens = request.next_tokens(count)
                 complete = count == request.remaining()
-                entries.append(StepEntry(request.request_id, tokens, [count - 1] if complete else []))
+                entries.append(StepEntry(request.request_id, tokens, [count - 1] if complete else [], request.next_inputs(count)))
                 if complete:
                     wanted.append(request)
             try:

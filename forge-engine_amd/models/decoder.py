@@ -80,6 +80,15 @@ class DecoderModel:
             names |= part.kernel_libraries()
         return names
 
+    def token_inputs(self) -> dict[str, int]:
+        """The per-token inputs that the model's parts ask for, name -> integers a token."""
+        asked: dict[str, int] = {}
+        for part in self.parts():
+            for name, width in part.token_inputs().items():
+                if asked.setdefault(name, int(width)) != int(width):
+                    raise ValueError(f"parts ask for the token input '{name}' at widths {asked[name]} and {width}")
+        return asked
+
     def cache_needs(self) -> list[CacheNeeds]:
         """One entry per schedule call (what its mixer asks of the cache)."""
         return [self.layers[call.layer].mixer.cache_needs() for call in self.schedule]

@@ -157,6 +157,9 @@ class GroupedQueryAttention(Mixer):
                     x.dtype, q_heads=self.num_heads, kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                     rotary_dim=rotary_dim, block_size=cache.key_pages.shape[2]))
 
+    def token_inputs(self):
+        return self.position.token_inputs()
+
     def kernel_libraries(self):
         return {"qk_rope", "attention_generic", "attention_decode", "attention_prefill", "gemm_f32", "gemm_skinny", "gemm_mid", "gemm_wide"}
 

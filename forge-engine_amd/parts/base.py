@@ -100,6 +100,13 @@ class Part:
     def kernel_libraries(self) -> set[str]:
         return set()
 
+    def token_inputs(self) -> dict[str, int]:
+        """Per-token integers that this part reads beside the positions: name -> integers a token
+        (a position encoding with several axes, a token type).  A step's entries bring them
+        (``StepEntry.inputs``) and the part finds them as ``batch.inputs[name]``, int32 [T, width];
+        tokens whose entry brings none get their position on every axis."""
+        return {}
+
 
 class Embedding(Part):
     role = "embedding"

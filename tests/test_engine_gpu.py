@@ -21,6 +21,7 @@ from forge_engine_amd.config import EngineConfig, SchedulerConfig, load_model_co
 from forge_engine_amd.config.model import KeyReader, ModelConfig
 from forge_engine_amd.engine import (GenerationEngine, ModelRunner, StepEntry, build_model,
                                      engine_from_folder, load_model)
+from forge_engine_amd.engine.api import build_engine
 from forge_engine_amd.parts import (BuildContext, LayerCall, LayerSpec, Mixer, ModelPlan, ParamSpec, PartSpec,
                                     Residual, build_part)
 from forge_engine_amd.parts.base import Embedding, FeedForward
@@ -992,6 +993,186 @@ def test_routed_feed_forward_and_learned_positions_registered_from_a_test(tmp_pa
     # the routing really spreads: every expert is some token's choice
     y = plain.rms_norm(w["model.embed_tokens.weight"], w["model.norm.weight"], 1e-6)
     assert len(set((y @ w["model.layers.0.moe.router.weight"].T).argmax(-1).tolist())) == 3
+
+
+# ------------------- a third toy: a position encoding with two axes a token (per-token inputs of a step)
+
+class GridEmbedding(Embedding):
+    """h0 = E[token] + R[row] + C[column]: a learned position encoding over two axes, which a step's
+    entries bring per token (an image's patches have a row and a column; text has its position on
+    both).  The part asks for them by name; the framework carries them beside the positions."""
+
+    def __init__(self, ctx, prefix, *, vocab_size: int, hidden_size: int, max_positions: int) -> None:
+        super().__init__(ctx, prefix)
+        self.vocab_size, self.hidden_size, self.max_positions = vocab_size, hidden_size, max_positions
+        self.tables = {}
+
+    def token_inputs(self):
+        return {"grid": 2}
+
+    def param_specs(self):
+        return {self.name("weight"): ParamSpec((self.vocab_size, self.hidden_size)),
+                self.name("rows"): ParamSpec((self.max_positions, self.hidden_size)),
+                self.name("columns"): ParamSpec((self.max_positions, self.hidden_size))}
+
+    def set_param(self, name, tensor):
+        self.tables[name[len(self.prefix) + 1:]] = tensor
+
+    def forward(self, batch) -> Residual:
+        grid = batch.inputs["grid"].long()
+        h = (self.tables["weight"][batch.token_ids.long()].float() + self.tables["rows"][grid[:, 0]].float()
+             + self.tables["columns"][grid[:, 1]].float())
+        return Residual(h.contiguous())
+
+
+@dataclass(frozen=True)
+class GridConfig(ModelConfig):
+    vocab_size: int
+    hidden_size: int
+    intermediate_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    max_positions: int
+    rms_norm_eps: float
+    architecture: ClassVar[str] = "ToyGridLM"
+
+    @classmethod
+    def from_dict(cls, raw):
+        read = KeyReader(raw)
+        return cls(*(read.integer(k) for k in ("vocab_size", "hidden_size", "intermediate_size", "num_attention_heads",
+                                              "num_key_value_heads", "head_dim", "max_positions")),
+                   read.number("rms_norm_eps"))
+
+
+def grid_plan(config: GridConfig) -> ModelPlan:
+    def norm(prefix):
+        return PartSpec("rms_norm", {"size": config.hidden_size, "eps": config.rms_norm_eps}, prefix)
+
+    prefix = "model.layers.0"
+    attention = PartSpec("gqa_attention", {
+        "hidden_size": config.hidden_size, "num_heads": config.num_attention_heads,
+        "num_kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+        "position": PartSpec("none", {})}, f"{prefix}.self_attn")
+    mlp = PartSpec("swiglu", {"hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size}, f"{prefix}.mlp")
+    layer = LayerSpec("pre_norm", attention, mlp,
+                      {"input": norm(f"{prefix}.input_layernorm"), "post_mixer": norm(f"{prefix}.post_attention_layernorm")})
+    table = {"vocab_size": config.vocab_size, "hidden_size": config.hidden_size}
+    return ModelPlan(config.hidden_size, config.vocab_size,
+                     PartSpec("toy_grid", dict(table, max_positions=config.max_positions), "model.embed_tokens"),
+                     (layer,), (LayerCall(0),), norm("model.norm"), PartSpec("lm_head", dict(table, tied=False), "lm_head"))
+
+
+def grid_plain_forward(w, config: GridConfig, tokens, grid):
+    t = len(tokens)
+    eps = config.rms_norm_eps
+    heads, kv_heads, d = config.num_attention_heads, config.num_key_value_heads, config.head_dim
+    grid = torch.tensor(grid)
+    h = (w["model.embed_tokens.weight"][torch.tensor(tokens)] + w["model.embed_tokens.rows"][grid[:, 0]]
+         + w["model.embed_tokens.columns"][grid[:, 1]])
+    p = "model.layers.0"
+    x = plain.rms_norm(h, w[f"{p}.input_layernorm.weight"], eps)
+    q = (x @ w[f"{p}.self_attn.q_proj.weight"].T).view(t, heads, d).transpose(0, 1)
+    k = (x @ w[f"{p}.self_attn.k_proj.weight"].T).view(t, kv_heads, d).transpose(0, 1)
+    v = (x @ w[f"{p}.self_attn.v_proj.weight"].T).view(t, kv_heads, d).transpose(0, 1)
+    attn = plain.causal_attention(q, k, v, d ** -0.5).transpose(0, 1).reshape(t, heads * d)
+    h, y = plain.add_rms_norm(h, attn @ w[f"{p}.self_attn.o_proj.weight"].T, w[f"{p}.post_attention_layernorm.weight"], eps)
+    h = h + plain.swiglu_mlp(y, w, f"{p}.mlp")
+    return plain.rms_norm(h, w["model.norm.weight"], eps) @ w["lm_head.weight"].T
+
+
+def test_a_position_encoding_with_two_axes_registered_from_a_test(tmp_path):
+    """A part may ask for integers per token beside the positions (`token_inputs`); a step's entries
+    bring them, the batch carries them, eager and in captured graphs.  Here: rows and columns of a
+    learned two-axis position encoding.  Prompt tokens lie on a grid of their own (six to a row), the
+    tokens after the prompt bring nothing and get their position on both axes, except one request whose
+    decode steps bring explicit rows.  Against a plain whole-sequence implementation; then the same
+    through the scheduler, greedy."""
+    register_part("embedding", "toy_grid", GridEmbedding, replace=True)
+    register_architecture("ToyGridLM", GridConfig, grid_plan, replace=True)
+    raw = {"architectures": ["ToyGridLM"], "vocab_size": 61, "hidden_size": 48, "intermediate_size": 40,
+           "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 16, "max_positions": 80, "rms_norm_eps": 1e-6}
+    config = load_model_config(raw)
+    folder = write_random_model(config, 13, tmp_path, dtype=torch.float32)
+    w = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
+    for name in ("rows", "columns"):
+        w[f"model.embed_tokens.{name}"] *= 20.0           # positions that matter
+    from safetensors.torch import save_file
+    save_file({k: v.contiguous() for k, v in w.items()}, str(folder / "model.safetensors"))
+    _, model = load_model(folder, dtype="float32", device=DEV)
+    assert model.token_inputs() == {"grid": 2} and model.graph_safe
+    requests = ru.make_requests(raw, 6, (29, 40, 17))
+    tail = 8                                               # tokens fed one by one at the end
+    explicit = "r1"                                        # this request's single tokens bring rows of their own
+    assert explicit in requests
+
+    def grid_of(name, length):
+        prompt = length - tail
+        rows = [[i // 6, i % 6 + 7] for i in range(prompt)]
+        if name == explicit:
+            rows += [[70 - j, 3 * j] for j in range(tail)]
+        else:
+            rows += [[i, i] for i in range(prompt, length)]
+        return rows
+
+    grids = {k: grid_of(k, len(v)) for k, v in requests.items()}
+    want = {k: grid_plain_forward(w, config, v, grids[k]) for k, v in requests.items()}
+    # the encoding matters: with every token's position on both axes the logits differ
+    plain_positions = grid_plain_forward(w, config, requests["r0"], [[i, i] for i in range(len(requests["r0"]))])
+    assert float((plain_positions - want["r0"]).abs().max()) > 0.1 * float(want["r0"].abs().max())
+
+    runner = ModelRunner(model, block_size=4, block_capacity=30, num_state_slots=3, eager_sightings=1)
+    got = {k: [] for k in requests}
+    for k in requests:
+        runner.begin(k)
+    cut = {k: len(v) - tail for k, v in requests.items()}
+    at = {k: 0 for k in requests}
+    step = 0
+    while any(at[k] < cut[k] for k in requests):          # prompts in portions of changing size, side by side
+        entries = []
+        for k in requests:
+            size = min((7, 2, 5, 3)[(step + len(requests[k])) % 4], cut[k] - at[k])
+            if size > 0:
+                entries.append(StepEntry(k, requests[k][at[k]:at[k] + size], list(range(size)),
+                                         {"grid": grids[k][at[k]:at[k] + size]}))
+                at[k] += size
+        logits = runner.step(entries).cpu()
+        row = 0
+        for e in entries:
+            got[e.request_id].append(logits[row:row + len(e.tokens)])
+            row += len(e.tokens)
+        step += 1
+    assert runner.portion_graph_replays >= 1
+    for i in range(tail):                                  # then single tokens: captured graphs, steady steps
+        entries = [StepEntry(k, [requests[k][cut[k] + i]], [0],
+                             {"grid": [grids[k][cut[k] + i]]} if k == explicit else None) for k in requests]
+        logits = runner.step(entries).cpu()
+        for row, e in enumerate(entries):
+            got[e.request_id].append(logits[row:row + 1])
+    assert runner.graph_replays >= tail - 2 and runner.steady_steps >= 1
+    for k in requests:
+        rows = torch.cat(got[k])
+        scale = float(want[k].abs().max())
+        assert float((rows - want[k]).abs().max()) <= 1e-4 * scale + 1e-5, k
+    with pytest.raises(ValueError, match="rows of 2 integers"):
+        runner.step([StepEntry("r0", [1, 2], [], {"grid": [[1, 2]]})])
+
+    # through the scheduler: the prompt's rows come with the request, sampled tokens get their position
+    scheduler = SchedulerConfig(block_size=4, block_capacity=40, token_budget=11, max_batch_size=4, max_requests=4,
+                                prefill_chunk=6)
+    engine = build_engine(model, scheduler_config=scheduler)
+    prompts = {k: v[:cut[k]] for k, v in requests.items()}
+    ids = {k: engine.submit(prompts[k], sampling_params=SamplingParams(max_new_tokens=5),
+                            inputs={"grid": grids[k][:cut[k]]}) for k in requests}
+    engine.run_until_idle()
+    for k, request_id in ids.items():
+        tokens, grid = list(prompts[k]), list(grids[k][:cut[k]])
+        for _ in range(5):
+            tokens.append(int(grid_plain_forward(w, config, tokens, grid)[-1].argmax()))
+            grid.append([len(grid), len(grid)])           # a sampled token: its position on both axes
+        assert list(engine.request(request_id).output_token_ids) == tokens[cut[k]:], k
+    with pytest.raises(ValueError, match="asks for no token input"):
+        engine.submit([1, 2, 3], inputs={"axes": [[0], [1], [2]]})
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

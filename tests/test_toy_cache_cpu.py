@@ -265,3 +265,29 @@ def test_admission_reserves_in_every_cache_group_against_that_groups_capacity():
                                    SchedulerConfig(block_size=4, block_capacity=20))
     with pytest.raises(ValueError, match="cache groups"):
         SchedulerConfig(block_size=4, block_capacity=(20, 10, 5)).capacities(2)
+
+
+def test_per_token_inputs_lie_behind_the_block_tables():
+    """What a model's parts ask for per token (`token_inputs`) is carried in the step's one buffer,
+    name after name: rows that an entry brings, or the token's position on every axis; a captured
+    step's buffer has the same places."""
+    from forge_engine_amd.engine.batch import StepEntry, build_batch, static_batch, static_batch_size, token_input_places
+    entries = [StepEntry("a", [5, 6, 7], [2], {"grid": [[1, 2], [3, 4], [5, 6]]}),
+               StepEntry("b", [8], [0]),
+               StepEntry("c", [9, 10], [], {"kind": [7, 8]})]
+    asked = {"kind": 1, "grid": 2}
+    batch = build_batch(entries, [10, 4, 0], [0, 1, 2], [[[3, 4, 5, 6], [1, 2], [0]]], torch.device("cpu"), token_inputs=asked)
+    assert batch.inputs["grid"].tolist() == [[1, 2], [3, 4], [5, 6], [4, 4], [0, 0], [1, 1]]
+    assert batch.inputs["kind"].tolist() == [[10], [11], [12], [4], [7], [8]]
+    assert batch.positions.tolist() == [10, 11, 12, 4, 0, 1]
+    size = static_batch_size(3, [4], 6, 2, asked)
+    assert size == static_batch_size(3, [4], 6, 2) + 6 * 3
+    places = token_input_places(3, [4], 6, 2, asked)
+    assert places == {"grid": (static_batch_size(3, [4], 6, 2), 2), "kind": (static_batch_size(3, [4], 6, 2) + 12, 1)}
+    flat = torch.arange(size, dtype=torch.int32)
+    fixed = static_batch(flat, num_tokens=6, num_seqs=3, num_wanted=2, widths=[4], max_q_len=6, max_ctx=16, token_inputs=asked)
+    assert fixed.inputs["grid"].shape == (6, 2) and int(fixed.inputs["grid"][0, 0]) == places["grid"][0]
+    assert fixed.inputs["kind"].shape == (6, 1) and int(fixed.inputs["kind"][5, 0]) == size - 1
+    with pytest.raises(ValueError, match="3 rows of 2 integers"):
+        build_batch([StepEntry("a", [5, 6, 7], [], {"grid": [[1, 2], [3, 4]]})], [0], [0], [[[0]]], torch.device("cpu"), token_inputs=asked)
+    assert build_batch(entries[:2], [0, 0], [0, 1], [[[0], [1]]], torch.device("cpu")).inputs == {}
