@@ -1438,6 +1438,24 @@ def test_a_portion_of_two_thousand_tokens_at_the_large_widths(wide_folder, tmp_p
     ru.compare(got, want, "bfloat16")
 
 
+def test_a_portion_of_three_thousand_tokens_at_the_large_widths(wide_folder, tmp_path):
+    """A prompt of 3,300 tokens fed as 3,100 + 200 at the widths of the large model, bfloat16: with 32
+    query heads the first step is the size from which the prefill attention launch chooses blocks of 128
+    query rows (two sets of rows a wave, two LDS buffers) by itself, its last block a partly filled one;
+    the gate/up product runs 13 row tiles in the kernel that keeps tiles of x in LDS; the second portion
+    reads 3,100 cached keys through a table of 207 pages.  Logits at two positions."""
+    folder, config, weights = wide_folder
+    tokens = ru.make_requests(config, 76, (3300,))["r0"]
+    trace = ru.TraceBuilder(False)
+    trace.step([("r0", tokens[:3100])], want_all=False)
+    trace.step([("r0", tokens[3100:])], end=["r0"], want_all=False)
+    got = ru.run_trace(folder, "bfloat16", trace, tmp_path, block_size=16)
+    positions = [3099, 3299]
+    want = {("r0", p): row for p, row in zip(positions, plain.forward(weights, config, tokens, rows=positions))}
+    assert set(got) == set(want)
+    ru.compare(got, want, "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_scheduler_with_sixty_four_rows_at_the_large_widths(dtype, wide_folder):
     """Forty requests through the scheduler at its largest batch (64 requests a step, 256 tokens):
