@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
       const int mid = (lo + hi) >> 1;
       if (wave_total(min(tiles, mid)) <= slot) lo = mid; else hi = mid;
     }
-    const int rank = slot - wave_total(min(tiles, lo));          // among the sequences with a tile in this round
+    const int rank = slot - wave_total(min(tiles, lo));          // among the sequences that have a tile in round lo
     const unsigned long long in_round = __ballot(tiles > lo);
     const int before_me = __builtin_popcountll(in_round & ((1ull << me) - 1ull));
     const unsigned long long mine = __ballot(tiles > lo && before_me == rank);
