@@ -249,6 +249,13 @@ class ModelRunner:
             for place in entry.want:
                 if not 0 <= place < len(entry.tokens):
                     raise ValueError(f"wanted place {place} is outside the {len(entry.tokens)} tokens of '{entry.request_id}'")
+            self._check_inputs(entry)
+
+    def _check_inputs(self, entry: StepEntry) -> None:
+        for name in entry.inputs or ():
+            if name not in self.token_inputs:
+                raise ValueError(f"request '{entry.request_id}' brings the token input '{name}', which no part of the model "
+                                 f"asks for (asked for: {sorted(self.token_inputs)})")
 
     def prepare(self, entries: list[StepEntry]) -> StepBatch:
         """Lease the pages the step needs (all or none) and build its batch."""
@@ -299,6 +306,9 @@ class ModelRunner:
             tokens = [0] * len(entries)
         elif min(tokens) < 0 or max(tokens) >= vocab:
             raise ValueError(f"a token id is outside the vocabulary of {vocab}")
+        for entry in entries:
+            if entry.inputs:
+                self._check_inputs(entry)
         steady = self._steady
         if (steady is not None and steady.room > 0 and len(entries) == len(steady.ids)
                 and all(e.request_id == name for e, name in zip(entries, steady.ids))

@@ -1156,6 +1156,8 @@ def test_a_position_encoding_with_two_axes_registered_from_a_test(tmp_path):
         assert float((rows - want[k]).abs().max()) <= 1e-4 * scale + 1e-5, k
     with pytest.raises(ValueError, match="rows of 2 integers"):
         runner.step([StepEntry("r0", [1, 2], [], {"grid": [[1, 2]]})])
+    with pytest.raises(ValueError, match="no part of the model"):
+        runner.step([StepEntry("r0", [1, 2], [], {"axes": [[1], [2]]})])
 
     # through the scheduler: the prompt's rows come with the request, sampled tokens get their position
     scheduler = SchedulerConfig(block_size=4, block_capacity=40, token_budget=11, max_batch_size=4, max_requests=4,
