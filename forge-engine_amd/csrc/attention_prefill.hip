@@ -307,32 +307,9 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
     }
   };
 
-  // fragments of a tile in LDS: 16 keys (rows blk, h of the interleaved order) x 32 dims (step c) of the
-  // keys at Kt; 16 dims (tile t) x 32 keys (block blk) of the values at Vt
-  auto key_fragment = [&](const uintx4* Kt, int blk, int h, int c) -> uintx4 {
-    const int r = blk * 32 + krow + 4 * h;
-    return Kt[r * CH + ((c * 4 + lq) ^ key_swizzle(r, CH))];
-  };
-  auto value_fragment = [&](const uintx4* Vt, int t, int blk) -> uintx4 { return Vt[(blk * 4 + lq) * D + t * 16 + lr]; };
-
-  // S^T of one tile: a fragment of keys read from LDS serves the wave's RM sets of rows
-  auto scores = [&](const uintx4* Kt, floatx4 (&st)[RM][2][2]) {
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int c = 0; c < KC; ++c) {
-          const bf16x8 ka = __builtin_bit_cast(bf16x8, key_fragment(Kt, blk, h, c));
-#pragma unroll
-          for (int rm = 0; rm < RM; ++rm)
-            st[rm][blk][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                ka, qb[rm][c], c == 0 ? floatx4{0.f, 0.f, 0.f, 0.f} : st[rm][blk][h], 0, 0, 0);
-        }
-  };
-  // The softmax of one tile for one set of rows, cut into SOFTMAX_ITEMS pieces of a few instructions
-  // (so that a walk can spread them between the MFMAs of other tiles): the scores become the
-  // probabilities in place, then the second product's B operands, rounded to bfloat16.
+  // The softmax of one tile for one set of rows, in SOFTMAX_ITEMS pieces of a few instructions each:
+  // the scores become the probabilities in place, then the second product's B operands, rounded to
+  // bfloat16.
   // lane (lr = query row, lq): st[rm][blk][h][i] = score of key key_base + 32 blk + 8lq + 4h + i
   constexpr int SOFTMAX_ITEMS = 24;
   float item_mx[RM], item_m_use[RM], corr[RM];
@@ -437,21 +414,10 @@ __global__ __launch_bounds__(256 * KG, RM == 1 ? 4 : 2 / KG) void paged_prefill_
       for (int rm = 0; rm < RM; ++rm)
         l_sum[rm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, __builtin_bit_cast(bf16x8, pw[rm][blk]), l_sum[rm], 0, 0, 0);
   };
-  // O^T += V^T P^T
-  auto weighted = [&](const uintx4* Vt, uintx4 (&pw)[RM][2]) {
-#pragma unroll
-    for (int t = 0; t < DT; ++t)
-#pragma unroll
-      for (int blk = 0; blk < 2; ++blk) {
-        const bf16x8 va = __builtin_bit_cast(bf16x8, value_fragment(Vt, t, blk));
-#pragma unroll
-        for (int rm = 0; rm < RM; ++rm)
-          o[rm][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, __builtin_bit_cast(bf16x8, pw[rm][blk]), o[rm][t], 0, 0, 0);
-      }
-    row_sums(pw);
-  };
-
-  // The same two products with every fragment requested AHEAD fragments before the MFMAs that use it,
+  // The two products of a tile.  S^T: the fragment of keys (blk, h, c) holds 16 keys (rows 32 blk + 4 h +
+  // krow of the tile, the interleaved order) x 32 dims (step c) and serves the wave's RM sets of rows;
+  // O^T += V^T P^T: the fragment of values (t, blk) holds 16 dims (16 t + lr) x 32 keys (chunk 4 blk + lq).
+  // Every fragment is requested AHEAD fragments before the MFMAs that use it,
   // in an order in which the MFMAs on one accumulator stand apart, and with the waits written out (the
   // compiler, left to itself, requests four fragments and waits for all that is under way).  A lane's
   // address is a part that the lane keeps (for the keys one for each step c: the swizzle mixes c in) plus
