@@ -37,6 +37,32 @@ typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
 
 __device__ __forceinline__ float silu_times(float g, float u) { return g / (1.f + __expf(-g)) * u; }
 
+// 16 bytes from LDS byte address `at` + 2048 * STEP (sixteen rows of a stage further); nothing waits for them here
+template <int STEP>
+__device__ __forceinline__ uintx4 lds_read16(unsigned int at) {
+  uintx4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(at), "n"(STEP * 2048) : "memory");
+  return v;
+}
+// ... with a step that is a constant only once the loop around the call is unrolled
+__device__ __forceinline__ uintx4 lds_read16_step(unsigned int at, int step) {
+  switch (step) {
+#define FE_CASE(I) case I: return lds_read16<I>(at);
+    FE_CASE(0) FE_CASE(1) FE_CASE(2) FE_CASE(3) FE_CASE(4) FE_CASE(5) FE_CASE(6) FE_CASE(7)
+    FE_CASE(8) FE_CASE(9) FE_CASE(10) FE_CASE(11) FE_CASE(12) FE_CASE(13) FE_CASE(14) FE_CASE(15)
+#undef FE_CASE
+  }
+  return uintx4{0u, 0u, 0u, 0u};
+}
+// wait until at most PENDING of this wave's LDS accesses are outstanding; `v` is what the wait is for.
+// (LDS accesses finish in order.  Whatever else the compiler has under way on the same counter, its own
+// LDS stores or a scalar load, makes such a wait stricter, never weaker; and its own waits, which do not
+// know of the reads above, likewise.)
+template <int PENDING>
+__device__ __forceinline__ void lds_arrived(uintx4& v) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(PENDING));
+}
+
 // LDS holds a step of x as [row][8 chunks of 16 bytes], chunk c of row r at position c ^ (r % 8):
 // the eight lanes that a 16-byte read serves in one cycle then hit eight different bank groups.
 template <int MT, int EPI, int R, int WPB>
@@ -100,16 +126,48 @@ __global__ __launch_bounds__(64 * WPB, 2) void gemm_wide_kernel(
         *(uintx4*)&xs[stage][row][((p & 7) ^ (row & 7)) * 8] = xsrc[i];
       }
     };
+    // Tiles of 128 rows: the fragments of x (k half c, row tile mt) are requested from LDS AHEAD
+    // fragments before the MFMAs that use them, with the waits written out.  The compiler, left to
+    // itself, reads every fragment into the same registers and waits for it right there; other waves
+    // fill most of those waits (a step of 256 tokens 5.69 -> 5.63 ms with the reads ahead, of 128
+    // tokens 4.28 -> 4.21 ms), and with tiles of up to 64 rows all of them (64 rows: 4.84 against 4.87
+    // ms a decode step), so those keep the compiler's order.  A lane's address is its place in a
+    // stage's first sixteen rows (one for each k half: the swizzle mixes it in) plus a multiple of
+    // 2,048 bytes (stage and row tile) that is a constant of the instruction.
+    constexpr int FRAGMENTS = 2 * MT;
+    constexpr int AHEAD = 3, RING = AHEAD + 1;
+    const unsigned int xs_at = (unsigned int)(size_t)(const __attribute__((address_space(3))) char*)&xs[0][0][0];
+    const unsigned int a_lane[2] = {xs_at + (unsigned int)(lr * 128 + ((0 + lq) ^ (lr & 7)) * 16),
+                                    xs_at + (unsigned int)(lr * 128 + ((4 + lq) ^ (lr & 7)) * 16)};
     auto multiply = [&](int stage, const uintx4* wreg) {
+      if constexpr (MT < 8) {
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < 2; ++c) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const int row = mt * 16 + lr;
-          const bf16x8 a = *(const bf16x8*)&xs[stage][row][((c * 4 + lq) ^ (lr & 7)) * 8];
+          for (int mt = 0; mt < MT; ++mt) {
+            const int row = mt * 16 + lr;
+            const bf16x8 a = *(const bf16x8*)&xs[stage][row][((c * 4 + lq) ^ (lr & 7)) * 8];
 #pragma unroll
-          for (int f = 0; f < WF; ++f)
-            acc[f][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, wreg[f * 2 + c]), acc[f][mt], 0, 0, 0);
+            for (int t = 0; t < WF; ++t)
+              acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, wreg[t * 2 + c]), acc[t][mt], 0, 0, 0);
+          }
+        }
+      } else {
+        auto fragment = [&](int f) -> uintx4 { return lds_read16_step(a_lane[f / MT], stage * MT + f % MT); };
+        uintx4 ring[RING];
+#pragma unroll
+        for (int f = 0; f < AHEAD; ++f) ring[f] = fragment(f);
+#pragma unroll
+        for (int f = 0; f < FRAGMENTS; ++f) {
+          if (f + AHEAD < FRAGMENTS) ring[(f + AHEAD) % RING] = fragment(f + AHEAD);
+          const int pending = FRAGMENTS - 1 - f < AHEAD ? FRAGMENTS - 1 - f : AHEAD;
+          if (pending >= 3) lds_arrived<3>(ring[f % RING]); else if (pending == 2) lds_arrived<2>(ring[f % RING]);
+          else if (pending == 1) lds_arrived<1>(ring[f % RING]); else lds_arrived<0>(ring[f % RING]);
+          const bf16x8 a = __builtin_bit_cast(bf16x8, ring[f % RING]);
+          const int c = f / MT, mt = f % MT;
+#pragma unroll
+          for (int t = 0; t < WF; ++t)
+            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, wreg[t * 2 + c]), acc[t][mt], 0, 0, 0);
         }
       }
     };
