@@ -396,3 +396,21 @@ def test_detokenizer_holds_back_stop_prefixes_and_half_characters():
     assert d.push(5) == "è"
     d = IncrementalDetokenizer(WordTokenizer(), ("two STOP",))
     assert d.push(2) == "" and d.finish() == "two "   # a stop prefix is flushed when generation ends
+
+
+def test_a_requests_token_inputs_follow_its_tokens():
+    """Per-token inputs that came with a prompt are cut as the prompt is: a portion gets its rows; tokens
+    past the prompt (sampled ones, fed again after a preemption or for the first time) bring their
+    position on every axis, at the width of the prompt's rows."""
+    from forge_engine_amd.engine.scheduler import _Request
+    request = _Request("r", [5, 6, 7, 8], SamplingParams(max_new_tokens=4), 1, frozenset(), None, [0], 1,
+                       inputs={"grid": [[9, 1], [9, 2], [9, 3], [9, 4]], "kind": [7, 7, 8, 8]})
+    assert request.next_inputs(3) == {"grid": [[9, 1], [9, 2], [9, 3]], "kind": [7, 7, 8]}
+    request.fed = 3
+    request.outputs = [11, 12]
+    assert request.next_tokens(3) == [8, 11, 12]
+    assert request.next_inputs(3) == {"grid": [[9, 4], [4, 4], [5, 5]], "kind": [8, [4], [5]]}
+    request.fed = 5
+    assert request.next_inputs(1) == {"grid": [[5, 5]], "kind": [[5]]}
+    request.inputs = None
+    assert request.next_inputs(2) is None
