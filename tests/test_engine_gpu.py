@@ -1494,6 +1494,46 @@ def test_scheduler_with_sixty_four_rows_at_the_large_widths(dtype, wide_folder):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_beyond_the_reach_of_32_bit_offsets(dtype, wide_folder):
+    """A pool of a layer with more than 2**32 elements, and a request whose pages lie at its
+    far end: an offset into the pool that a kernel computed in 32 bits, signed or not, would
+    wrap and read or write another page.  The same steps in a small pool give the same logits."""
+    folder, config, _ = wide_folder
+    _, model = load_model(folder, dtype=dtype, device=DEV)
+    tokens = ru.make_requests(config, 67, (150, 40))
+    page_elements = config["num_key_value_heads"] * 16 * config["head_dim"]
+    low_pages = 2 ** 32 // page_elements + 64
+
+    def run(capacity, held):
+        runner = ModelRunner(model, block_size=16, block_capacity=capacity, num_state_slots=4)
+        taken = runner.cache.pools[0].allocate(held) if held else []
+        rows = []
+        runner.begin("a")
+        runner.begin("b")
+        rows.append(runner.step([StepEntry("a", tokens["r0"][:140], [138, 139])]))                  # a prompt whole
+        rows.append(runner.step([StepEntry("a", tokens["r0"][140:146], [5]),                        # portions together
+                                 StepEntry("b", tokens["r1"][:37], [36])]))
+        for i in range(3):                                                                          # single tokens
+            rows.append(runner.step([StepEntry("a", [tokens["r0"][146 + i]], [0]),
+                                     StepEntry("b", [tokens["r1"][37 + i]], [0])]))
+        pages = [page for name in "ab" for table in runner.cache.request(name).tables for page in table]
+        runner.end("a")
+        runner.end("b")
+        if taken:
+            runner.cache.pools[0].release(taken)
+        runner.cache.check_invariants()
+        return torch.cat([r.float().cpu() for r in rows]), pages
+
+    want, near = run(40, 0)
+    torch.cuda.empty_cache()
+    got, far = run(low_pages + 40, low_pages)
+    torch.cuda.empty_cache()
+    assert max(near) < 40 and min(far) >= low_pages and min(far) * page_elements >= 2 ** 32
+    scale = float(want.abs().max())
+    assert float((got - want).abs().max()) <= (1e-5 if dtype == "float32" else 1e-3) * scale
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_name_used_again_decodes_from_its_new_pages(dtype, folders):
     """A request ends and another begins under the same name with a table of the same length
     but other pages (a third request took the old ones meanwhile): the captured decode step
