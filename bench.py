@@ -24,6 +24,9 @@ published peak and against a streaming read measured when the program starts.
 (admission, selection, sampling and finishing included) instead of calling the
 step function directly.  ``--workload mixed`` runs requests with prompts of
 random lengths to completion through the scheduler and reports the whole job.
+``--phase check`` times nothing: it feeds one prompt of ``--prefill-tokens`` whole
+and eight more tokens one by one through the chosen model in bfloat16 and in
+32-bit, built from the same seed, and prints how far the logits lie apart.
 """
 
 from __future__ import annotations
@@ -94,7 +97,7 @@ def parse_args():
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
     parser.add_argument("--dtype", choices=("bf16", "fp32"), default="bf16")
     parser.add_argument("--points", default=None, help="other decode batch sizes to report")
-    parser.add_argument("--phase", choices=("all", "decode", "prefill", "micro"), default="all",
+    parser.add_argument("--phase", choices=("all", "decode", "prefill", "micro", "check"), default="all",
                         help="run one phase only (for profiles); the record then holds that phase alone")
     parser.add_argument("--through", choices=("step", "scheduler"), default="step",
                         help="decode by calling the step function, or through the scheduler's step()")
@@ -214,6 +217,49 @@ def micro_benchmarks() -> int:
     return 0
 
 
+def cross_check(args) -> int:
+    """The model at the benchmark's sizes in bfloat16 against the same weights in 32-bit: a
+    prompt whole (logits at a place in its middle and at its end), then eight single tokens.
+    Rounding grows slowly with the number of layers; a kernel that is wrong at these sizes
+    only (a width, a head count, a cache of this length) shows as a jump."""
+    import torch
+
+    from forge_engine_amd.config import load_model_config
+    from forge_engine_amd.engine import ModelRunner, StepEntry, random_model
+
+    chosen = MODELS[args.model]
+    raw = dict(chosen["config"])
+    full_layers = raw["num_hidden_layers"]
+    if args.layers is not None:
+        raw["num_hidden_layers"] = args.layers
+    config = load_model_config(raw)
+    prompt = args.prefill_tokens
+    generator = torch.Generator().manual_seed(args.seed)
+    tokens = torch.randint(0, config.vocab_size, (prompt + 8,), generator=generator).tolist()
+    rows = {}
+    for dtype in ("bfloat16", "float32"):
+        model = random_model(config, args.seed, dtype=dtype, device=torch.device("cuda:0"))
+        runner = ModelRunner(model, block_size=args.block_size,
+                             block_capacity=-(-(prompt + 8) // args.block_size) + 1, num_state_slots=2)
+        runner.begin("a")
+        got = [runner.step([StepEntry("a", tokens[:prompt], [prompt // 2, prompt - 1])]).float().cpu()]
+        for token in tokens[prompt:]:
+            got.append(runner.step([StepEntry("a", [token], [0])]).float().cpu())
+        rows[dtype] = torch.cat(got)
+        del runner, model
+        torch.cuda.empty_cache()
+    want, got = rows["float32"], rows["bfloat16"]
+    scale = float(want.abs().max())
+    apart = (got - want).abs().max(dim=1).values
+    print(json.dumps({
+        "check": "bfloat16 against float32", "model": chosen["label"], "layers_run": config.num_hidden_layers,
+        "layers_model": full_layers, "prompt_tokens": prompt, "rows": len(apart), "largest_logit": round(scale, 3),
+        "largest_difference": round(float(apart.max()), 4), "fraction": round(float(apart.max()) / scale, 4),
+        "argmax_agree": int((got.argmax(1) == want.argmax(1)).sum()),
+    }))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -221,6 +267,8 @@ def main() -> int:
         return 2
     if args.phase == "micro":
         return micro_benchmarks()
+    if args.phase == "check":
+        return cross_check(args)
     import torch
 
     from forge_engine_amd.config import SchedulerConfig, load_model_config
