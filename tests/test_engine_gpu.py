@@ -24,7 +24,7 @@ from forge_engine_amd.engine import (GenerationEngine, ModelRunner, StepEntry, b
 from forge_engine_amd.engine.api import build_engine
 from forge_engine_amd.parts import (BuildContext, LayerCall, LayerSpec, Mixer, ModelPlan, ParamSpec, PartSpec,
                                     Residual, build_part)
-from forge_engine_amd.parts.base import Embedding, FeedForward
+from forge_engine_amd.parts.base import Block, Embedding, FeedForward
 from forge_engine_amd.registry import register_architecture, register_part
 from forge_engine_amd.sampling import SamplingParams
 from forge_engine_amd.weights import fill_random_weights, write_random_model
@@ -1175,6 +1175,161 @@ def test_a_position_encoding_with_two_axes_registered_from_a_test(tmp_path):
         assert list(engine.request(request_id).output_token_ids) == tokens[cut[k]:], k
     with pytest.raises(ValueError, match="asks for no token input"):
         engine.submit([1, 2, 3], inputs={"axes": [[0], [1], [2]]})
+
+
+class ParallelBlock(Block):
+    """``h += mixer(norm(h)) + ffn(norm(h))``: one norm, both parts read the same rows."""
+
+    def forward(self, residual: Residual, batch, cache, writes_cache: bool = True) -> None:
+        x = self.norms["input"].forward(residual)
+        residual.add(self.mixer.forward(x, batch, cache, writes_cache))
+        residual.add(self.feed_forward.forward(x, batch))
+
+
+class SandwichBlock(Block):
+    """``h += norm_a(mixer(norm_in(h))); h += norm_b(ffn(norm_post(h)))``: a norm on what each part
+    returns as well as on what it reads."""
+
+    def normalised(self, update, norm, like):
+        inner = Residual(torch.zeros_like(like))      # an update may come as partial sums: added up here
+        inner.add(update)
+        return norm.forward(inner).float()
+
+    def forward(self, residual: Residual, batch, cache, writes_cache: bool = True) -> None:
+        x = self.norms["input"].forward(residual)
+        residual.add(self.normalised(self.mixer.forward(x, batch, cache, writes_cache), self.norms["after_mixer"], residual.h))
+        y = self.norms["post_mixer"].forward(residual)
+        residual.add(self.normalised(self.feed_forward.forward(y, batch), self.norms["after_ffn"], residual.h))
+
+
+ARRANGEMENTS = ("pre_norm", "toy_parallel", "toy_sandwich", "toy_parallel")
+ARRANGED_NORMS = {"pre_norm": ("input_layernorm", "post_attention_layernorm"), "toy_parallel": ("input_layernorm",),
+                  "toy_sandwich": ("input_layernorm", "after_mixer_norm", "post_attention_layernorm", "after_ffn_norm")}
+NORM_ROLES = {"input_layernorm": "input", "post_attention_layernorm": "post_mixer", "after_mixer_norm": "after_mixer",
+              "after_ffn_norm": "after_ffn"}
+
+
+@dataclass(frozen=True)
+class ArrangedConfig(ModelConfig):
+    vocab_size: int
+    hidden_size: int
+    intermediate_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    rms_norm_eps: float
+    rope_theta: float
+    architecture: ClassVar[str] = "ToyArrangedLM"
+
+    @classmethod
+    def from_dict(cls, raw):
+        read = KeyReader(raw)
+        return cls(*(read.integer(k) for k in ("vocab_size", "hidden_size", "intermediate_size", "num_attention_heads",
+                                              "num_key_value_heads", "head_dim")),
+                   read.number("rms_norm_eps"), read.number("rope_theta"))
+
+
+def arranged_plan(config: ArrangedConfig) -> ModelPlan:
+    def norm(prefix):
+        return PartSpec("rms_norm", {"size": config.hidden_size, "eps": config.rms_norm_eps}, prefix)
+
+    def layer(index, arrangement):
+        prefix = f"model.layers.{index}"
+        attention = PartSpec("gqa_attention", {
+            "hidden_size": config.hidden_size, "num_heads": config.num_attention_heads,
+            "num_kv_heads": config.num_key_value_heads, "head_dim": config.head_dim, "qk_norm_eps": config.rms_norm_eps,
+            "position": PartSpec("rotary", {"head_dim": config.head_dim, "theta": config.rope_theta})}, f"{prefix}.self_attn")
+        mlp = PartSpec("swiglu", {"hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size}, f"{prefix}.mlp")
+        return LayerSpec(arrangement, attention, mlp,
+                         {NORM_ROLES[name]: norm(f"{prefix}.{name}") for name in ARRANGED_NORMS[arrangement]})
+
+    layers = tuple(layer(i, a) for i, a in enumerate(ARRANGEMENTS))
+    table = {"vocab_size": config.vocab_size, "hidden_size": config.hidden_size}
+    return ModelPlan(config.hidden_size, config.vocab_size, PartSpec("token_embedding", dict(table), "model.embed_tokens"),
+                     layers, tuple(LayerCall(i) for i in range(len(layers))), norm("model.norm"),
+                     PartSpec("lm_head", dict(table, tied=False), "lm_head"))
+
+
+def arranged_plain_forward(w, config: ArrangedConfig, tokens):
+    t = len(tokens)
+    eps = config.rms_norm_eps
+    heads, kv_heads, d = config.num_attention_heads, config.num_key_value_heads, config.head_dim
+    cos, sin = plain.rotary_tables(torch.arange(t), d, config.rope_theta)
+
+    def attention(x, p):
+        q = plain.rms_norm((x @ w[f"{p}.q_proj.weight"].T).view(t, heads, d), w[f"{p}.q_norm.weight"], eps).transpose(0, 1)
+        k = plain.rms_norm((x @ w[f"{p}.k_proj.weight"].T).view(t, kv_heads, d), w[f"{p}.k_norm.weight"], eps).transpose(0, 1)
+        v = (x @ w[f"{p}.v_proj.weight"].T).view(t, kv_heads, d).transpose(0, 1)
+        out = plain.causal_attention(plain.apply_rotary(q, cos, sin), plain.apply_rotary(k, cos, sin), v, d ** -0.5)
+        return out.transpose(0, 1).reshape(t, heads * d) @ w[f"{p}.o_proj.weight"].T
+
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    for index, arrangement in enumerate(ARRANGEMENTS):
+        p = f"model.layers.{index}"
+        x = plain.rms_norm(h, w[f"{p}.input_layernorm.weight"], eps)
+        update = attention(x, f"{p}.self_attn")
+        if arrangement == "pre_norm":
+            h, y = plain.add_rms_norm(h, update, w[f"{p}.post_attention_layernorm.weight"], eps)
+            h = h + plain.swiglu_mlp(y, w, f"{p}.mlp")
+        elif arrangement == "toy_parallel":
+            h = h + update + plain.swiglu_mlp(x, w, f"{p}.mlp")
+        else:
+            h = h + plain.rms_norm(update, w[f"{p}.after_mixer_norm.weight"], eps)
+            y = plain.rms_norm(h, w[f"{p}.post_attention_layernorm.weight"], eps)
+            h = h + plain.rms_norm(plain.swiglu_mlp(y, w, f"{p}.mlp"), w[f"{p}.after_ffn_norm.weight"], eps)
+    return plain.rms_norm(h, w["model.norm.weight"], eps) @ w["lm_head.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_block_arrangements_registered_from_a_test(dtype, tmp_path):
+    """How a layer's parts and norms are arranged is a part like the others: a model whose layers
+    are the framework's arrangement, one with a single norm whose parts run side by side, and one
+    with norms behind its parts too, each chosen by name layer by layer.  Portions of changing
+    size, then single tokens through captured graphs, against a plain whole-sequence implementation."""
+    register_part("block", "toy_parallel", ParallelBlock, replace=True)
+    register_part("block", "toy_sandwich", SandwichBlock, replace=True)
+    register_architecture("ToyArrangedLM", ArrangedConfig, arranged_plan, replace=True)
+    raw = {"architectures": ["ToyArrangedLM"], "vocab_size": 83, "hidden_size": 48, "intermediate_size": 56,
+           "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 16, "rms_norm_eps": 1e-5, "rope_theta": 1e4}
+    config = load_model_config(raw)
+    folder = write_random_model(config, 19, tmp_path)
+    w = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
+    assert "model.layers.2.after_ffn_norm.weight" in w and "model.layers.1.post_attention_layernorm.weight" not in w
+    _, model = load_model(folder, dtype=dtype, device=DEV)
+    requests = ru.make_requests(raw, 8, (37, 22, 30))
+    want = {k: arranged_plain_forward(w, config, v) for k, v in requests.items()}
+    runner = ModelRunner(model, block_size=4, block_capacity=30, num_state_slots=3, eager_sightings=1)
+    got = {k: [] for k in requests}
+    for k in requests:
+        runner.begin(k)
+    tail = 9
+    cut = {k: len(v) - tail for k, v in requests.items()}
+    at = {k: 0 for k in requests}
+    step = 0
+    while any(at[k] < cut[k] for k in requests):
+        entries = []
+        for k in requests:
+            size = min((6, 2, 5, 3)[(step + len(requests[k])) % 4], cut[k] - at[k])
+            if size > 0:
+                entries.append(StepEntry(k, requests[k][at[k]:at[k] + size], list(range(size))))
+                at[k] += size
+        logits = runner.step(entries).float().cpu()
+        row = 0
+        for e in entries:
+            got[e.request_id].append(logits[row:row + len(e.tokens)])
+            row += len(e.tokens)
+        step += 1
+    for i in range(tail):
+        entries = [StepEntry(k, [requests[k][cut[k] + i]], [0]) for k in requests]
+        logits = runner.step(entries).float().cpu()
+        for row, e in enumerate(entries):
+            got[e.request_id].append(logits[row:row + 1])
+    assert runner.graph_replays >= tail - 2
+    for k in requests:
+        rows = torch.cat(got[k])
+        scale = float(want[k].abs().max())
+        bound = 1e-4 * scale + 1e-5 if dtype == "float32" else ru.BF16_FRACTION * scale
+        assert float((rows - want[k]).abs().max()) <= bound, k
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
