@@ -24,7 +24,7 @@ from forge_engine_amd.engine import (GenerationEngine, ModelRunner, StepEntry, b
 from forge_engine_amd.engine.api import build_engine
 from forge_engine_amd.parts import (BuildContext, LayerCall, LayerSpec, Mixer, ModelPlan, ParamSpec, PartSpec,
                                     Residual, build_part)
-from forge_engine_amd.parts.base import Block, Embedding, FeedForward
+from forge_engine_amd.parts.base import Block, Embedding, FeedForward, Head, Norm
 from forge_engine_amd.registry import register_architecture, register_part
 from forge_engine_amd.sampling import SamplingParams
 from forge_engine_amd.weights import fill_random_weights, write_random_model
@@ -1310,6 +1310,169 @@ def test_block_arrangements_registered_from_a_test(dtype, tmp_path):
         entries = []
         for k in requests:
             size = min((6, 2, 5, 3)[(step + len(requests[k])) % 4], cut[k] - at[k])
+            if size > 0:
+                entries.append(StepEntry(k, requests[k][at[k]:at[k] + size], list(range(size))))
+                at[k] += size
+        logits = runner.step(entries).float().cpu()
+        row = 0
+        for e in entries:
+            got[e.request_id].append(logits[row:row + len(e.tokens)])
+            row += len(e.tokens)
+        step += 1
+    for i in range(tail):
+        entries = [StepEntry(k, [requests[k][cut[k] + i]], [0]) for k in requests]
+        logits = runner.step(entries).float().cpu()
+        for row, e in enumerate(entries):
+            got[e.request_id].append(logits[row:row + 1])
+    assert runner.graph_replays >= tail - 2
+    for k in requests:
+        rows = torch.cat(got[k])
+        scale = float(want[k].abs().max())
+        bound = 1e-4 * scale + 1e-5 if dtype == "float32" else ru.BF16_FRACTION * scale
+        assert float((rows - want[k]).abs().max()) <= bound, k
+
+
+class CentredNorm(Norm):
+    """``y = (s - mean(s)) / sqrt(var(s) + eps) * w + b`` with ``s`` the stream plus what is pending:
+    a norm that subtracts the mean and has a bias, in plain tensor operations."""
+
+    def __init__(self, ctx, prefix, *, size: int, eps: float) -> None:
+        super().__init__(ctx, prefix)
+        self.size, self.eps = size, float(eps)
+        self.tensors = {}
+
+    def param_specs(self):
+        return {self.name("weight"): ParamSpec((self.size,), kind="vector", init="norm"),
+                self.name("bias"): ParamSpec((self.size,), kind="vector", init="norm")}
+
+    def set_param(self, name, tensor):
+        self.tensors[name[len(self.prefix) + 1:]] = tensor
+
+    def forward(self, residual: Residual, rows=None):
+        if rows is None:
+            s = residual.flush()
+        else:                       # the chosen rows; the stream and what is pending stay as they are
+            s = residual.h[rows.long()]
+            if residual.pending is not None:
+                pending = residual.pending if residual.pending.dim() == 2 else residual.pending.sum(0)
+                s = s + pending[rows.long()]
+        centred = s - s.mean(-1, keepdim=True)
+        y = centred * torch.rsqrt(centred.square().mean(-1, keepdim=True) + self.eps)
+        return (y * self.tensors["weight"] + self.tensors["bias"]).to(self.ctx.dtype)
+
+
+class CappedHead(Head):
+    """``logits = cap * tanh((z W^T) / cap)``: a head with a matrix of its own that bounds its logits."""
+
+    def __init__(self, ctx, prefix, *, vocab_size: int, hidden_size: int, cap: float) -> None:
+        super().__init__(ctx, prefix)
+        self.vocab_size, self.hidden_size, self.cap = vocab_size, hidden_size, float(cap)
+        self.weight = None
+
+    def param_specs(self):
+        return {self.name("weight"): ParamSpec((self.vocab_size, self.hidden_size))}
+
+    def set_param(self, name, tensor):
+        self.weight = tensor
+
+    def forward(self, z):
+        return self.cap * torch.tanh(z.float() @ self.weight.float().T / self.cap)
+
+
+@dataclass(frozen=True)
+class CentredConfig(ModelConfig):
+    vocab_size: int
+    hidden_size: int
+    intermediate_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    norm_eps: float
+    rope_theta: float
+    logit_cap: float
+    architecture: ClassVar[str] = "ToyCentredLM"
+
+    @classmethod
+    def from_dict(cls, raw):
+        read = KeyReader(raw)
+        return cls(*(read.integer(k) for k in ("vocab_size", "hidden_size", "intermediate_size", "num_attention_heads",
+                                              "num_key_value_heads", "head_dim")),
+                   read.number("norm_eps"), read.number("rope_theta"), read.number("logit_cap"))
+
+
+def centred_plan(config: CentredConfig) -> ModelPlan:
+    def norm(prefix):
+        return PartSpec("toy_centred", {"size": config.hidden_size, "eps": config.norm_eps}, prefix)
+
+    def layer(index):
+        prefix = f"model.layers.{index}"
+        attention = PartSpec("gqa_attention", {
+            "hidden_size": config.hidden_size, "num_heads": config.num_attention_heads,
+            "num_kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+            "position": PartSpec("rotary", {"head_dim": config.head_dim, "theta": config.rope_theta})}, f"{prefix}.self_attn")
+        mlp = PartSpec("swiglu", {"hidden_size": config.hidden_size, "intermediate_size": config.intermediate_size}, f"{prefix}.mlp")
+        return LayerSpec("pre_norm", attention, mlp,
+                         {"input": norm(f"{prefix}.input_layernorm"), "post_mixer": norm(f"{prefix}.post_attention_layernorm")})
+
+    table = {"vocab_size": config.vocab_size, "hidden_size": config.hidden_size}
+    return ModelPlan(config.hidden_size, config.vocab_size, PartSpec("token_embedding", dict(table), "model.embed_tokens"),
+                     (layer(0), layer(1)), (LayerCall(0), LayerCall(1)), norm("model.norm"),
+                     PartSpec("toy_capped", dict(table, cap=config.logit_cap), "lm_head"))
+
+
+def centred_plain_forward(w, config: CentredConfig, tokens):
+    t = len(tokens)
+    heads, kv_heads, d = config.num_attention_heads, config.num_key_value_heads, config.head_dim
+    cos, sin = plain.rotary_tables(torch.arange(t), d, config.rope_theta)
+
+    def norm(x, prefix):
+        return torch.nn.functional.layer_norm(x, (config.hidden_size,), w[f"{prefix}.weight"], w[f"{prefix}.bias"], config.norm_eps)
+
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    for index in range(2):
+        p = f"model.layers.{index}"
+        x = norm(h, f"{p}.input_layernorm")
+        q = (x @ w[f"{p}.self_attn.q_proj.weight"].T).view(t, heads, d).transpose(0, 1)
+        k = (x @ w[f"{p}.self_attn.k_proj.weight"].T).view(t, kv_heads, d).transpose(0, 1)
+        v = (x @ w[f"{p}.self_attn.v_proj.weight"].T).view(t, kv_heads, d).transpose(0, 1)
+        out = plain.causal_attention(plain.apply_rotary(q, cos, sin), plain.apply_rotary(k, cos, sin), v, d ** -0.5)
+        h = h + out.transpose(0, 1).reshape(t, heads * d) @ w[f"{p}.self_attn.o_proj.weight"].T
+        h = h + plain.swiglu_mlp(norm(h, f"{p}.post_attention_layernorm"), w, f"{p}.mlp")
+    return config.logit_cap * torch.tanh(norm(h, "model.norm") @ w["lm_head.weight"].T / config.logit_cap)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_norm_and_a_head_registered_from_a_test(dtype, tmp_path):
+    """The two roles that the other toys leave to the framework's own parts: a norm that subtracts
+    the mean and adds a bias (against the library's layer norm), and a head that bounds its logits.
+    The norm meets every way the stream reaches it: an update pending whole or in partial sums,
+    nothing pending, and the wanted rows only before the head."""
+    register_part("norm", "toy_centred", CentredNorm, replace=True)
+    register_part("head", "toy_capped", CappedHead, replace=True)
+    register_architecture("ToyCentredLM", CentredConfig, centred_plan, replace=True)
+    raw = {"architectures": ["ToyCentredLM"], "vocab_size": 77, "hidden_size": 64, "intermediate_size": 48,
+           "num_attention_heads": 2, "num_key_value_heads": 2, "head_dim": 32, "norm_eps": 1e-3, "rope_theta": 1e3,
+           "logit_cap": 0.4}
+    config = load_model_config(raw)
+    folder = write_random_model(config, 23, tmp_path)
+    w = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
+    assert float(w["model.norm.bias"].abs().min()) > 0.5           # a bias that is left out would show
+    _, model = load_model(folder, dtype=dtype, device=DEV)
+    requests = ru.make_requests(raw, 10, (33, 18))
+    want = {k: centred_plain_forward(w, config, v) for k, v in requests.items()}
+    assert float(want["r0"].abs().max()) > 0.5 * config.logit_cap     # the cap bends the logits
+    runner = ModelRunner(model, block_size=4, block_capacity=20, num_state_slots=2, eager_sightings=1)
+    got = {k: [] for k in requests}
+    for k in requests:
+        runner.begin(k)
+    tail = 7
+    cut = {k: len(v) - tail for k, v in requests.items()}
+    at = {k: 0 for k in requests}
+    step = 0
+    while any(at[k] < cut[k] for k in requests):
+        entries = []
+        for k in requests:
+            size = min((4, 7, 2)[(step + len(requests[k])) % 3], cut[k] - at[k])
             if size > 0:
                 entries.append(StepEntry(k, requests[k][at[k]:at[k] + size], list(range(size))))
                 at[k] += size
