@@ -180,6 +180,7 @@ def _qk_case(g, dtype, tokens, q_heads, kv_heads, head_dim, block_size, num_bloc
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,block_size,rotary_dim", [
     (4, 2, 16, 4, 16), (6, 2, 32, 8, 32), (5, 1, 128, 16, 128), (3, 3, 64, 1, 32), (8, 2, 256, 32, 256),
     (2, 1, 48, 5, 0), (4, 2, 64, 8, 64), (32, 8, 128, 16, 128),
+    (64, 16, 128, 16, 128), (20, 4, 256, 32, 256),       # more heads than a block of the vector kernel takes: two blocks a token
 ])
 @pytest.mark.parametrize("tokens", [11, 300])       # few tokens: four heads a block; many: a block per token
 def test_qk_norm_rope_write(ops, dtype, q_heads, kv_heads, head_dim, block_size, rotary_dim, tokens):
