@@ -144,3 +144,41 @@ def test_the_two_references_of_paged_attention_agree(window):
                                        num_seqs=len(seqs), max_q_len=9, **kw)
     fast = kernel_refs.paged_attention_by_matrices(q, kp, vp, cu, ctx, table, **kw)
     torch.testing.assert_close(fast, slow, atol=1e-5, rtol=1e-5)
+
+
+def test_a_library_that_is_missing_and_cannot_be_built_fails_loudly(monkeypatch, tmp_path):
+    """No fallback: without a compiled library and without a compiler, loading raises, and so does
+    the preparation of a model's libraries; a file at the library's place that was built from other
+    sources is not opened in its stead."""
+    from forge_engine_amd.kernels import build, library
+
+    monkeypatch.setattr(build, "library_dirs", lambda: [tmp_path])
+    monkeypatch.setattr(library, "_LOADED", {})
+
+    def no_compiler() -> str:
+        raise build.KernelBuildError("hipcc not found: the HIP kernels cannot be compiled")
+
+    monkeypatch.setattr(build, "find_hipcc", no_compiler)
+    assert not library.is_built("rowwise")
+    with pytest.raises(library.KernelUnavailable, match="not built and could not be compiled.*hipcc not found"):
+        library.load("rowwise")
+    with pytest.raises(library.KernelUnavailable, match="hipcc not found"):
+        library.ensure_built(["rowwise", "sample"], announce=False)
+    stale = build.library_path("rowwise", tmp_path)
+    stale.write_bytes(b"\x7fELF built from sources with another hash")
+    assert not library.is_built("rowwise")
+    with pytest.raises(library.KernelUnavailable):
+        library.load("rowwise")
+    assert "rowwise" not in library._LOADED
+    with pytest.raises(build.KernelBuildError, match="no kernel source"):
+        build.compile_one("no_such_kernel", tmp_path)
+
+
+def test_operands_on_the_cpu_are_refused_before_anything_is_loaded():
+    import torch
+
+    h = torch.zeros(2, 8)
+    with pytest.raises(ops.KernelError, match="no CPU path"):
+        ops.add_rmsnorm(h, None, torch.ones(8), 1e-6, torch.empty(2, 8))
+    with pytest.raises(ops.KernelError, match="no CPU path"):
+        ops.linear(torch.zeros(2, 8), torch.zeros(4, 8))
