@@ -4,6 +4,7 @@ other, with the metadata the kernels index by."""
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from functools import cached_property
 
 import torch
 from torch import Tensor
@@ -47,6 +48,73 @@ class StepBatch:
     state_slots_host: list
 
 
+@dataclass(frozen=True)
+class BatchLayout:
+    """Where each part of a step's metadata lies in the step's one int32 buffer: what there is per
+    token, per request, the wanted rows, a block table per cache group, and the per-token inputs
+    that the model's parts asked for, name after name.  ``build_batch`` packs a step this way, and
+    the buffers of captured steps are refilled through the same description."""
+
+    num_tokens: int
+    num_seqs: int
+    num_wanted: int
+    widths: tuple            # block-table width of every cache group
+    token_inputs: tuple = ()   # (name, integers a token), in the order of the names
+
+    @classmethod
+    def of(cls, num_tokens: int, num_seqs: int, num_wanted: int, widths, token_inputs=None) -> "BatchLayout":
+        return cls(num_tokens, num_seqs, num_wanted, tuple(widths), tuple(sorted((token_inputs or {}).items())))
+
+    def parts(self):
+        """(key, int32 entries) in the order of the buffer; a block table's key is ("table", group),
+        a per-token input's ("input", name)."""
+        t, b = self.num_tokens, self.num_seqs
+        yield from (("token_ids", t), ("positions", t), ("token_seq", t), ("cu_q", b + 1), ("ctx_len", b),
+                    ("ctx_before", b), ("state_slots", b), ("want_rows", self.num_wanted))
+        for group, width in enumerate(self.widths):
+            yield ("table", group), b * width
+        for name, width in self.token_inputs:
+            yield ("input", name), t * width
+
+    @cached_property
+    def spans(self) -> dict:
+        found, offset = {}, 0
+        for key, size in self.parts():
+            found[key] = slice(offset, offset + size)
+            offset += size
+        return found
+
+    @property
+    def size(self) -> int:
+        return sum(size for _, size in self.parts())
+
+    def span(self, key) -> slice:
+        return self.spans[key]
+
+    def views(self, flat) -> dict:
+        """The buffer's parts by key (of a tensor or an array): block tables as [requests, width],
+        per-token inputs as [tokens, integers a token]."""
+        found = {key: flat[span] for key, span in self.spans.items()}
+        for group, width in enumerate(self.widths):
+            found[("table", group)] = found[("table", group)].reshape(self.num_seqs, width)
+        for name, width in self.token_inputs:
+            found[("input", name)] = found[("input", name)].reshape(self.num_tokens, width)
+        return found
+
+    def batch(self, flat: Tensor, *, max_q_len: int, max_ctx: int, num_decode: int | None, request_ids=(), q_lens=(),
+              ctx_before_host=(), state_slots_host=()) -> "StepBatch":
+        """The step's batch over the device buffer ``flat``."""
+        v = self.views(flat)
+        return StepBatch(
+            num_tokens=self.num_tokens, num_seqs=self.num_seqs, num_wanted=self.num_wanted, max_q_len=max_q_len,
+            max_ctx=max_ctx, num_decode=num_decode, token_ids=v["token_ids"], positions=v["positions"],
+            token_seq=v["token_seq"], cu_q=v["cu_q"], ctx_len=v["ctx_len"], ctx_before=v["ctx_before"],
+            state_slots=v["state_slots"], want_rows=v["want_rows"],
+            block_tables=[v[("table", group)] for group in range(len(self.widths))],
+            inputs={name: v[("input", name)] for name, _ in self.token_inputs}, request_ids=list(request_ids),
+            q_lens=list(q_lens), ctx_before_host=list(ctx_before_host), state_slots_host=list(state_slots_host))
+
+
 def token_input_values(entry: StepEntry, name: str, width: int, start: int) -> list[int]:
     """One named per-token input for an entry's tokens, row after row: what the entry brings, else
     the token's position (``start`` is the first token's) on every axis."""
@@ -73,7 +141,6 @@ def build_batch(entries, lengths_before, state_slots, tables_per_group, device, 
     a bound, not for one step's lengths); ``token_inputs`` (name -> integers a token) are the
     per-token inputs that the model's parts asked for, laid out behind the block tables in the
     order of their names."""
-    token_inputs = dict(sorted((token_inputs or {}).items()))
     num_seqs = len(entries)
     q_lens = [len(e.tokens) for e in entries]
     total = sum(q_lens)
@@ -89,18 +156,20 @@ def build_batch(entries, lengths_before, state_slots, tables_per_group, device, 
     ctx_len = [lengths_before[i] + q_lens[i] for i in range(num_seqs)]
     if widths is None:
         widths = [max(1, max((len(t) for t in tables), default=1)) for tables in tables_per_group]
-    flat_tables = []
-    for tables, width in zip(tables_per_group, widths):
+    layout = BatchLayout.of(total, num_seqs, len(want_rows), widths, token_inputs)
+    values = {"token_ids": token_ids, "positions": positions, "token_seq": token_seq, "cu_q": cu_q, "ctx_len": ctx_len,
+              "ctx_before": list(lengths_before), "state_slots": list(state_slots), "want_rows": want_rows}
+    for group, (tables, width) in enumerate(zip(tables_per_group, widths)):
+        flat_table = values[("table", group)] = []
         for table in tables:
             if len(table) > width:
                 raise ValueError(f"a block table of {len(table)} pages does not fit the width {width}")
-            flat_tables.extend(table)
-            flat_tables.extend([-1] * (width - len(table)))
-    sections = [token_ids, positions, token_seq, cu_q, ctx_len, list(lengths_before), list(state_slots),
-                want_rows, flat_tables]
-    for name, width in token_inputs.items():
-        sections.append([v for i, entry in enumerate(entries) for v in token_input_values(entry, name, width, lengths_before[i])])
-    host = torch.tensor([v for section in sections for v in section], dtype=torch.int32)
+            flat_table.extend(table)
+            flat_table.extend([-1] * (width - len(table)))
+    for name, width in layout.token_inputs:
+        values[("input", name)] = [v for i, entry in enumerate(entries)
+                                   for v in token_input_values(entry, name, width, lengths_before[i])]
+    host = torch.tensor([v for key, _ in layout.parts() for v in values[key]], dtype=torch.int32)
     if static is not None:
         host_static, flat = static
         if host.numel() > flat.numel():
@@ -111,67 +180,15 @@ def build_batch(entries, lengths_before, state_slots, tables_per_group, device, 
         if device.type == "cuda":
             host = host.pin_memory()
         flat = host.to(device, non_blocking=True)
-    views = []
-    offset = 0
-    for section in sections:
-        views.append(flat[offset:offset + len(section)])
-        offset += len(section)
-    block_tables = []
-    table_flat = views[8]
-    offset = 0
-    for width in widths:
-        block_tables.append(table_flat[offset:offset + num_seqs * width].view(num_seqs, width))
-        offset += num_seqs * width
-    inputs = {name: views[9 + i].view(total, width) for i, (name, width) in enumerate(token_inputs.items())}
-    return StepBatch(
-        num_tokens=total, num_seqs=num_seqs, num_wanted=len(want_rows), max_q_len=max(q_lens),
-        max_ctx=max(ctx_len) if max_ctx is None else max_ctx,
-        num_decode=sum(1 for n in q_lens if n == 1), token_ids=views[0], positions=views[1],
-        token_seq=views[2], cu_q=views[3], ctx_len=views[4], ctx_before=views[5], state_slots=views[6],
-        want_rows=views[7], block_tables=block_tables, inputs=inputs, request_ids=[e.request_id for e in entries],
-        q_lens=q_lens, ctx_before_host=list(lengths_before), state_slots_host=list(state_slots))
+    return layout.batch(flat, max_q_len=max(q_lens), max_ctx=max(ctx_len) if max_ctx is None else max_ctx,
+                        num_decode=sum(1 for n in q_lens if n == 1), request_ids=[e.request_id for e in entries],
+                        q_lens=q_lens, ctx_before_host=lengths_before, state_slots_host=state_slots)
 
 
-def static_batch_size(num_seqs: int, widths, num_tokens: int | None = None, num_wanted: int | None = None,
-                      token_inputs=None) -> int:
-    """int32 entries of a batch of ``num_seqs`` requests (by default with one token and one
-    wanted row each)."""
-    tokens = num_seqs if num_tokens is None else num_tokens
-    wanted = num_seqs if num_wanted is None else num_wanted
-    return 3 * tokens + 4 * num_seqs + 1 + wanted + num_seqs * sum(widths) + tokens * sum((token_inputs or {}).values())
-
-
-def token_input_places(num_seqs: int, widths, num_tokens: int, num_wanted: int, token_inputs) -> dict:
-    """name -> (first int32 entry, integers a token) of the per-token inputs in a batch's buffer."""
-    offset = static_batch_size(num_seqs, widths, num_tokens, num_wanted)
-    places = {}
-    for name, width in sorted((token_inputs or {}).items()):
-        places[name] = (offset, width)
-        offset += num_tokens * width
-    return places
-
-
-def static_batch(flat: Tensor, *, num_tokens: int, num_seqs: int, num_wanted: int, widths, max_q_len: int,
-                 max_ctx: int, num_decode: int | None = None, token_inputs=None) -> StepBatch:
-    """The batch of a captured step: views into a device buffer at fixed addresses, laid out as
-    ``build_batch`` lays a batch out, for ``num_seqs`` sequences of which some may be empty.
-    What the kernels cannot read from the buffer is a bound (``max_q_len``, ``max_ctx``) or
-    unknown (how many sequences bring one token, unless the caller knows that none ever does:
-    ``num_decode=0``); the host-side lists are not filled in, so a model with a part that reads
-    them is not captured."""
-    sizes = [num_tokens, num_tokens, num_tokens, num_seqs + 1, num_seqs, num_seqs, num_seqs, num_wanted]
-    views, offset = [], 0
-    for size in sizes:
-        views.append(flat[offset:offset + size])
-        offset += size
-    block_tables = []
-    for width in widths:
-        block_tables.append(flat[offset:offset + num_seqs * width].view(num_seqs, width))
-        offset += num_seqs * width
-    inputs = {name: flat[at:at + num_tokens * width].view(num_tokens, width)
-              for name, (at, width) in token_input_places(num_seqs, widths, num_tokens, num_wanted, token_inputs).items()}
-    return StepBatch(
-        num_tokens=num_tokens, num_seqs=num_seqs, num_wanted=num_wanted, max_q_len=max_q_len, max_ctx=max_ctx,
-        num_decode=num_decode, token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
-        ctx_len=views[4], ctx_before=views[5], state_slots=views[6], want_rows=views[7],
-        block_tables=block_tables, inputs=inputs, request_ids=[], q_lens=[], ctx_before_host=[], state_slots_host=[])
+def static_batch(flat: Tensor, layout: BatchLayout, *, max_q_len: int, max_ctx: int, num_decode: int | None = None) -> StepBatch:
+    """The batch of a captured step: views into a device buffer at fixed addresses, for
+    ``layout.num_seqs`` sequences of which some may be empty.  What the kernels cannot read from
+    the buffer is a bound (``max_q_len``, ``max_ctx``) or unknown (how many sequences bring one
+    token, unless the caller knows that none ever does: ``num_decode=0``); the host-side lists are
+    not filled in, so a model with a part that reads them is not captured."""
+    return layout.batch(flat, max_q_len=max_q_len, max_ctx=max_ctx, num_decode=num_decode)

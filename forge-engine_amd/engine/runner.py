@@ -14,7 +14,7 @@ from torch import Tensor
 from ..cache import CacheCapacityError, CacheManager, CacheView, plan_groups
 from ..kernels import library, ops
 from ..models.decoder import DecoderModel
-from .batch import StepBatch, StepEntry, build_batch, static_batch, static_batch_size, token_input_places, token_input_values
+from .batch import BatchLayout, StepBatch, StepEntry, build_batch, static_batch, token_input_values
 
 GRAPH_MAX_REQUESTS = 256     # steps of up to this many requests replay a captured graph
 GRAPH_TABLE_STEP = 64        # block-table widths of graphs are multiples of this many pages
@@ -40,22 +40,17 @@ class _DecodeGraph:
 
     def __init__(self, num_seqs: int, widths, device, token_inputs=None) -> None:
         n = num_seqs
-        size = static_batch_size(n, widths, token_inputs=token_inputs)
-        self.inputs_at = token_input_places(n, widths, n, n, token_inputs)
-        self.host = torch.empty(size, dtype=torch.int32).pin_memory()
-        self.dev = torch.zeros(size, dtype=torch.int32, device=device)
+        self.layout = BatchLayout.of(n, n, n, widths, token_inputs)
+        self.host = torch.empty(self.layout.size, dtype=torch.int32).pin_memory()
+        self.dev = torch.zeros(self.layout.size, dtype=torch.int32, device=device)
         self.np = self.host.numpy()
+        self.part = self.layout.views(self.np)          # the pinned buffer's parts by name
         self.widths = list(widths)
         self.n = n
         self.np[:] = -1
-        self.np[2 * n:3 * n] = np.arange(n)              # token_seq
-        self.np[3 * n:4 * n + 1] = np.arange(n + 1)      # cu_q
-        self.np[7 * n + 1:8 * n + 1] = np.arange(n)      # want_rows
-        self.table_at = []
-        offset = 8 * n + 1
-        for width in self.widths:
-            self.table_at.append(offset)
-            offset += n * width
+        self.part["token_seq"][:] = np.arange(n)
+        self.part["cu_q"][:] = np.arange(n + 1)
+        self.part["want_rows"][:] = np.arange(n)
         self.row_keys = [[None] * n for _ in self.widths]
         self.graph = None
         self.logits = None
@@ -65,30 +60,44 @@ class _DecodeGraph:
 
     def fill_inputs(self, entries, positions) -> None:
         """The per-token inputs of a step of single tokens at ``positions``."""
-        n, buf = self.n, self.np
-        for name, (at, width) in self.inputs_at.items():
+        for name, width in self.layout.token_inputs:
+            rows = self.part[("input", name)]
             for i, entry in enumerate(entries):
-                buf[at + i * width:at + (i + 1) * width] = token_input_values(entry, name, width, int(positions[i]))
+                rows[i] = token_input_values(entry, name, width, int(positions[i]))
 
     def fill(self, tokens, before, records, entries) -> None:
-        n, buf = self.n, self.np
+        part = self.part
         before = np.asarray(before, dtype=np.int32)
         self.fill_inputs(entries, before)
-        buf[0:n] = tokens
-        buf[n:2 * n] = before                            # positions
-        buf[4 * n + 1:5 * n + 1] = before + 1            # ctx_len
-        buf[5 * n + 1:6 * n + 1] = before                # ctx_before
-        buf[6 * n + 1:7 * n + 1] = [r.state_slot for r in records]
-        for g, width in enumerate(self.widths):
-            keys, base = self.row_keys[g], self.table_at[g]
+        part["token_ids"][:] = tokens
+        part["positions"][:] = before
+        part["ctx_len"][:] = before + 1
+        part["ctx_before"][:] = before
+        part["state_slots"][:] = [r.state_slot for r in records]
+        for g in range(len(self.widths)):
+            keys, rows = self.row_keys[g], part[("table", g)]
             for i, record in enumerate(records):
                 table = record.tables[g]
                 key = (record.lease, len(table), record.first_block[g])   # pages are only ever appended or given back from the front
                 if keys[i] != key:
-                    row = buf[base + i * width:base + (i + 1) * width]
-                    row[:len(table)] = table
-                    row[len(table):] = -1
+                    rows[i, :len(table)] = table
+                    rows[i, len(table):] = -1
                     keys[i] = key
+
+    def move_on(self, tokens, entries) -> None:
+        """The same requests again, each one token further: only the tokens change and every
+        position moves on by one."""
+        part = self.part
+        part["token_ids"][:] = tokens
+        part["positions"] += 1
+        part["ctx_len"] += 1
+        part["ctx_before"] += 1
+        self.fill_inputs(entries, part["positions"])
+
+    def feed(self, device_tokens: Tensor) -> None:
+        """Tokens that are still on the device go into the step's buffer there."""
+        tokens = self.dev[self.layout.span("token_ids")]
+        tokens.copy_(device_tokens[:tokens.numel()])
 
 
 class _SteadyDecode:
@@ -109,61 +118,51 @@ class _PortionGraph:
     def __init__(self, num_tokens: int, num_seqs: int, num_wanted: int, widths, device, pad_state_slot: int = 0,
                  token_inputs=None) -> None:
         self.pad_state_slot = pad_state_slot
-        size = static_batch_size(num_seqs, widths, num_tokens, num_wanted, token_inputs)
-        self.inputs_at = token_input_places(num_seqs, widths, num_tokens, num_wanted, token_inputs)
-        self.host = torch.empty(size, dtype=torch.int32).pin_memory()
-        self.dev = torch.zeros(size, dtype=torch.int32, device=device)
+        self.layout = BatchLayout.of(num_tokens, num_seqs, num_wanted, widths, token_inputs)
+        self.host = torch.empty(self.layout.size, dtype=torch.int32).pin_memory()
+        self.dev = torch.zeros(self.layout.size, dtype=torch.int32, device=device)
         self.np = self.host.numpy()
+        self.part = self.layout.views(self.np)
         self.np[:] = 0
-        self.t, self.b, self.w, self.widths = num_tokens, num_seqs, num_wanted, list(widths)
-        self.table_at = []
-        offset = 3 * num_tokens + 4 * num_seqs + 1 + num_wanted
-        for width in self.widths:
-            self.table_at.append(offset)
-            self.np[offset:offset + num_seqs * width] = -1
-            offset += num_seqs * width
+        for g in range(len(self.layout.widths)):
+            self.part[("table", g)][:] = -1
         self.graph = None
         self.logits = None
         self.copied = torch.cuda.Event()
 
     def fill(self, entries, before, records) -> None:
-        t, b, w, buf = self.t, self.b, self.w, self.np
+        part = self.part
         n = len(entries)
-        at = 0
-        cu = buf[3 * t:3 * t + b + 1]
-        want = buf[3 * t + 4 * b + 1:3 * t + 4 * b + 1 + w]
-        rows = 0
+        at = rows = 0
+        cu, want = part["cu_q"], part["want_rows"]
         for i, entry in enumerate(entries):
             count = len(entry.tokens)
-            buf[at:at + count] = entry.tokens
-            buf[t + at:t + at + count] = np.arange(before[i], before[i] + count)
-            buf[2 * t + at:2 * t + at + count] = i
+            part["token_ids"][at:at + count] = entry.tokens
+            part["positions"][at:at + count] = np.arange(before[i], before[i] + count)
+            part["token_seq"][at:at + count] = i
             cu[i] = at
             for place in entry.want:
                 want[rows] = at + place
                 rows += 1
-            for name, (first, width) in self.inputs_at.items():
-                buf[first + at * width:first + (at + count) * width] = token_input_values(entry, name, width, before[i])
+            for name, width in self.layout.token_inputs:
+                part[("input", name)][at:at + count] = np.asarray(
+                    token_input_values(entry, name, width, before[i]), dtype=np.int32).reshape(count, width)
             at += count
         cu[n:] = at                                                   # the other sequences are empty
         want[rows:] = 0
-        ctx = buf[3 * t + b + 1:3 * t + 2 * b + 1]
-        ctx[:n] = [before[i] + len(e.tokens) for i, e in enumerate(entries)]
-        ctx[n:] = 0
-        start = buf[3 * t + 2 * b + 1:3 * t + 3 * b + 1]
-        start[:n] = before
-        start[n:] = 0
-        slots = buf[3 * t + 3 * b + 1:3 * t + 4 * b + 1]
-        slots[:n] = [r.state_slot for r in records]
-        slots[n:] = self.pad_state_slot
-        for g, width in enumerate(self.widths):
-            base = self.table_at[g]
+        part["ctx_len"][:n] = [before[i] + len(e.tokens) for i, e in enumerate(entries)]
+        part["ctx_len"][n:] = 0
+        part["ctx_before"][:n] = before
+        part["ctx_before"][n:] = 0
+        part["state_slots"][:n] = [r.state_slot for r in records]
+        part["state_slots"][n:] = self.pad_state_slot
+        for g in range(len(self.layout.widths)):
+            table_rows = part[("table", g)]
             for i, record in enumerate(records):
                 table = record.tables[g]
-                row = buf[base + i * width:base + (i + 1) * width]
-                row[:len(table)] = table
-                row[len(table):] = -1
-            buf[base + n * width:base + b * width] = -1
+                table_rows[i, :len(table)] = table
+                table_rows[i, len(table):] = -1
+            table_rows[n:] = -1
 
 
 class ModelRunner:
@@ -315,17 +314,13 @@ class ModelRunner:
                 and cache.holds(steady.records)):
             # the same requests as the last step, none ended since, every one with room in its last
             # page: only the tokens change and every position moves on by one
-            slot, n = steady.slot, len(entries)
+            slot = steady.slot
             slot.copied.synchronize()
-            buf = slot.np
-            buf[0:n] = tokens
-            buf[n:2 * n] += 1                                # positions
-            buf[4 * n + 1:6 * n + 1] += 1                    # ctx_len, ctx_before
-            slot.fill_inputs(entries, buf[n:2 * n])
+            slot.move_on(tokens, entries)
             slot.dev.copy_(slot.host, non_blocking=True)
             slot.copied.record(torch.cuda.current_stream(self.device))
             if device_tokens is not None:
-                slot.dev[0:n].copy_(device_tokens[0:n])
+                slot.feed(device_tokens)
             slot.graph.replay()
             for record in steady.records:
                 record.length += 1
@@ -369,7 +364,7 @@ class ModelRunner:
                 slot.logits = self.model.forward(batch, views)
             slot.graph, slot.views, slot.batch = graph, views, batch
         if device_tokens is not None:
-            slot.dev[0:len(entries)].copy_(device_tokens[0:len(entries)])
+            slot.feed(device_tokens)
         slot.graph.replay()
         self.graph_replays += 1
         cache.commit_single_tokens(records)
@@ -440,9 +435,9 @@ class ModelRunner:
         slot.dev.copy_(slot.host, non_blocking=True)
         slot.copied.record(torch.cuda.current_stream(self.device))
         if slot.graph is None:
-            batch = static_batch(slot.dev, num_tokens=shape[0], num_seqs=shape[1], num_wanted=shape[2],
-                                 widths=widths, max_q_len=shape[0], max_ctx=widths[0] * self.block_size if widths else 0,
-                                 num_decode=None if shape[3] else 0, token_inputs=self.token_inputs)
+            batch = static_batch(slot.dev, slot.layout, max_q_len=shape[0],
+                                 max_ctx=widths[0] * self.block_size if widths else 0,
+                                 num_decode=None if shape[3] else 0)
             views = self.cache_views(batch)
             self._warm_up(batch)
             graph = torch.cuda.CUDAGraph()

@@ -271,7 +271,7 @@ def test_per_token_inputs_lie_behind_the_block_tables():
     """What a model's parts ask for per token (`token_inputs`) is carried in the step's one buffer,
     name after name: rows that an entry brings, or the token's position on every axis; a captured
     step's buffer has the same places."""
-    from forge_engine_amd.engine.batch import StepEntry, build_batch, static_batch, static_batch_size, token_input_places
+    from forge_engine_amd.engine.batch import BatchLayout, StepEntry, build_batch, static_batch
     entries = [StepEntry("a", [5, 6, 7], [2], {"grid": [[1, 2], [3, 4], [5, 6]]}),
                StepEntry("b", [8], [0]),
                StepEntry("c", [9, 10], [], {"kind": [7, 8]})]
@@ -280,14 +280,20 @@ def test_per_token_inputs_lie_behind_the_block_tables():
     assert batch.inputs["grid"].tolist() == [[1, 2], [3, 4], [5, 6], [4, 4], [0, 0], [1, 1]]
     assert batch.inputs["kind"].tolist() == [[10], [11], [12], [4], [7], [8]]
     assert batch.positions.tolist() == [10, 11, 12, 4, 0, 1]
-    size = static_batch_size(3, [4], 6, 2, asked)
-    assert size == static_batch_size(3, [4], 6, 2) + 6 * 3
-    places = token_input_places(3, [4], 6, 2, asked)
-    assert places == {"grid": (static_batch_size(3, [4], 6, 2), 2), "kind": (static_batch_size(3, [4], 6, 2) + 12, 1)}
-    flat = torch.arange(size, dtype=torch.int32)
-    fixed = static_batch(flat, num_tokens=6, num_seqs=3, num_wanted=2, widths=[4], max_q_len=6, max_ctx=16, token_inputs=asked)
-    assert fixed.inputs["grid"].shape == (6, 2) and int(fixed.inputs["grid"][0, 0]) == places["grid"][0]
-    assert fixed.inputs["kind"].shape == (6, 1) and int(fixed.inputs["kind"][5, 0]) == size - 1
+    assert batch.block_tables[0].tolist() == [[3, 4, 5, 6], [1, 2, -1, -1], [0, -1, -1, -1]]
+    layout, bare = BatchLayout.of(6, 3, 2, [4], asked), BatchLayout.of(6, 3, 2, [4])
+    assert layout.size == bare.size + 6 * 3 and bare.size == 3 * 6 + 4 * 3 + 1 + 2 + 3 * 4
+    assert layout.span(("table", 0)) == bare.span(("table", 0)) == slice(bare.size - 12, bare.size)
+    assert layout.span(("input", "grid")) == slice(bare.size, bare.size + 12)       # name after name, in the names' order
+    assert layout.span(("input", "kind")) == slice(bare.size + 12, bare.size + 18)
+    flat = torch.arange(layout.size, dtype=torch.int32)
+    fixed = static_batch(flat, layout, max_q_len=6, max_ctx=16)
+    assert fixed.inputs["grid"].shape == (6, 2) and int(fixed.inputs["grid"][0, 0]) == bare.size
+    assert fixed.inputs["kind"].shape == (6, 1) and int(fixed.inputs["kind"][5, 0]) == layout.size - 1
+    assert fixed.cu_q.tolist() == list(range(18, 22)) and fixed.block_tables[0].shape == (3, 4)
+    # a step packed by build_batch lies exactly as the layout says
+    packed = BatchLayout.of(6, 3, 1, [4], asked)
+    assert packed.size == batch.inputs["kind"].numel() + batch.inputs["grid"].numel() + 3 * 6 + 4 * 3 + 1 + 1 + 12
     with pytest.raises(ValueError, match="3 rows of 2 integers"):
         build_batch([StepEntry("a", [5, 6, 7], [], {"grid": [[1, 2], [3, 4]]})], [0], [0], [[[0]]], torch.device("cpu"), token_inputs=asked)
     assert build_batch(entries[:2], [0, 0], [0, 1], [[[0], [1]]], torch.device("cpu")).inputs == {}
