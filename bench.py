@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model qwen3-4b|qwen3-8b|qwen3-32b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--model qwen3-4b|qwen3-8b|qwen3-14b|qwen3-32b|qwen3-0.6b|qwen3-1.7b]
 
 The default run has the layer sizes of Qwen3-4B with random weights (bfloat16),
 eight requests decoding from 1,024-token random prompts in a cache pool sized
@@ -72,6 +72,19 @@ MODELS = {
         "label": "Qwen3-14B",
         "config": _qwen3(hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40,
                          rope_theta=1000000.0, tie_word_embeddings=False),
+        "batch": 8, "points": "1,64", "prompt_len": 1024, "context": 8192,
+    },
+    # ... and the two smallest of the family, whose products have fewer blocks than the chip has CUs
+    "qwen3-0.6b": {
+        "label": "Qwen3-0.6B",
+        "config": _qwen3(hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16,
+                         rope_theta=1000000.0, tie_word_embeddings=True),
+        "batch": 8, "points": "1,64", "prompt_len": 1024, "context": 8192,
+    },
+    "qwen3-1.7b": {
+        "label": "Qwen3-1.7B",
+        "config": _qwen3(hidden_size=2048, intermediate_size=6144, num_hidden_layers=28, num_attention_heads=16,
+                         rope_theta=1000000.0, tie_word_embeddings=True),
         "batch": 8, "points": "1,64", "prompt_len": 1024, "context": 8192,
     },
     "qwen3-32b": {

@@ -283,7 +283,8 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None, out_dtype=None
     if (bias is None and _skinny_fits(x, weight) and out_dtype in (torch.float32, torch.bfloat16)
             and not (out_dtype == torch.bfloat16 and _few_rows_to_library(x, weight))):
         return gemm_skinny(x, weight, "f32" if out_dtype == torch.float32 else "bf16")
-    if bias is None and out_dtype == torch.bfloat16 and _wide_fits(x, weight, WIDE_STORE_MAX_ROWS, SKINNY_MAX_ROWS + 1):
+    if (bias is None and out_dtype == torch.bfloat16 and _wide_fits(x, weight, WIDE_STORE_MAX_ROWS, SKINNY_MAX_ROWS + 1)
+            and _wide_store_pays(x.shape[0], weight.shape[0], weight.shape[1])):
         rows = x.shape[0]        # up to 64 rows: blocks of 32 weight rows, so that the launch has twice the blocks
         return gemm_wide(x, weight, "bf16", row_tile=64 if rows <= 128 else 128, block_rows=32 if rows <= 64 else 64)
     if out_dtype == torch.float32:
@@ -354,9 +355,20 @@ WIDE_UPDATE_FEW_WEIGHT_ROWS = 3072   # weight measured (hidden sizes 2560, 4096,
                                      # against 25 / 26 / 73, down projection 30 / 55 / 146 against 46 / 59 / 178); at 384 rows the
                                      # hidden sizes 4096 and 5120 are the library's by a tenth
 WIDE_STORE_MAX_ROWS = 256      # ... and a product that stores bfloat16
+WIDE_STORE_MIN_BLOCKS = 140    # ... with more than 64 rows, if its launch has at least this many blocks (row tiles x 64 weight
+                               # rows): q/k/v of 6144 rows 18-26 against 24-33 us and of 4608 to 5120 rows level with the library,
+                               # but of 4096 rows (K = 2048, 128 blocks) 13-17 against 10-12 us
 WIDE_MAX_WEIGHT_ROWS = 8192    # weights with more rows fill the chip in the library's large tiles
 WIDE_GATE_MAX_K = 4096         # the gate/up product for 17 to 64 rows: beyond this K the matrix library is faster
 WIDE_CUS = 256                 # the product's blocks run one a CU, round after round: the parts of K are chosen to fill the rounds
+
+
+def _wide_store_pays(rows: int, weight_rows: int, k: int = 0) -> bool:
+    """Whether the product for portions that stores bfloat16 beats the library: up to 64 rows unless the
+    weight is large (8192 x 6144, 100 MB: 32-35 against 25-28 us), beyond if it has the blocks to fill the chip."""
+    if rows <= MID_ROWS:
+        return weight_rows * k * 2 <= MID_IN_PARTS_MAX_WEIGHT_BYTES
+    return -(-weight_rows // 64) * -(-rows // (64 if rows <= 128 else 128)) >= WIDE_STORE_MIN_BLOCKS
 
 
 def _wide_fits(x: Tensor, weight: Tensor, most_rows: int, least_rows: int = MID_ROWS + 1) -> bool:
@@ -457,6 +469,7 @@ def linear_update(x: Tensor, weight: Tensor, bias: Tensor | None = None, stream:
 # rows take 10.1 instead of 12.0 us, two parts at 64 rows 11.8 instead of the library's 15.8.
 IN_PARTS_MIN_STEPS = 8
 IN_PARTS_FEW_ROWS = 2
+MID_IN_PARTS_MAX_WEIGHT_BYTES = 80 << 20   # 17 to 64 rows in parts of K: a larger weight than this is the library's
 
 
 def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
@@ -478,8 +491,10 @@ def linear_in_parts(x: Tensor, weight: Tensor) -> Tensor | None:
         return gemm_wide(x, weight, "parts", parts, row_tile=16, block_rows=32)
     if _skinny_fits(x, weight) and rows <= FEW_ROWS:
         return gemm_skinny(x, weight, "f32", tiles=1, waves=4, splits=IN_PARTS_FEW_ROWS)
-    if _mid_fits(x, weight) and weight.shape[0] <= WIDE_MAX_WEIGHT_ROWS:
-        # (a weight of 10240 rows, K = 5120: 30 us at 32 rows against the library's 26; 7168 rows: 18 against 20)
+    if (_mid_fits(x, weight) and weight.shape[0] <= WIDE_MAX_WEIGHT_ROWS
+            and weight.shape[0] * weight.shape[1] * weight.element_size() <= MID_IN_PARTS_MAX_WEIGHT_BYTES):
+        # (a weight of 10240 rows, K = 5120: 30 us at 32 rows against the library's 26; 7168 rows: 18 against 20;
+        # 8192 rows at K = 6144, 100 MB: 35-41 against 25-27)
         return gemm_mid_parts(x, weight, _mid_parts(steps, -(-weight.shape[0] // 64), most=4))
     return None
 

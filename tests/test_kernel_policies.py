@@ -182,3 +182,13 @@ def test_operands_on_the_cpu_are_refused_before_anything_is_loaded():
         ops.add_rmsnorm(h, None, torch.ones(8), 1e-6, torch.empty(2, 8))
     with pytest.raises(ops.KernelError, match="no CPU path"):
         ops.linear(torch.zeros(2, 8), torch.zeros(4, 8))
+
+
+def test_the_product_that_stores_bfloat16_needs_blocks_enough_beyond_64_rows():
+    # q/k/v of Qwen3-4B and 8B (6144 weight rows) fill the chip at 65 to 256 rows; of Qwen3-0.6B and 1.7B (4096) they do not
+    for rows in (65, 128, 129, 256):
+        assert ops._wide_store_pays(rows, 6144) and ops._wide_store_pays(rows, 5120)
+        assert not ops._wide_store_pays(rows, 4096) and not ops._wide_store_pays(rows, 2048)
+    for rows in (17, 32, 64):
+        assert ops._wide_store_pays(rows, 4096, 2048) and ops._wide_store_pays(rows, 7168, 5120)
+        assert not ops._wide_store_pays(rows, 8192, 6144)       # 100 MB of weight: the library's

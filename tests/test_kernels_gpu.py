@@ -867,9 +867,16 @@ def test_gemm_wide_refuses_and_routes(ops, monkeypatch):
     assert update is not None and update.dim() == 3 and taken == ["fe_gemm_wide"]
     torch.testing.assert_close(update.sum(0).cpu(), x.float().cpu() @ w.float().cpu().t(), atol=1e-3, rtol=1e-3)
     y = ops.linear(x, w)
-    assert taken == ["fe_gemm_wide", "fe_gemm_wide"] and y.dtype == torch.bfloat16
+    assert taken == ["fe_gemm_wide"] and y.dtype == torch.bfloat16      # 100 rows x 320 weight rows: too few blocks, the library's
+    wide = rand(g, 4544, 256, dtype=torch.bfloat16, scale=0.05).to(DEV)  # 71 blocks of 64 weight rows x 2 row tiles: its own
+    y = ops.linear(x, wide)
+    assert taken == ["fe_gemm_wide", "fe_gemm_wide"] and y.shape == (100, 4544)
+    torch.testing.assert_close(y.float().cpu(), x.float().cpu() @ wide.float().cpu().t(), atol=2e-2, rtol=2e-2)
+    y = ops.linear(x[:64], w)
+    assert taken == ["fe_gemm_wide"] * 3                                 # up to 64 rows it takes any weight that fits
+    torch.testing.assert_close(y.float().cpu(), x[:64].float().cpu() @ w.float().cpu().t(), atol=2e-2, rtol=2e-2)
     big = rand(g, 600, 256, dtype=torch.bfloat16).to(DEV)
-    assert ops.linear_update(big, w, None, torch.zeros(600, 320, device=DEV)) is None and len(taken) == 2   # the library's
+    assert ops.linear_update(big, w, None, torch.zeros(600, 320, device=DEV)) is None and len(taken) == 3   # the library's
 
 
 def test_gemm_mid_parts_refuses_a_k_that_is_no_multiple_of_its_step(ops):
